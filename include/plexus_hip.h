@@ -1,0 +1,148 @@
+/*
+ * plexus_hip.h -- C ABI of libplexus_hip.so: the GCN-layer hot path of Plexus as gfx950 kernels.
+ *
+ * The reference (hpcgroup/plexus) is pure Python and has no FFI: its hot path is a handful of
+ * stock PyTorch operator calls inside two autograd functions.  Each entry point below replaces one
+ * of those operator calls; the citation names the call it replaces.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in `_host`;
+ *   - matrices are row-major with an explicit leading dimension in ELEMENTS (ld >= row width);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls are
+ *     stream-ordered and asynchronous, they never synchronise the device unless stated;
+ *   - the return value is 0 on success or a negative plx_status; nothing throws;
+ *     plx_last_error() gives a thread-local message for the last failure;
+ *   - apart from plx_spmm_plan_create (which owns a few small device tables until
+ *     plx_spmm_plan_destroy) no call allocates: scratch comes from the caller, sized by the
+ *     matching *_workspace_bytes query;
+ *   - results are deterministic: no atomics, fixed summation order for given inputs and plan.
+ */
+#ifndef PLEXUS_HIP_H
+#define PLEXUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum plx_status {
+    PLX_OK = 0,
+    PLX_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, ld < width, ...) */
+    PLX_ERR_HIP = -2,         /* a HIP runtime call failed; see plx_last_error() */
+    PLX_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+    PLX_ERR_UNSUPPORTED = -4, /* shape outside what the kernels cover */
+    PLX_ERR_NOMEM = -5        /* host or device allocation failed */
+} plx_status;
+
+/* epilogue / prologue flags of the GEMM entry points */
+#define PLX_GEMM_RELU 1u /* C = max(C, 0) (examples/train.py:77-78 fused into the producer) */
+
+int plx_version(void);
+const char *plx_error_string(int status);
+const char *plx_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * CSR preparation.  torch CSR tensors carry int64 crow/col indices (plexus/utils/dataloader.py:367-371
+ * moves them to the device as they are); the kernels read int32.
+ * ---------------------------------------------------------------------------------------- */
+
+/* rowptr32[i] = rowptr64[i] (M+1 entries), col32[j] = col64[j] (nnz entries).  The caller has
+ * checked nnz < 2^31 and K < 2^31. */
+int plx_csr_narrow_i64(int64_t M, int64_t nnz, const int64_t *rowptr64, const int64_t *col64, int32_t *rowptr32,
+                       int32_t *col32, void *stream);
+
+/* Host-only row analysis behind plx_spmm_plan_create, exported so it can be tested without a GPU.
+ * Rows longer than seg_len are split into ceil(len/seg_len) near-equal segments.  Writes at most
+ * `cap_long` row ids to long_rows_host, cap_long+1 entries to seg_first_host and `cap_seg` entries to
+ * seg_begin_host / seg_end_host (any of them may be NULL to only count).  n_long / n_seg receive
+ * the totals. */
+int plx_spmm_segments_host(int64_t M, const int32_t *rowptr_host, int32_t seg_len, int64_t *n_long, int64_t *n_seg,
+                           int32_t *long_rows_host, int32_t *seg_first_host, int64_t cap_long, int32_t *seg_begin_host,
+                           int32_t *seg_end_host, int64_t cap_seg);
+
+/* ------------------------------------------------------------------------------------------
+ * CSR SpMM  Y[M x D] = A[M x K] . H[K x D]
+ *   replaces torch.sparse.mm(edge_index, H)      plexus/gcn_conv.py:98, :188   (AGG = A.H)
+ *        and torch.sparse.mm(adj_t, grad_agg)    plexus/gcn_conv.py:265       (GRAD_H = A^T.GRAD_AGG,
+ *                                                 A^T being its own CSR, dataloader.py:368)
+ * ---------------------------------------------------------------------------------------- */
+typedef struct plx_spmm_plan plx_spmm_plan;
+
+/* Reads rowptr (M+1 int32 on the device; synchronises `stream` once), bins the rows and keeps the
+ * segment tables on the device.  rowptr/col are BORROWED: they must outlive the plan.
+ * seg_len <= 0 selects the default. */
+int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr,
+                         const int32_t *col, int32_t seg_len, void *stream);
+int plx_spmm_plan_destroy(plx_spmm_plan *plan);
+/* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len */
+int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
+/* bytes of scratch an SpMM of width D needs (fp32 partial sums of the split rows; 0 if none) */
+size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D);
+
+/* fp32 values, fp32 H and Y. */
+int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
+                     int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+/* fp32 values, bf16 H and Y (raw uint16 bit patterns), fp32 accumulation, round-to-nearest-even store. */
+int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
+                      uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dense products of the layer (all replace tuned_matmul -> torch.mm, plexus/utils/matmul_tuning.py:94-95)
+ * ---------------------------------------------------------------------------------------- */
+
+/* C[M x N] = A[M x K] . B[K x N]               OUT = AGG . W         plexus/gcn_conv.py:211 */
+int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, unsigned flags, void *stream);
+
+/* C[M x N] = (A ⊙ [mask > 0])[M x K] . B[N x K]^T   GRAD_AGG = GRAD_OUT . W^T   plexus/gcn_conv.py:256-258
+ * mask (same shape and ld as A) may be NULL; when given, A is multiplied elementwise by (mask > 0)
+ * on the way in -- the ReLU backward of examples/train.py:77-78 fused into the consumer. */
+int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *stream);
+
+/* C[K x N] = A[M x K]^T . (B ⊙ [mask > 0])[M x N]   GRAD_W = AGG^T . GRAD_OUT   plexus/gcn_conv.py:237-239
+ * The reduction over M is split over workgroups; partial tiles go to `workspace` and are summed
+ * in a fixed order. */
+size_t plx_gemm_tn_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *workspace,
+                    size_t workspace_bytes, void *stream);
+
+/* Y = max(X, 0) and dX = dY ⊙ [Y > 0] for callers that keep F.relu outside the layer
+ * (examples/train.py:77-78). */
+int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream);
+int plx_relu_bwd_f32(int64_t M, int64_t N, const float *dY, int64_t lddy, const float *Y, int64_t ldy, float *dX,
+                     int64_t lddx, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Row-softmax cross-entropy, forward and gradient in one pass
+ *   replaces the operator chain of TensorParallelCrossEntropy.forward/backward,
+ *   plexus/cross_entropy.py:35-101 and :111-114, at one rank.
+ *
+ *   classes c >= num_classes have probability 0; rows with (row_offset + i) >= num_nodes or
+ *   label < 0 have a zero softmax row; labels outside [0, C) give a zero one-hot row;
+ *   loss = sum_i -log(max(p[i, label_i], 1e-9)) / num_nodes;
+ *   dlogits = (softmax - onehot) / num_nodes * gscale.
+ * Inputs are NOT modified (the reference overwrites padded logits and labels in place).
+ * loss receives one float.  dlogits may alias logits.
+ * ---------------------------------------------------------------------------------------- */
+size_t plx_softmax_xent_workspace_bytes(int64_t M, int64_t C);
+int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
+                         int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
+                         float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Symmetric GCN normalisation of a CSR matrix that already holds its self loops
+ *   val_out[j] = val_in[j] / sqrt(d[row(j)] d[col[j]]),  d[i] = sum of row i of val_in
+ *   (the device-side counterpart of T.GCNNorm, plexus/utils/dataset.py:101).
+ * dinv is scratch of M floats.  Requires a square matrix.  val_out may alias val_in.
+ * ---------------------------------------------------------------------------------------- */
+int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, const float *val_in, float *val_out,
+                         float *dinv, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLEXUS_HIP_H */

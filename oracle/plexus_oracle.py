@@ -1,0 +1,347 @@
+"""CPU oracle for the Plexus GCN hot path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, in stock CPU ``torch`` operators, what the reference computes on
+its GCN hot path when every process group has one rank (all collectives are
+identities, ``pad_dimension(d, 1) == d``).  It is the checker that the GPU kernels
+are compared against; it is never imported by the product package.  Only tests,
+the smoke check and the ``cpu_baseline`` leg of the benchmark may import it.
+
+The arithmetic of the reference lives in a third-party dependency (PyTorch:
+``torch.sparse.mm``, ``torch.mm`` and elementwise ops; unpinned in the
+reference's requirements.txt:1).  The same operators are called here, at the
+reference's own call sites and in the reference's order.  The reference holds
+no tests, golden vectors or fixtures for this path, so every function below is
+pinned by mathematics instead: dense matmul / scipy / brute-force loops for the
+SpMM, numpy fp64 for the GEMMs, ``F.cross_entropy`` and autograd for the loss and
+the backward formulas (see tests/test_oracle.py).
+
+Every function takes ``dtype`` so that an fp64 twin of the same restatement can
+arbitrate when two fp32 summation orders disagree.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------
+# plexus/utils/general.py
+# --------------------------------------------------------------------------
+def pad_dimension(dim_value: int, num_gpus: int, second_num_gpus: int = 1) -> int:
+    """general.py:20-23 -- round ``dim_value`` up to a multiple of the group sizes."""
+    prod = num_gpus * second_num_gpus
+    rem = dim_value % prod
+    return dim_value if rem == 0 else dim_value + prod - rem
+
+
+# --------------------------------------------------------------------------
+# CSR construction as the data loader does it (dataloader.py:343-368)
+# --------------------------------------------------------------------------
+def build_csr_pair(
+    edge_index: torch.Tensor,
+    edge_weight: torch.Tensor,
+    shape: Tuple[int, int],
+    row_range: Optional[Tuple[int, int]] = None,
+    col_range: Optional[Tuple[int, int]] = None,
+):
+    """Mask edges to a block, re-base them, COO -> CSR and CSR of the transpose.
+
+    Follows dataloader.py:343-368 (and benchmarking/spmm.py:67-84 for the block
+    extraction): the transpose is materialised as its own CSR tensor.
+    """
+    if row_range is not None or col_range is not None:
+        r0, r1 = row_range if row_range is not None else (0, shape[0])
+        c0, c1 = col_range if col_range is not None else (0, shape[1])
+        mask = (
+            (edge_index[0] >= r0)
+            & (edge_index[0] < r1)
+            & (edge_index[1] >= c0)
+            & (edge_index[1] < c1)
+        )
+        edge_index = edge_index[:, mask].clone()
+        edge_index[0] -= r0
+        edge_index[1] -= c0
+        edge_weight = edge_weight[mask]
+        shape = (r1 - r0, c1 - c0)
+    coo = torch.sparse_coo_tensor(edge_index, edge_weight, shape)
+    a = coo.to_sparse_csr()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    return a, a_t
+
+
+# --------------------------------------------------------------------------
+# GCN normalisation (consumed by the path; dataset.py:101, PyG T.GCNNorm)
+# --------------------------------------------------------------------------
+def gcn_norm(edge_index: torch.Tensor, num_nodes: int, edge_weight=None, dtype=torch.float32):
+    """w_ij <- w_ij / sqrt(d_i d_j) after adding weight-1 self loops to nodes lacking one.
+
+    PyG's GCNNorm is not in the reference tree (dataset.py:101 only calls it); its
+    published definition is restated: existing self loops are kept, missing ones
+    are filled with 1, the degree is the weighted in-degree by target index.
+    """
+    row, col = edge_index[0], edge_index[1]
+    if edge_weight is None:
+        edge_weight = torch.ones(row.numel(), dtype=dtype)
+    edge_weight = edge_weight.to(dtype)
+    has_loop = torch.zeros(num_nodes, dtype=torch.bool)
+    has_loop[row[row == col]] = True
+    missing = torch.nonzero(~has_loop).reshape(-1)
+    row = torch.cat([row, missing])
+    col = torch.cat([col, missing])
+    w = torch.cat([edge_weight, torch.ones(missing.numel(), dtype=dtype)])
+    deg = torch.zeros(num_nodes, dtype=dtype).index_add_(0, col, w)
+    dinv = deg.pow(-0.5)
+    dinv[torch.isinf(dinv)] = 0.0
+    w = dinv[row] * w * dinv[col]
+    return torch.stack([row, col]), w
+
+
+def gcn_norm_csr_values(crow: torch.Tensor, col: torch.Tensor, val: torch.Tensor):
+    """Symmetric normalisation applied to a CSR matrix that already holds its self loops.
+
+    out_ij = val_ij / sqrt(d_i d_j) with d_i the sum of row i (for a symmetric
+    matrix the row sum equals the column sum PyG uses).
+    """
+    m = crow.numel() - 1
+    counts = crow[1:] - crow[:-1]
+    rows = torch.repeat_interleave(torch.arange(m), counts)
+    deg = torch.zeros(m, dtype=val.dtype).index_add_(0, rows, val)
+    dinv = deg.pow(-0.5)
+    dinv[torch.isinf(dinv)] = 0.0
+    return dinv[rows] * val * dinv[col]
+
+
+# --------------------------------------------------------------------------
+# plexus/gcn_conv.py
+# --------------------------------------------------------------------------
+def extract_csr_submatrix(csr: torch.Tensor, start_row: int, end_row: int) -> torch.Tensor:
+    """gcn_conv.py:25-64 -- rows [start_row, end_row) of a CSR matrix as a new CSR matrix."""
+    crow = csr.crow_indices()
+    col = csr.col_indices()
+    val = csr.values()
+    p0 = int(crow[start_row])
+    p1 = int(crow[end_row])
+    sub_crow = crow[start_row : end_row + 1] - p0
+    return torch.sparse_csr_tensor(
+        sub_crow, col[p0:p1], val[p0:p1], size=(end_row - start_row, csr.size(1)), dtype=csr.dtype
+    )
+
+
+def chunk_bounds(num_rows: int, max_rows_per_chunk: int = 1000000) -> List[Tuple[int, int]]:
+    """gcn_conv.py:77-91 -- the row ranges of the blocked aggregation."""
+    num_chunks = (num_rows + max_rows_per_chunk - 1) // max_rows_per_chunk
+    rows_per_chunk = num_rows // num_chunks
+    out = []
+    for i in range(num_chunks):
+        s = i * rows_per_chunk
+        e = num_rows if i == num_chunks - 1 else (i + 1) * rows_per_chunk
+        out.append((s, e))
+    return out
+
+
+def spmm(a_csr: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
+    """gcn_conv.py:188 (forward) and :265 (backward, on the transposed CSR)."""
+    return torch.sparse.mm(a_csr, h)
+
+
+def chunked_spmm(a_csr: torch.Tensor, h: torch.Tensor, max_rows_per_chunk: int = 1000000) -> torch.Tensor:
+    """gcn_conv.py:67-128 with a one-rank all-reduce group: SpMM per row chunk, concatenated."""
+    parts = [
+        torch.sparse.mm(extract_csr_submatrix(a_csr, s, e), h)
+        for s, e in chunk_bounds(a_csr.size(0), max_rows_per_chunk)
+    ]
+    return torch.cat(parts, dim=0)
+
+
+def gcn_conv_forward(x, a_csr, weight, local_features_shape, local_weight_shape, block_agg=False):
+    """gcn_conv.py:137-219 at one rank.  Returns (OUT, AGG); AGG is what the reference saves."""
+    h = x.reshape(local_features_shape)  # :176-180 (layer-0 input arrives flat)
+    agg = chunked_spmm(a_csr, h) if block_agg else spmm(a_csr, h)  # :184-191
+    w = weight.reshape(local_weight_shape)  # :207
+    out = torch.mm(agg, w)  # :211 -> matmul_tuning.py:95
+    return out, agg
+
+
+def gcn_conv_backward(grad_output, agg, weight, a_t_csr, local_weight_shape, flatten_grad_x=False):
+    """gcn_conv.py:222-296 at one rank.  Returns (grad_x, grad_weight_flat)."""
+    w = weight.reshape(local_weight_shape)  # :232
+    grad_weight = torch.mm(torch.t(agg), grad_output).reshape(-1)  # :237-239, :252
+    grad_agg = torch.mm(grad_output, torch.t(w))  # :256-258
+    grad_x = torch.sparse.mm(a_t_csr, grad_agg)  # :265
+    if flatten_grad_x:  # :271 (layer 0)
+        grad_x = grad_x.reshape(-1)
+    return grad_x, grad_weight
+
+
+def kaiming_uniform_weight(in_channels: int, out_channels: int, generator: torch.Generator, dtype=torch.float32):
+    """gcn_conv.py:332-333 -- kaiming_uniform_(a=sqrt(5)) on an (in, out) tensor.
+
+    torch computes fan_in from size(1), so fan_in = out_channels here; the bound is
+    gain * sqrt(3 / fan_in) with gain = sqrt(2 / (1 + 5)) = 1 / sqrt(fan_in).  The values
+    are drawn on a host generator so both paths share them.  Returned flat, as the
+    reference stores the parameter (:372-390 at one rank).
+    """
+    bound = 1.0 / math.sqrt(out_channels)
+    w = (torch.rand(in_channels, out_channels, generator=generator, dtype=torch.float64) * 2 - 1) * bound
+    return w.to(dtype).reshape(-1)
+
+
+# --------------------------------------------------------------------------
+# plexus/cross_entropy.py
+# --------------------------------------------------------------------------
+def cross_entropy_forward(logits, target, num_nodes: int, num_classes: int):
+    """cross_entropy.py:19-105 at one rank.  Inputs are not mutated (the reference mutates both).
+
+    Returns (loss, softmax, onehot) -- the last two are what the reference saves.
+    """
+    logits = logits.clone()
+    target = target.clone()
+    m, c = logits.shape
+    invalid_classes = torch.arange(c) >= num_classes  # :35-38
+    logits[:, invalid_classes] = float("-inf")  # :40
+    logits_max = torch.max(logits, dim=1)[0]  # :43
+    numerator = torch.exp(logits - logits_max.unsqueeze(1))  # :49
+    denominator = torch.sum(numerator, dim=1)  # :53
+    softmax = numerator / denominator.unsqueeze(1)  # :57
+    invalid_nodes = (torch.arange(m) >= num_nodes) | (target < 0)  # :60-66
+    softmax[invalid_nodes, :] = 0.0  # :67
+    invalid_logits_mask = (target < 0) | (target >= c)  # :70-72
+    target[invalid_logits_mask] = 0  # :75-76
+    onehot = F.one_hot(target, num_classes=c)  # :79
+    onehot[invalid_logits_mask] = 0  # :82
+    eps = 1e-9
+    loss = torch.sum(-torch.log(softmax.clamp(min=eps)) * onehot, dim=1)  # :88-89
+    loss_sum = torch.sum(loss)  # :97
+    return loss_sum / num_nodes, softmax, onehot  # :101
+
+
+def cross_entropy_backward(softmax, onehot, num_nodes: int, grad_output=1.0):
+    """cross_entropy.py:108-114."""
+    return (softmax - onehot) / num_nodes * grad_output
+
+
+# --------------------------------------------------------------------------
+# examples/train.py: Net + train()
+# --------------------------------------------------------------------------
+class OracleNet:
+    """examples/train.py:55-79 with hand-written backward (gcn_conv.py:222-296).
+
+    Layers are (A.H).W with ReLU after every layer except the last, no bias.  The weights
+    (flat, as the reference keeps them) and the input features are the trained tensors.
+    """
+
+    def __init__(self, weights: Sequence[torch.Tensor], dims: Sequence[int]):
+        self.weights = [w.clone() for w in weights]
+        self.dims = list(dims)
+
+    def forward(self, x, adj_shards):
+        saved = []
+        h = x
+        n_layers = len(self.weights)
+        for i, w in enumerate(self.weights):
+            a, a_t = adj_shards[i % len(adj_shards)]  # gcn_conv.py:394-396
+            fshape = (a.shape[1], self.dims[i])
+            wshape = (self.dims[i], self.dims[i + 1])
+            out, agg = gcn_conv_forward(h, a, w, fshape, wshape)
+            pre = out
+            if i != n_layers - 1:
+                out = F.relu(out)  # train.py:77-78
+            saved.append((agg, a_t, wshape, pre))
+            h = out
+        self._saved = saved
+        return h
+
+    def backward(self, grad_logits):
+        g = grad_logits
+        grads_w = [None] * len(self.weights)
+        n_layers = len(self.weights)
+        for i in reversed(range(n_layers)):
+            agg, a_t, wshape, pre = self._saved[i]
+            if i != n_layers - 1:
+                g = g * (pre > 0).to(g.dtype)
+            g, grads_w[i] = gcn_conv_backward(g, agg, self.weights[i], a_t, wshape, flatten_grad_x=(i == 0))
+        return g, grads_w
+
+
+def adamw_step(params, grads, state, lr=3e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0):
+    """torch.optim.AdamW as examples/train.py:155-159 configures it (published update rule)."""
+    state["t"] = state.get("t", 0) + 1
+    t = state["t"]
+    b1, b2 = betas
+    for k, (p, g) in enumerate(zip(params, grads)):
+        m = state.setdefault(("m", k), torch.zeros_like(p))
+        v = state.setdefault(("v", k), torch.zeros_like(p))
+        p.mul_(1 - lr * weight_decay)
+        m.mul_(b1).add_(g, alpha=1 - b1)
+        v.mul_(b2).addcmul_(g, g, value=1 - b2)
+        denom = (v.sqrt() / math.sqrt(1 - b2**t)).add_(eps)
+        p.addcdiv_(m, denom, value=-lr / (1 - b1**t))
+
+
+def train_epochs(x0, weights, dims, adj_shards, labels, num_nodes, num_classes, epochs=10, lr=3e-3):
+    """examples/train.py:83-112,164-193: zero_grad -> fwd -> CE -> bwd -> AdamW over weights and features.
+
+    Returns the loss of every epoch and the final (features, weights).
+    """
+    net = OracleNet(weights, dims)
+    x = x0.clone().reshape(-1)
+    state = {}
+    losses = []
+    for _ in range(epochs):
+        logits = net.forward(x, adj_shards)
+        loss, softmax, onehot = cross_entropy_forward(logits, labels, num_nodes, num_classes)
+        g = cross_entropy_backward(softmax, onehot.to(softmax.dtype), num_nodes)
+        gx, gws = net.backward(g)
+        adamw_step(net.weights + [x], gws + [gx], state, lr=lr)
+        losses.append(float(loss))
+    return losses, x, net.weights
+
+
+# --------------------------------------------------------------------------
+# dropout (not in the reference; counter-based so host and device agree bit for bit)
+# --------------------------------------------------------------------------
+_PHILOX_M0 = np.uint64(0xD2511F53)
+_PHILOX_M1 = np.uint64(0xCD9E8D57)
+_PHILOX_W0 = np.uint32(0x9E3779B9)
+_PHILOX_W1 = np.uint32(0xBB67AE85)
+
+
+def philox4x32_10(counter: np.ndarray, key: Tuple[int, int]) -> np.ndarray:
+    """Philox-4x32-10 (Salmon et al., SC'11) on an array of 4x uint32 counters, shape (n, 4)."""
+    c = counter.astype(np.uint32).copy()
+    k0 = np.uint32(key[0])
+    k1 = np.uint32(key[1])
+    mask = np.uint64(0xFFFFFFFF)
+    with np.errstate(over="ignore"):
+        for _ in range(10):
+            p0 = _PHILOX_M0 * c[:, 0].astype(np.uint64)
+            p1 = _PHILOX_M1 * c[:, 2].astype(np.uint64)
+            hi0 = (p0 >> np.uint64(32)).astype(np.uint32)
+            lo0 = (p0 & mask).astype(np.uint32)
+            hi1 = (p1 >> np.uint64(32)).astype(np.uint32)
+            lo1 = (p1 & mask).astype(np.uint32)
+            n0 = hi1 ^ c[:, 1] ^ k0
+            n2 = hi0 ^ c[:, 3] ^ k1
+            c = np.stack([n0, lo1, n2, lo0], axis=1)
+            k0 = np.uint32(k0 + _PHILOX_W0)
+            k1 = np.uint32(k1 + _PHILOX_W1)
+    return c
+
+
+def dropout_keep_mask(n_elems: int, seed: int, offset: int, p: float) -> np.ndarray:
+    """Keep-mask of element e: word (e % 4) of Philox(counter=(e//4, offset, 0, 0), key=seed) >= p * 2^32."""
+    n4 = (n_elems + 3) // 4
+    ctr = np.zeros((n4, 4), dtype=np.uint32)
+    idx = np.arange(n4, dtype=np.uint64)
+    ctr[:, 0] = (idx & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    ctr[:, 1] = (idx >> np.uint64(32)).astype(np.uint32)
+    ctr[:, 2] = np.uint32(offset & 0xFFFFFFFF)
+    ctr[:, 3] = np.uint32((offset >> 32) & 0xFFFFFFFF)
+    r = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)).reshape(-1)[:n_elems]
+    thresh = np.uint64(min(int(p * 4294967296.0), 4294967295))
+    return r.astype(np.uint64) >= thresh

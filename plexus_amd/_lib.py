@@ -1,0 +1,76 @@
+"""ctypes binding of libplexus_hip.so -- the C ABI declared in include/plexus_hip.h.
+
+There is no CPU fallback: if the shared library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libplexus_hip.so")
+
+_vp = C.c_void_p
+_i64 = C.c_int64
+_i32 = C.c_int32
+_sz = C.c_size_t
+_f32 = C.c_float
+_u32 = C.c_uint
+
+# name -> (restype, argtypes); mirrors include/plexus_hip.h one to one
+SIGNATURES = {
+    "plx_version": (C.c_int, []),
+    "plx_error_string": (C.c_char_p, [C.c_int]),
+    "plx_last_error": (C.c_char_p, []),
+    "plx_csr_narrow_i64": (C.c_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "plx_spmm_segments_host": (C.c_int, [_i64, _vp, _i32, C.POINTER(_i64), C.POINTER(_i64), _vp, _vp, _i64, _vp, _vp, _i64]),
+    "plx_spmm_plan_create": (C.c_int, [C.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _i32, _vp]),
+    "plx_spmm_plan_destroy": (C.c_int, [_vp]),
+    "plx_spmm_plan_info": (_i64, [_vp, C.c_int]),
+    "plx_spmm_workspace_bytes": (_sz, [_vp, _i64]),
+    "plx_spmm_csr_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_spmm_csr_bf16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_gemm_nn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp]),
+    "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_relu_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "plx_relu_bwd_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "plx_softmax_xent_workspace_bytes": (_sz, [_i64, _i64]),
+    "plx_softmax_xent_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "plx_gcn_norm_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+}
+
+PLX_GEMM_RELU = 1
+
+_lib = None
+
+
+class PlexusHipError(RuntimeError):
+    """A libplexus_hip entry point returned a negative status."""
+
+
+def load():
+    """Load the shared library once.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise PlexusHipError(
+                f"{LIB_PATH} is missing: build it with `make -C plexus_amd/csrc` "
+                "(or `python -c 'import __graft_entry__ as g; g.build()'`); there is no CPU fallback"
+            )
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        lib = load()
+        raise PlexusHipError(
+            f"{what}: {lib.plx_error_string(status).decode()} ({status}): {lib.plx_last_error().decode()}"
+        )

@@ -1,0 +1,54 @@
+// Shared host-side helpers of libplexus_hip: error reporting and argument checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "plexus_hip.h"
+
+namespace plx {
+
+void set_last_error(const char *fmt, ...);
+
+inline int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+inline int fail(int status, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    set_last_error("%s", buf);
+    return status;
+}
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+constexpr int kWave = 64;
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace plx
+
+#define PLX_HIP_CHECK(expr)                                                                            \
+    do {                                                                                               \
+        hipError_t e__ = (expr);                                                                       \
+        if (e__ != hipSuccess)                                                                         \
+            return plx::fail(PLX_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__), __FILE__, \
+                             __LINE__);                                                                \
+    } while (0)
+
+#define PLX_LAUNCH_CHECK(name)                                                                        \
+    do {                                                                                               \
+        hipError_t e__ = hipGetLastError();                                                            \
+        if (e__ != hipSuccess)                                                                         \
+            return plx::fail(PLX_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(e__));   \
+    } while (0)
+
+#define PLX_REQUIRE(cond, ...)                                  \
+    do {                                                        \
+        if (!(cond)) return plx::fail(PLX_ERR_INVALID, __VA_ARGS__); \
+    } while (0)

@@ -1,0 +1,129 @@
+// Bandwidth-bound helpers of the GCN layer: ReLU forward/backward for callers that keep the
+// activation outside the layer, and the symmetric GCN normalisation of a CSR matrix.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "common.h"
+
+namespace {
+
+// grid-stride over rows x (cols / 4) float4 lanes when everything is 16-byte aligned, scalars otherwise
+template <bool BWD, bool VEC4>
+__global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const float *__restrict__ in, int64_t ldi,
+                                                   const float *__restrict__ ref, int64_t ldr, float *__restrict__ out,
+                                                   int64_t ldo)
+{
+    const int64_t per_row = VEC4 ? N / 4 : N;
+    const int64_t total = M * per_row;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / per_row;
+        const int64_t c = (i % per_row) * (VEC4 ? 4 : 1);
+        if constexpr (VEC4) {
+            const float4 x = *reinterpret_cast<const float4 *>(in + r * ldi + c);
+            float4 y;
+            if constexpr (BWD) {
+                const float4 m = *reinterpret_cast<const float4 *>(ref + r * ldr + c);
+                y = make_float4(m.x > 0.f ? x.x : 0.f, m.y > 0.f ? x.y : 0.f, m.z > 0.f ? x.z : 0.f, m.w > 0.f ? x.w : 0.f);
+            } else {
+                y = make_float4(fmaxf(x.x, 0.f), fmaxf(x.y, 0.f), fmaxf(x.z, 0.f), fmaxf(x.w, 0.f));
+            }
+            *reinterpret_cast<float4 *>(out + r * ldo + c) = y;
+        } else {
+            const float x = in[r * ldi + c];
+            if constexpr (BWD)
+                out[r * ldo + c] = ref[r * ldr + c] > 0.f ? x : 0.f;
+            else
+                out[r * ldo + c] = fmaxf(x, 0.f);
+        }
+    }
+}
+
+bool aligned4(const void *p, int64_t ld) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0; }
+
+// one wavefront per row: dinv[r] = 1 / sqrt(sum of row r), 0 for an empty or zero row
+__global__ void __launch_bounds__(256) row_dinv_kernel(int64_t M, const int32_t *__restrict__ rowptr,
+                                                       const float *__restrict__ val, float *__restrict__ dinv)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= M) return;
+    const int a = rowptr[r], b = rowptr[r + 1];
+    float s = 0.f;
+    for (int j = a + lane; j < b; j += 64) s += val[j];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if (lane == 0) dinv[r] = s > 0.f ? 1.f / sqrtf(s) : 0.f;
+}
+
+__global__ void __launch_bounds__(256) gcn_scale_kernel(int64_t M, const int32_t *__restrict__ rowptr,
+                                                        const int32_t *__restrict__ col, const float *__restrict__ val,
+                                                        const float *__restrict__ dinv, float *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= M) return;
+    const int a = rowptr[r], b = rowptr[r + 1];
+    const float dr = dinv[r];
+    for (int j = a + lane; j < b; j += 64) out[j] = (dr * val[j]) * dinv[col[j]];
+}
+
+int relu_common(bool bwd, int64_t M, int64_t N, const float *in, int64_t ldi, const float *ref, int64_t ldr, float *out,
+                int64_t ldo, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0, "relu: negative shape");
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(in && out && (!bwd || ref), "relu: NULL operand");
+    PLX_REQUIRE(ldi >= N && ldo >= N && (!bwd || ldr >= N), "relu: leading dimension smaller than N");
+    const bool v4 = N % 4 == 0 && aligned4(in, ldi) && aligned4(out, ldo) && (!bwd || aligned4(ref, ldr));
+    const int64_t total = M * (v4 ? N / 4 : N);
+    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(total, 256), 256 * 32);
+    hipStream_t st = plx::as_stream(stream);
+    if (bwd) {
+        if (v4)
+            relu_kernel<true, true><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+        else
+            relu_kernel<true, false><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+    } else {
+        if (v4)
+            relu_kernel<false, true><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+        else
+            relu_kernel<false, false><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+    }
+    PLX_LAUNCH_CHECK("relu_kernel");
+    return PLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream)
+{
+    return relu_common(false, M, N, X, ldx, nullptr, 0, Y, ldy, stream);
+}
+
+int plx_relu_bwd_f32(int64_t M, int64_t N, const float *dY, int64_t lddy, const float *Y, int64_t ldy, float *dX,
+                     int64_t lddx, void *stream)
+{
+    return relu_common(true, M, N, dY, lddy, Y, ldy, dX, lddx, stream);
+}
+
+int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, const float *val_in, float *val_out,
+                         float *dinv, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && M < (1ll << 31) - 1, "gcn_norm: bad row count");
+    if (M == 0) return PLX_OK;
+    PLX_REQUIRE(rowptr && col && val_in && val_out && dinv, "gcn_norm: NULL operand");
+    hipStream_t st = plx::as_stream(stream);
+    const unsigned blocks = (unsigned)plx::ceil_div(M, 4);
+    row_dinv_kernel<<<blocks, 256, 0, st>>>(M, rowptr, val_in, dinv);
+    PLX_LAUNCH_CHECK("row_dinv_kernel");
+    gcn_scale_kernel<<<blocks, 256, 0, st>>>(M, rowptr, col, val_in, dinv, val_out);
+    PLX_LAUNCH_CHECK("gcn_scale_kernel");
+    return PLX_OK;
+}
+
+}  // extern "C"

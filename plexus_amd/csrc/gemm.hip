@@ -1,0 +1,407 @@
+// Dense products of the GCN layer on the gfx950 matrix cores, fp32 in / fp32 accumulate.
+//
+//   NN  C[M x N] = A[M x K] . B[K x N]            OUT      = AGG . W
+//   NT  C[M x N] = (A*mask)[M x K] . B[N x K]^T   GRAD_AGG = GRAD_OUT . W^T
+//   TN  C[K x N] = A[M x K]^T . (B*mask)[M x N]   GRAD_W   = AGG^T . GRAD_OUT   (split over M)
+//
+// All three are "tall-skinny": one dimension is the node count (millions), the others are feature
+// widths (tens to hundreds).  One kernel template covers them.  A workgroup of four wavefronts owns
+// a 128 x BN output tile (each wavefront 32 x BN = TN tiles of v_mfma_f32_32x32x2_f32) and walks
+// the contraction in chunks of 32.  Chunks are fetched global -> registers -> LDS with two LDS
+// buffers, so the fetch of chunk c+1 overlaps the MFMAs of chunk c.
+//
+// LDS tile layouts are chosen so that the global side is always read along contiguous memory:
+//   "x-major"  T[x][k] (row stride 36 floats): rows of the source are rows of the tile; a lane reads
+//              four consecutive k with one 128-bit LDS load;
+//   "k-major"  T[k][x]: the source is already contraction-major (B of NN, both operands of TN); a
+//              lane reads single floats, consecutive lanes consecutive x.
+// Both layouts agree on which k a lane feeds to MFMA number (s, m) of a chunk: k = 8 s + 4 h + m with
+// h = lane / 32, which is a permutation of the chunk and therefore leaves the product unchanged.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128;   // output rows per workgroup
+constexpr int kBK = 32;    // contraction chunk
+constexpr int kXS = 36;    // row stride of an x-major tile (floats)
+constexpr int kThreads = 256;
+
+enum Mode { kNN = 0, kNT = 1, kTN = 2 };
+
+struct GemmArgs {
+    const float *A;
+    const float *B;
+    float *C;
+    const float *mask;
+    int64_t lda, ldb, ldc, ldmask;
+    int64_t M, N, K;       // as in the header of each entry point
+    int64_t rows_per_split;  // TN only
+    float *ws;             // TN only: partial tiles [split][Kpad][Npad]
+    int64_t ws_ld, ws_slab;
+    unsigned flags;
+    int a_vec, b_vec, m_vec;  // 1 when 128-bit global loads of that operand are legal
+};
+
+// ROWS x COLS tile of a row-major source, fetched as float4 per thread, zero-filled outside the source
+template <int ROWS, int COLS, int STRIDE>
+struct Tile {
+    static constexpr int kV4PerRow = COLS / 4;
+    static constexpr int kPer = ROWS * COLS / 4 / kThreads;
+    static_assert(ROWS * COLS / 4 % kThreads == 0 && kPer >= 1, "tile does not divide over the workgroup");
+    float4 reg[kPer];
+
+    __device__ __forceinline__ void fetch(const float *__restrict__ src, int64_t ld, int64_t r0, int64_t c0, int64_t nrows,
+                                          int64_t ncols, int vec_ok, const float *__restrict__ mask, int64_t ldm,
+                                          int mvec_ok)
+    {
+#pragma unroll
+        for (int p = 0; p < kPer; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            const int64_t r = r0 + idx / kV4PerRow;
+            const int64_t c = c0 + (idx % kV4PerRow) * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (r < nrows && c < ncols) {
+                const float *q = src + r * ld + c;
+                if (vec_ok && c + 3 < ncols) {
+                    v = *reinterpret_cast<const float4 *>(q);
+                } else {
+                    v.x = q[0];
+                    if (c + 1 < ncols) v.y = q[1];
+                    if (c + 2 < ncols) v.z = q[2];
+                    if (c + 3 < ncols) v.w = q[3];
+                }
+                if (mask != nullptr) {
+                    const float *mq = mask + r * ldm + c;
+                    float4 m = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (mvec_ok && c + 3 < ncols) {
+                        m = *reinterpret_cast<const float4 *>(mq);
+                    } else {
+                        m.x = mq[0];
+                        if (c + 1 < ncols) m.y = mq[1];
+                        if (c + 2 < ncols) m.z = mq[2];
+                        if (c + 3 < ncols) m.w = mq[3];
+                    }
+                    v.x = m.x > 0.f ? v.x : 0.f;
+                    v.y = m.y > 0.f ? v.y : 0.f;
+                    v.z = m.z > 0.f ? v.z : 0.f;
+                    v.w = m.w > 0.f ? v.w : 0.f;
+                }
+            }
+            reg[p] = v;
+        }
+    }
+
+    __device__ __forceinline__ void stash(float *lds) const
+    {
+#pragma unroll
+        for (int p = 0; p < kPer; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            const int r = idx / kV4PerRow;
+            const int c = (idx % kV4PerRow) * 4;
+            *reinterpret_cast<float4 *>(lds + r * STRIDE + c) = reg[p];
+        }
+    }
+};
+
+template <int MODE, int TN>
+__global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr bool kAX = (MODE != kTN);  // A tile x-major?
+    constexpr bool kBX = (MODE == kNT);  // B tile x-major?
+    constexpr int kAStride = kAX ? kXS : kBM;
+    constexpr int kBStride = kBX ? kXS : BN;
+    constexpr int kASize = kAX ? kBM * kXS : kBK * kBM;
+    constexpr int kBSize = kBX ? BN * kXS : kBK * BN;
+    using ATile = Tile<(kAX ? kBM : kBK), (kAX ? kBK : kBM), kAStride>;
+    using BTile = Tile<(kBX ? BN : kBK), (kBX ? kBK : BN), kBStride>;
+
+    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+    auto a_buf = [&](int i) { return lds + i * kASize; };
+    auto b_buf = [&](int i) { return lds + 2 * kASize + i * kBSize; };
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+
+    // output tile origin and contraction range
+    int64_t row0, col0, kbeg, kend;
+    if constexpr (MODE == kTN) {
+        row0 = (int64_t)blockIdx.y * kBM;  // rows of C = columns of A
+        col0 = (int64_t)blockIdx.z * BN;
+        kbeg = (int64_t)blockIdx.x * g.rows_per_split;
+        kend = min(kbeg + g.rows_per_split, g.M);
+    } else {
+        row0 = (int64_t)blockIdx.x * kBM;
+        col0 = (int64_t)blockIdx.y * BN;
+        kbeg = 0;
+        kend = g.K;
+    }
+
+    ATile at;
+    BTile bt;
+    auto fetch = [&](int64_t k0) {
+        if constexpr (MODE == kNN) {
+            at.fetch(g.A, g.lda, row0, k0, g.M, g.K, g.a_vec, nullptr, 0, 0);
+            bt.fetch(g.B, g.ldb, k0, col0, g.K, g.N, g.b_vec, nullptr, 0, 0);
+        } else if constexpr (MODE == kNT) {
+            at.fetch(g.A, g.lda, row0, k0, g.M, g.K, g.a_vec, g.mask, g.ldmask, g.m_vec);
+            bt.fetch(g.B, g.ldb, col0, k0, g.N, g.K, g.b_vec, nullptr, 0, 0);
+        } else {
+            at.fetch(g.A, g.lda, k0, row0, kend, g.K, g.a_vec, nullptr, 0, 0);
+            bt.fetch(g.B, g.ldb, k0, col0, kend, g.N, g.b_vec, g.mask, g.ldmask, g.m_vec);
+        }
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    int buf = 0;
+    if (kbeg < kend) {
+        fetch(kbeg);
+        at.stash(a_buf(0));
+        bt.stash(b_buf(0));
+    }
+    __syncthreads();
+
+    for (int64_t k0 = kbeg; k0 < kend; k0 += kBK) {
+        const bool more = k0 + kBK < kend;
+        if (more) fetch(k0 + kBK);
+
+        const float *as = a_buf(buf);
+        const float *bs = b_buf(buf);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            float a[4];
+            if constexpr (kAX) {
+                const float4 t4 = *reinterpret_cast<const float4 *>(as + (wave * 32 + li) * kXS + 8 * s + 4 * h);
+                a[0] = t4.x;
+                a[1] = t4.y;
+                a[2] = t4.z;
+                a[3] = t4.w;
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) a[m] = as[(8 * s + 4 * h + m) * kAStride + wave * 32 + li];
+            }
+            float b[TN][4];
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                if constexpr (kBX) {
+                    const float4 t4 = *reinterpret_cast<const float4 *>(bs + (t * 32 + li) * kXS + 8 * s + 4 * h);
+                    b[t][0] = t4.x;
+                    b[t][1] = t4.y;
+                    b[t][2] = t4.z;
+                    b[t][3] = t4.w;
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) b[t][m] = bs[(8 * s + 4 * h + m) * kBStride + t * 32 + li];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[m], b[t][m], acc[t], 0, 0, 0);
+        }
+
+        if (more) {
+            at.stash(a_buf(buf ^ 1));
+            bt.stash(b_buf(buf ^ 1));
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // accumulator register v of a lane is C[8 (v / 4) + 4 h + v % 4][lane % 32] of the 32 x 32 tile
+    float *out;
+    int64_t ldo, nrows, ncols;
+    if constexpr (MODE == kTN) {
+        if (g.ws != nullptr) {
+            out = g.ws + (int64_t)blockIdx.x * g.ws_slab;
+            ldo = g.ws_ld;
+        } else {
+            out = g.C;
+            ldo = g.ldc;
+        }
+        nrows = g.K;
+        ncols = g.N;
+    } else {
+        out = g.C;
+        ldo = g.ldc;
+        nrows = g.M;
+        ncols = g.N;
+    }
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int64_t c = col0 + t * 32 + li;
+        if (c >= ncols) continue;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t r = row0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+            if (r < nrows) {
+                float x = acc[t][v];
+                if (relu) x = fmaxf(x, 0.f);
+                out[r * ldo + c] = x;
+            }
+        }
+    }
+}
+
+// C[e] = sum over splits of ws[s][e], s ascending within four interleaved chains that are then
+// added in chain order -- a fixed order, so the result does not depend on scheduling.
+__global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ ws, int64_t ws_ld, int64_t ws_slab,
+                                                      int splits, int64_t rows, int64_t cols, float *__restrict__ C,
+                                                      int64_t ldc)
+{
+    __shared__ float part[4][64];
+    const int e_local = threadIdx.x & 63;
+    const int chain = threadIdx.x >> 6;
+    const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
+    const int64_t total = rows * cols;
+    float s = 0.f;
+    int64_t r = 0, c = 0;
+    if (e < total) {
+        r = e / cols;
+        c = e % cols;
+        const float *p = ws + r * ws_ld + c;
+        for (int i = chain; i < splits; i += 4) s += p[(int64_t)i * ws_slab];
+    }
+    part[chain][e_local] = s;
+    __syncthreads();
+    if (chain == 0 && e < total) C[r * ldc + c] = ((part[0][e_local] + part[1][e_local]) + part[2][e_local]) + part[3][e_local];
+}
+
+int vec_ok(const float *p, int64_t ld) { return (p == nullptr || (reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0)) ? 1 : 0; }
+
+int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
+
+template <int MODE>
+void launch_gemm(const GemmArgs &g, int tn, dim3 grid, hipStream_t st)
+{
+    switch (tn) {
+        case 1: gemm_f32_kernel<MODE, 1><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_f32_kernel<MODE, 2><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_f32_kernel<MODE, 4><<<grid, kThreads, 0, st>>>(g); break;
+    }
+}
+
+int check_common(const char *who, int64_t M, int64_t N, int64_t K, const void *A, const void *B, const void *C)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative dimension", who);
+    PLX_REQUIRE(N < (1ll << 30) && K < (1ll << 30), "%s: dimension too large", who);
+    if (M == 0 || N == 0) return 1;
+    PLX_REQUIRE(C != nullptr, "%s: NULL output", who);
+    PLX_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "%s: NULL operand", who);
+    return PLX_OK;
+}
+
+// TN split policy: enough workgroups to fill 256 compute units a few times over, at least 256 rows each
+int64_t tn_splits(int64_t M, int64_t N, int64_t K)
+{
+    const int64_t tiles = plx::ceil_div(K, kBM) * plx::ceil_div(N, 32 * pick_tn(N));
+    int64_t want = std::max<int64_t>(1, 1024 / tiles);
+    int64_t by_rows = std::max<int64_t>(1, M / 256);
+    return std::max<int64_t>(1, std::min(want, by_rows));
+}
+
+}  // namespace
+
+extern "C" {
+
+int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, unsigned flags, void *stream)
+{
+    int rc = check_common("gemm_nn", M, N, K, A, B, C);
+    if (rc != PLX_OK) return rc < 0 ? rc : PLX_OK;
+    PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_nn: leading dimension too small");
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+    g.M = M; g.N = N; g.K = K; g.flags = flags;
+    g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb);
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
+    launch_gemm<kNN>(g, tn, grid, plx::as_stream(stream));
+    PLX_LAUNCH_CHECK("gemm_f32_kernel<NN>");
+    return PLX_OK;
+}
+
+int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *stream)
+{
+    int rc = check_common("gemm_nt", M, N, K, A, B, C);
+    if (rc != PLX_OK) return rc < 0 ? rc : PLX_OK;
+    PLX_REQUIRE(lda >= K && ldb >= K && ldc >= N, "gemm_nt: leading dimension too small");
+    PLX_REQUIRE(mask == nullptr || ldmask >= K, "gemm_nt: mask leading dimension too small");
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
+    g.M = M; g.N = N; g.K = K;
+    g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
+    launch_gemm<kNT>(g, tn, grid, plx::as_stream(stream));
+    PLX_LAUNCH_CHECK("gemm_f32_kernel<NT>");
+    return PLX_OK;
+}
+
+size_t plx_gemm_tn_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t splits = tn_splits(M, N, K);
+    if (splits <= 1) return 0;
+    const int64_t ld = (N + 3) / 4 * 4;
+    return (size_t)splits * (size_t)K * (size_t)ld * sizeof(float);
+}
+
+int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *workspace,
+                    size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_tn: negative dimension");
+    if (K == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(C != nullptr, "gemm_tn: NULL output");
+    PLX_REQUIRE(M == 0 || (A != nullptr && B != nullptr), "gemm_tn: NULL operand");
+    PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_tn: leading dimension too small");
+    PLX_REQUIRE(mask == nullptr || ldmask >= N, "gemm_tn: mask leading dimension too small");
+    hipStream_t st = plx::as_stream(stream);
+    const int64_t splits = tn_splits(std::max<int64_t>(M, 1), N, K);
+    const size_t need = plx_gemm_tn_workspace_bytes(M, N, K);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
+        return plx::fail(PLX_ERR_WORKSPACE, "gemm_tn: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
+    g.M = M; g.N = N; g.K = K;
+    g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
+    // every split covers a multiple of the 32-row chunk so that chunk boundaries do not depend on the split
+    g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;
+    const int64_t used = plx::ceil_div(std::max<int64_t>(M, 1), g.rows_per_split);
+    if (splits > 1) {
+        g.ws = static_cast<float *>(workspace);
+        g.ws_ld = (N + 3) / 4 * 4;
+        g.ws_slab = K * g.ws_ld;
+    }
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
+    launch_gemm<kTN>(g, tn, grid, st);
+    PLX_LAUNCH_CHECK("gemm_f32_kernel<TN>");
+    if (splits > 1) {
+        const int64_t total = K * N;
+        gemm_tn_reduce<<<(unsigned)plx::ceil_div(total, 64), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc);
+        PLX_LAUNCH_CHECK("gemm_tn_reduce");
+    }
+    return PLX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,613 @@
+// CSR SpMM  Y = A . H  for gfx950.
+//
+// Work decomposition (no atomics, fixed summation order):
+//   * one 64-lane wavefront per task; a task is either a whole row of A (rows of at most
+//     seg_len non-zeros) or one segment of a longer row;
+//   * segment tasks come first in the grid (they are the longest) and write fp32 partial rows to a
+//     workspace; a second small kernel adds the partial rows of each split row in segment order;
+//   * inside a task the 64 lanes are cut into G = 64 / LPR groups of LPR lanes.  A group covers
+//     one row of H with VEC-element (up to 128-bit) loads per lane, so one gather instruction of
+//     the wavefront pulls G rows of H.  Group g handles non-zeros g, g+G, g+2G, ... of the task;
+//     the G partial sums are combined with cross-lane shuffles at the end;
+//   * column indices and values are read 64 at a time, one per lane (coalesced), and handed to the
+//     groups through cross-lane permutes, so no lane re-reads them from memory;
+//   * for rows of H wider than 64 lanes x VEC, each lane keeps NACC accumulator vectors; rows wider
+//     than that are tiled over gridDim.y.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+using plx::kWave;
+
+struct SpmmArgs {
+    const int32_t *rowptr;
+    const int32_t *col;
+    const float *val;
+    const void *H;
+    void *Y;
+    float *ws;
+    const int32_t *seg_begin;
+    const int32_t *seg_end;
+    int64_t ldh;
+    int64_t ldy;
+    int64_t ldws;
+    int32_t M;
+    int32_t n_seg;
+    int32_t D;
+    int32_t seg_len;
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // quiet the NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                  // round to nearest even
+    return u >> 16;
+}
+
+// ---- VEC-element loads / stores, fp32 or bf16 storage, fp32 in registers ----
+template <typename T, int VEC>
+struct VecIO;
+
+template <>
+struct VecIO<float, 1> {
+    static __device__ __forceinline__ void load(const float *p, float (&o)[1]) { o[0] = *p; }
+    static __device__ __forceinline__ void store(float *p, const float (&v)[1]) { *p = v[0]; }
+};
+template <>
+struct VecIO<float, 2> {
+    static __device__ __forceinline__ void load(const float *p, float (&o)[2])
+    {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        o[0] = t.x;
+        o[1] = t.y;
+    }
+    static __device__ __forceinline__ void store(float *p, const float (&v)[2])
+    {
+        *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+    }
+};
+template <>
+struct VecIO<float, 4> {
+    static __device__ __forceinline__ void load(const float *p, float (&o)[4])
+    {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        o[0] = t.x;
+        o[1] = t.y;
+        o[2] = t.z;
+        o[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float *p, const float (&v)[4])
+    {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <>
+struct VecIO<uint16_t, 1> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&o)[1]) { o[0] = bf16_to_f32(*p); }
+    static __device__ __forceinline__ void store(uint16_t *p, const float (&v)[1]) { *p = (uint16_t)f32_to_bf16(v[0]); }
+};
+template <>
+struct VecIO<uint16_t, 2> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&o)[2])
+    {
+        const uint32_t t = *reinterpret_cast<const uint32_t *>(p);
+        o[0] = __uint_as_float(t << 16);
+        o[1] = __uint_as_float(t & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(uint16_t *p, const float (&v)[2])
+    {
+        *reinterpret_cast<uint32_t *>(p) = f32_to_bf16(v[0]) | (f32_to_bf16(v[1]) << 16);
+    }
+};
+template <>
+struct VecIO<uint16_t, 4> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&o)[4])
+    {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        o[0] = __uint_as_float(t.x << 16);
+        o[1] = __uint_as_float(t.x & 0xffff0000u);
+        o[2] = __uint_as_float(t.y << 16);
+        o[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(uint16_t *p, const float (&v)[4])
+    {
+        uint2 t;
+        t.x = f32_to_bf16(v[0]) | (f32_to_bf16(v[1]) << 16);
+        t.y = f32_to_bf16(v[2]) | (f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2 *>(p) = t;
+    }
+};
+template <>
+struct VecIO<uint16_t, 8> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&o)[8])
+    {
+        const uint4 t = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i] = __uint_as_float(w[i] << 16);
+            o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ void store(uint16_t *p, const float (&v)[8])
+    {
+        uint4 t;
+        t.x = f32_to_bf16(v[0]) | (f32_to_bf16(v[1]) << 16);
+        t.y = f32_to_bf16(v[2]) | (f32_to_bf16(v[3]) << 16);
+        t.z = f32_to_bf16(v[4]) | (f32_to_bf16(v[5]) << 16);
+        t.w = f32_to_bf16(v[6]) | (f32_to_bf16(v[7]) << 16);
+        *reinterpret_cast<uint4 *>(p) = t;
+    }
+};
+
+// fp32 store of a VEC-element register vector (the workspace is fp32 whatever the storage type)
+template <int VEC>
+__device__ __forceinline__ void store_f32(float *p, const float (&v)[VEC])
+{
+    if constexpr (VEC == 8) {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        VecIO<float, VEC>::store(p, v);
+    }
+}
+
+// value of `x` held by lane `src`; `src` differs between lane groups when G > 1
+template <int G>
+__device__ __forceinline__ int pick_i(int x, int src)
+{
+    if constexpr (G == 1)
+        return __builtin_amdgcn_readlane(x, src);
+    else
+        return __shfl(x, src, kWave);
+}
+template <int G>
+__device__ __forceinline__ float pick_f(float x, int src)
+{
+    return __int_as_float(pick_i<G>(__float_as_int(x), src));
+}
+
+template <typename TIN, typename TOUT, int VEC, int LPR, int NACC>
+__global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
+{
+    constexpr int G = kWave / LPR;
+    static_assert(G == 1 || NACC == 1, "several accumulator vectors only with one group");
+    // gathers kept in flight per lane = U * NACC
+    constexpr int U = (G >= 8) ? 1 : (G == 4) ? 2 : (G == 2) ? 4 : (NACC <= 2 ? 4 : (NACC <= 4 ? 2 : 1));
+    constexpr int TILE = LPR * VEC * NACC;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t task = (int64_t)blockIdx.x * 4 + wid;
+    const int g = lane / LPR;
+    const int t = lane % LPR;
+    const int d0 = blockIdx.y * TILE;
+
+    int a, b;
+    bool to_ws;
+    int64_t out_row;
+    if (task < p.n_seg) {
+        a = p.seg_begin[task];
+        b = p.seg_end[task];
+        to_ws = true;
+        out_row = task;
+    } else {
+        const int64_t r = task - p.n_seg;
+        if (r >= p.M) return;
+        a = p.rowptr[r];
+        b = p.rowptr[r + 1];
+        if (b - a > p.seg_len) return;  // split row: its segments are separate tasks
+        to_ws = false;
+        out_row = r;
+    }
+    a = __builtin_amdgcn_readfirstlane(a);
+    b = __builtin_amdgcn_readfirstlane(b);
+
+    // element offsets of this lane's vectors inside a row of H; lanes past the row width
+    // gather element 0 instead (a valid address) and never store
+    int off[NACC];
+    bool ok[NACC];
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) {
+        const int e = d0 + (t + k * LPR) * VEC;
+        ok[k] = e < p.D;
+        off[k] = ok[k] ? e : 0;
+    }
+
+    float acc[NACC][VEC];
+#pragma unroll
+    for (int k = 0; k < NACC; ++k)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[k][e] = 0.f;
+
+    const TIN *__restrict__ Hp = static_cast<const TIN *>(p.H);
+
+    for (int j0 = a; j0 < b; j0 += kWave) {
+        const int n = min(kWave, b - j0);
+        int cl = 0;
+        float vl = 0.f;
+        if (lane < n) {
+            cl = p.col[j0 + lane];
+            vl = p.val[j0 + lane];
+        }
+        int i = 0;
+        for (; i + G * U <= n; i += G * U) {
+            int c[U];
+            float v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int src = i + u * G + g;
+                c[u] = pick_i<G>(cl, src);
+                v[u] = pick_f<G>(vl, src);
+            }
+            float h[U][NACC][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const TIN *row = Hp + (int64_t)c[u] * p.ldh;
+#pragma unroll
+                for (int k = 0; k < NACC; ++k) VecIO<TIN, VEC>::load(row + off[k], h[u][k]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int k = 0; k < NACC; ++k)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[k][e] = fmaf(v[u], h[u][k][e], acc[k][e]);
+        }
+        for (; i < n; i += G) {
+            const int src = i + g;
+            const int c = pick_i<G>(cl, src & (kWave - 1));
+            const float v = pick_f<G>(vl, src & (kWave - 1));
+            if (src < n) {
+                const TIN *row = Hp + (int64_t)c * p.ldh;
+#pragma unroll
+                for (int k = 0; k < NACC; ++k) {
+                    float h[VEC];
+                    VecIO<TIN, VEC>::load(row + off[k], h);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[k][e] = fmaf(v, h[e], acc[k][e]);
+                }
+            }
+        }
+    }
+
+    // combine the G group sums: group g ^ 1, g ^ 2, ... (fixed order)
+    if constexpr (G > 1) {
+#pragma unroll
+        for (int o = LPR; o < kWave; o <<= 1)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[0][e] += __shfl_xor(acc[0][e], o, kWave);
+    }
+
+    if (g == 0) {
+        if (to_ws) {
+            float *dst = p.ws + out_row * p.ldws;
+#pragma unroll
+            for (int k = 0; k < NACC; ++k)
+                if (ok[k]) store_f32<VEC>(dst + off[k], acc[k]);
+        } else {
+            TOUT *dst = static_cast<TOUT *>(p.Y) + out_row * p.ldy;
+#pragma unroll
+            for (int k = 0; k < NACC; ++k)
+                if (ok[k]) VecIO<TOUT, VEC>::store(dst + off[k], acc[k]);
+        }
+    }
+}
+
+// Y[row q] = sum over the segments of split row q, in segment order.
+template <typename TOUT>
+__global__ void __launch_bounds__(256) spmm_reduce_split_rows(const float *__restrict__ ws, int64_t ldws,
+                                                              const int32_t *__restrict__ long_rows,
+                                                              const int32_t *__restrict__ seg_first, int32_t D,
+                                                              TOUT *__restrict__ Y, int64_t ldy)
+{
+    const int q = blockIdx.x;
+    const int d = blockIdx.y * blockDim.x + threadIdx.x;
+    if (d >= D) return;
+    const int s0 = seg_first[q];
+    const int s1 = seg_first[q + 1];
+    float s = 0.f;
+    for (int i = s0; i < s1; ++i) s += ws[(int64_t)i * ldws + d];
+    TOUT *dst = Y + (int64_t)long_rows[q] * ldy + d;
+    if constexpr (sizeof(TOUT) == 4)
+        *dst = s;
+    else
+        *dst = (uint16_t)f32_to_bf16(s);
+}
+
+__global__ void narrow_i64_kernel(int64_t n, const int64_t *__restrict__ src, int32_t *__restrict__ dst)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = (int32_t)src[i];
+}
+
+int64_t ws_ld(int64_t D) { return (D + 3) / 4 * 4; }
+
+}  // namespace
+
+struct plx_spmm_plan {
+    int64_t M, K, nnz;
+    const int32_t *rowptr;
+    const int32_t *col;
+    int32_t seg_len;
+    int64_t n_long, n_seg;
+    int32_t *tables;  // device: long_rows[n_long] | seg_first[n_long+1] | seg_begin[n_seg] | seg_end[n_seg]
+    const int32_t *long_rows, *seg_first, *seg_begin, *seg_end;
+};
+
+namespace {
+
+template <typename TIN, typename TOUT, int VEC, int LPR, int NACC>
+void launch_variant(const SpmmArgs &a, dim3 grid, hipStream_t st)
+{
+    spmm_csr_kernel<TIN, TOUT, VEC, LPR, NACC><<<grid, 256, 0, st>>>(a);
+}
+
+template <typename TIN, typename TOUT, int VEC>
+int launch_for_vec(const SpmmArgs &a, int lpr, int nacc, dim3 grid, hipStream_t st)
+{
+    switch (lpr) {
+        case 4: launch_variant<TIN, TOUT, VEC, 4, 1>(a, grid, st); return 0;
+        case 8: launch_variant<TIN, TOUT, VEC, 8, 1>(a, grid, st); return 0;
+        case 16: launch_variant<TIN, TOUT, VEC, 16, 1>(a, grid, st); return 0;
+        case 32: launch_variant<TIN, TOUT, VEC, 32, 1>(a, grid, st); return 0;
+        default: break;
+    }
+    switch (nacc) {
+        case 1: launch_variant<TIN, TOUT, VEC, 64, 1>(a, grid, st); return 0;
+        case 2: launch_variant<TIN, TOUT, VEC, 64, 2>(a, grid, st); return 0;
+        case 3: launch_variant<TIN, TOUT, VEC, 64, 3>(a, grid, st); return 0;
+        case 4: launch_variant<TIN, TOUT, VEC, 64, 4>(a, grid, st); return 0;
+        case 5: launch_variant<TIN, TOUT, VEC, 64, 5>(a, grid, st); return 0;
+        case 6: launch_variant<TIN, TOUT, VEC, 64, 6>(a, grid, st); return 0;
+        case 7: launch_variant<TIN, TOUT, VEC, 64, 7>(a, grid, st); return 0;
+        case 8: launch_variant<TIN, TOUT, VEC, 64, 8>(a, grid, st); return 0;
+        default: return -1;
+    }
+}
+
+template <typename T>
+int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t ldh, int64_t D, T *Y, int64_t ldy,
+              void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
+    PLX_REQUIRE(D >= 0 && D < (1ll << 30), "spmm: bad feature width D=%lld", (long long)D);
+    if (plan->M == 0 || D == 0) return PLX_OK;
+    PLX_REQUIRE(val && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
+    PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
+                (long long)ldh, (long long)ldy, (long long)D);
+    const size_t need = plx_spmm_workspace_bytes(plan, D);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
+        return plx::fail(PLX_ERR_WORKSPACE, "spmm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    PLX_REQUIRE(need == 0 || (reinterpret_cast<uintptr_t>(workspace) % 16) == 0, "spmm: workspace not 16-byte aligned");
+
+    constexpr int kMaxVec = 16 / (int)sizeof(T);
+    int vec = kMaxVec;
+    while (vec > 1 && (D % vec || ldh % vec || ldy % vec || reinterpret_cast<uintptr_t>(H) % (vec * sizeof(T)) ||
+                       reinterpret_cast<uintptr_t>(Y) % (vec * sizeof(T))))
+        vec >>= 1;
+    const int64_t units = D / vec;
+    int lpr = 4;
+    while (lpr < kWave && lpr < units) lpr <<= 1;
+    int nacc = 1, tiles = 1;
+    if (lpr == kWave) {
+        const int64_t chunks = plx::ceil_div(units, kWave);
+        tiles = (int)plx::ceil_div(chunks, 8);
+        nacc = (int)plx::ceil_div(chunks, tiles);
+    }
+
+    SpmmArgs a;
+    a.rowptr = plan->rowptr;
+    a.col = plan->col;
+    a.val = val;
+    a.H = H;
+    a.Y = Y;
+    a.ws = static_cast<float *>(workspace);
+    a.seg_begin = plan->seg_begin;
+    a.seg_end = plan->seg_end;
+    a.ldh = ldh;
+    a.ldy = ldy;
+    a.ldws = ws_ld(D);
+    a.M = (int32_t)plan->M;
+    a.n_seg = (int32_t)plan->n_seg;
+    a.D = (int32_t)D;
+    a.seg_len = plan->seg_len;
+
+    hipStream_t st = plx::as_stream(stream);
+    const int64_t tasks = plan->M + plan->n_seg;
+    dim3 grid((unsigned)plx::ceil_div(tasks, 4), (unsigned)tiles, 1);
+    int rc = -1;
+    switch (vec) {
+        case 1: rc = launch_for_vec<T, T, 1>(a, lpr, nacc, grid, st); break;
+        case 2: rc = launch_for_vec<T, T, 2>(a, lpr, nacc, grid, st); break;
+        case 4: rc = launch_for_vec<T, T, 4>(a, lpr, nacc, grid, st); break;
+        case 8:
+            if constexpr (kMaxVec == 8) rc = launch_for_vec<T, T, 8>(a, lpr, nacc, grid, st);
+            break;
+        default: break;
+    }
+    if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "spmm: no kernel for vec=%d lpr=%d nacc=%d", vec, lpr, nacc);
+    PLX_LAUNCH_CHECK("spmm_csr_kernel");
+
+    if (plan->n_long > 0) {
+        const int bs = (int)std::min<int64_t>(256, plx::ceil_div(D, 64) * 64);
+        dim3 rgrid((unsigned)plan->n_long, (unsigned)plx::ceil_div(D, bs), 1);
+        spmm_reduce_split_rows<T><<<rgrid, bs, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)D, Y, ldy);
+        PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
+    }
+    return PLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int plx_csr_narrow_i64(int64_t M, int64_t nnz, const int64_t *rowptr64, const int64_t *col64, int32_t *rowptr32,
+                       int32_t *col32, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && nnz >= 0, "csr_narrow: negative size");
+    PLX_REQUIRE(nnz < (1ll << 31) && M < (1ll << 31) - 1, "csr_narrow: M=%lld nnz=%lld do not fit int32", (long long)M,
+                (long long)nnz);
+    PLX_REQUIRE(rowptr64 && rowptr32, "csr_narrow: NULL rowptr");
+    PLX_REQUIRE(nnz == 0 || (col64 && col32), "csr_narrow: NULL col");
+    hipStream_t st = plx::as_stream(stream);
+    {
+        const int64_t n = M + 1;
+        const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(n, 256), 65536);
+        narrow_i64_kernel<<<blocks, 256, 0, st>>>(n, rowptr64, rowptr32);
+        PLX_LAUNCH_CHECK("narrow_i64_kernel");
+    }
+    if (nnz > 0) {
+        const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(nnz, 256), 65536);
+        narrow_i64_kernel<<<blocks, 256, 0, st>>>(nnz, col64, col32);
+        PLX_LAUNCH_CHECK("narrow_i64_kernel");
+    }
+    return PLX_OK;
+}
+
+int plx_spmm_segments_host(int64_t M, const int32_t *rowptr_host, int32_t seg_len, int64_t *n_long, int64_t *n_seg,
+                           int32_t *long_rows_host, int32_t *seg_first_host, int64_t cap_long, int32_t *seg_begin_host,
+                           int32_t *seg_end_host, int64_t cap_seg)
+{
+    PLX_REQUIRE(M >= 0 && rowptr_host != nullptr && seg_len > 0, "spmm_segments: bad arguments");
+    PLX_REQUIRE(n_long != nullptr && n_seg != nullptr, "spmm_segments: NULL count outputs");
+    int64_t nl = 0, ns = 0;
+    for (int64_t r = 0; r < M; ++r) {
+        const int64_t a = rowptr_host[r], b = rowptr_host[r + 1];
+        PLX_REQUIRE(b >= a, "spmm_segments: rowptr decreases at row %lld", (long long)r);
+        const int64_t len = b - a;
+        if (len <= seg_len) continue;
+        const int64_t parts = plx::ceil_div(len, seg_len);
+        const int64_t base = len / parts, extra = len % parts;  // the first `extra` segments get one more
+        if (long_rows_host && nl < cap_long) long_rows_host[nl] = (int32_t)r;
+        if (seg_first_host && nl < cap_long) seg_first_host[nl] = (int32_t)ns;
+        int64_t pos = a;
+        for (int64_t s = 0; s < parts; ++s) {
+            const int64_t l = base + (s < extra ? 1 : 0);
+            if (seg_begin_host && ns < cap_seg) seg_begin_host[ns] = (int32_t)pos;
+            if (seg_end_host && ns < cap_seg) seg_end_host[ns] = (int32_t)(pos + l);
+            pos += l;
+            ++ns;
+        }
+        ++nl;
+    }
+    if (seg_first_host && nl <= cap_long) seg_first_host[nl] = (int32_t)ns;
+    *n_long = nl;
+    *n_seg = ns;
+    return PLX_OK;
+}
+
+int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr,
+                         const int32_t *col, int32_t seg_len, void *stream)
+{
+    PLX_REQUIRE(out != nullptr, "plan_create: NULL output");
+    *out = nullptr;
+    PLX_REQUIRE(M >= 0 && K >= 0 && nnz >= 0, "plan_create: negative size");
+    PLX_REQUIRE(M < (1ll << 31) - 1 && K < (1ll << 31) && nnz < (1ll << 31), "plan_create: sizes exceed int32 indexing");
+    PLX_REQUIRE(rowptr != nullptr, "plan_create: NULL rowptr");
+    PLX_REQUIRE(nnz == 0 || col != nullptr, "plan_create: NULL col");
+    if (seg_len <= 0) seg_len = 1024;
+    hipStream_t st = plx::as_stream(stream);
+
+    std::vector<int32_t> rp((size_t)M + 1);
+    PLX_HIP_CHECK(hipMemcpyAsync(rp.data(), rowptr, sizeof(int32_t) * (size_t)(M + 1), hipMemcpyDeviceToHost, st));
+    PLX_HIP_CHECK(hipStreamSynchronize(st));
+    PLX_REQUIRE(rp[0] == 0 && rp[(size_t)M] == nnz, "plan_create: rowptr[0]=%d rowptr[M]=%d but nnz=%lld", rp[0],
+                rp[(size_t)M], (long long)nnz);
+
+    int64_t nl = 0, ns = 0;
+    int rc = plx_spmm_segments_host(M, rp.data(), seg_len, &nl, &ns, nullptr, nullptr, 0, nullptr, nullptr, 0);
+    if (rc != PLX_OK) return rc;
+
+    plx_spmm_plan *p = new (std::nothrow) plx_spmm_plan();
+    if (!p) return plx::fail(PLX_ERR_NOMEM, "plan_create: host allocation failed");
+    p->M = M;
+    p->K = K;
+    p->nnz = nnz;
+    p->rowptr = rowptr;
+    p->col = col;
+    p->seg_len = seg_len;
+    p->n_long = nl;
+    p->n_seg = ns;
+    p->tables = nullptr;
+    p->long_rows = p->seg_first = p->seg_begin = p->seg_end = nullptr;
+    if (nl > 0) {
+        const size_t total = (size_t)nl + (size_t)(nl + 1) + 2 * (size_t)ns;
+        std::vector<int32_t> host(total);
+        int32_t *lr = host.data(), *sf = lr + nl, *sb = sf + nl + 1, *se = sb + ns;
+        rc = plx_spmm_segments_host(M, rp.data(), seg_len, &nl, &ns, lr, sf, nl, sb, se, ns);
+        if (rc != PLX_OK) {
+            delete p;
+            return rc;
+        }
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&p->tables), total * sizeof(int32_t));
+        if (e != hipSuccess) {
+            delete p;
+            return plx::fail(PLX_ERR_NOMEM, "plan_create: hipMalloc of %zu bytes failed: %s", total * sizeof(int32_t),
+                             hipGetErrorString(e));
+        }
+        e = hipMemcpy(p->tables, host.data(), total * sizeof(int32_t), hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(p->tables);
+            delete p;
+            return plx::fail(PLX_ERR_HIP, "plan_create: table upload failed: %s", hipGetErrorString(e));
+        }
+        p->long_rows = p->tables;
+        p->seg_first = p->tables + nl;
+        p->seg_begin = p->seg_first + nl + 1;
+        p->seg_end = p->seg_begin + ns;
+    }
+    *out = p;
+    return PLX_OK;
+}
+
+int plx_spmm_plan_destroy(plx_spmm_plan *plan)
+{
+    if (!plan) return PLX_OK;
+    if (plan->tables) (void)hipFree(plan->tables);
+    delete plan;
+    return PLX_OK;
+}
+
+int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what)
+{
+    if (!plan) return -1;
+    switch (what) {
+        case 0: return plan->M;
+        case 1: return plan->K;
+        case 2: return plan->nnz;
+        case 3: return plan->n_long;
+        case 4: return plan->n_seg;
+        case 5: return plan->seg_len;
+        default: return -1;
+    }
+}
+
+size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)
+{
+    if (!plan || D <= 0) return 0;
+    return (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+}
+
+int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
+                     int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_impl<float>(plan, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
+                      uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_impl<uint16_t>(plan, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,187 @@
+// Row-softmax cross-entropy: loss and d(loss)/d(logits) in one pass over the logits.
+//
+// A group of LPR lanes (LPR = power of two >= min(C, 64)) owns one row, so a wavefront covers
+// 64 / LPR consecutive rows -- consecutive rows are contiguous in memory when ld == C, which keeps
+// the loads of a wavefront in one contiguous span.  The row maximum and the row sum are reduced
+// with cross-lane shuffles inside the group.  Each workgroup adds the losses of its rows in a
+// fixed order and writes one partial; a one-workgroup kernel adds the partials in order (in fp64)
+// and divides by the node count.  No atomics.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kXentMaxBlocks = 4096;
+constexpr int kMaxPerLane = 16;  // classes per lane kept in registers: C <= 64 * 16
+
+struct XentArgs {
+    const float *logits;
+    const int64_t *labels;
+    float *dlogits;
+    float *partials;
+    int64_t ld, ldd;
+    int64_t M, C, num_nodes, num_classes, row_offset;
+    float scale;  // gscale / num_nodes
+};
+
+template <int LPR, int PER>
+__global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
+{
+    constexpr int RPW = 64 / LPR;  // rows per wavefront
+    __shared__ float wsum[4];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int grp = lane / LPR;
+    const int t = lane % LPR;
+    const int64_t cv = min(p.C, p.num_classes);
+    const int64_t rows_per_block = 4 * RPW;
+    const int64_t n_groups = (p.M + rows_per_block - 1) / rows_per_block;
+
+    float loss_acc = 0.f;  // per lane; only lane t == 0 of a group adds
+    for (int64_t gb = blockIdx.x; gb < n_groups; gb += gridDim.x) {
+        const int64_t r = gb * rows_per_block + wave * RPW + grp;
+        const bool row_ok = r < p.M;
+        const float *x = p.logits + (row_ok ? r : 0) * p.ld;
+        float v[PER];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int64_t c = t + (int64_t)k * LPR;
+            v[k] = (row_ok && c < cv) ? x[c] : -INFINITY;
+            mx = fmaxf(mx, v[k]);
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        float den = 0.f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            v[k] = (v[k] == -INFINITY) ? 0.f : expf(v[k] - mx);
+            den += v[k];
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) den += __shfl_xor(den, o, 64);
+
+        const int64_t y = row_ok ? p.labels[r] : -1;
+        const bool invalid_node = (p.row_offset + r >= p.num_nodes) || (y < 0);
+        const bool label_ok = (y >= 0) && (y < p.C);
+        const float inv = invalid_node ? 0.f : 1.f / den;
+        float py = 0.f;  // probability of the labelled class, held by the lane that owns it
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int64_t c = t + (int64_t)k * LPR;
+            const float prob = v[k] * inv;
+            const bool hit = label_ok && c == y;
+            if (hit) py = prob;
+            if (row_ok && c < p.C && p.dlogits != nullptr) p.dlogits[r * p.ldd + c] = (prob - (hit ? 1.f : 0.f)) * p.scale;
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) py += __shfl_xor(py, o, 64);  // one lane holds it, the rest 0
+        if (t == 0 && row_ok && label_ok) loss_acc += -logf(fmaxf(py, 1e-9f));
+    }
+    // fixed-order sum over the lanes of the wavefront, then over the four wavefronts
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) loss_acc += __shfl_xor(loss_acc, o, 64);
+    if (lane == 0) wsum[wave] = loss_acc;
+    __syncthreads();
+    if (threadIdx.x == 0) p.partials[blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+}
+
+__global__ void __launch_bounds__(256) xent_finish_kernel(const float *__restrict__ partials, int n, double inv_nodes,
+                                                          float *__restrict__ loss)
+{
+    __shared__ double part[256];
+    double s = 0.0;
+    for (int i = threadIdx.x; i < n; i += 256) s += (double)partials[i];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss = (float)(part[0] * inv_nodes);
+}
+
+template <int LPR>
+int launch_xent(const XentArgs &a, int per, unsigned blocks, hipStream_t st)
+{
+    switch (per) {
+        case 1: softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a); return 0;
+        case 2: softmax_xent_kernel<LPR, 2><<<blocks, 256, 0, st>>>(a); return 0;
+        case 4: softmax_xent_kernel<LPR, 4><<<blocks, 256, 0, st>>>(a); return 0;
+        case 8: softmax_xent_kernel<LPR, 8><<<blocks, 256, 0, st>>>(a); return 0;
+        case 16: softmax_xent_kernel<LPR, 16><<<blocks, 256, 0, st>>>(a); return 0;
+        default: return -1;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t plx_softmax_xent_workspace_bytes(int64_t M, int64_t C)
+{
+    (void)M;
+    (void)C;
+    return (size_t)kXentMaxBlocks * sizeof(float);
+}
+
+int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
+                         int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
+                         float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && C >= 1, "softmax_xent: bad shape M=%lld C=%lld", (long long)M, (long long)C);
+    PLX_REQUIRE(C <= 64 * kMaxPerLane, "softmax_xent: at most %d classes are supported, got %lld", 64 * kMaxPerLane,
+                (long long)C);
+    PLX_REQUIRE(num_nodes >= 1 && num_classes >= 1, "softmax_xent: num_nodes and num_classes must be positive");
+    PLX_REQUIRE(loss != nullptr, "softmax_xent: NULL loss");
+    PLX_REQUIRE(M == 0 || (logits != nullptr && labels != nullptr), "softmax_xent: NULL input");
+    PLX_REQUIRE(ld >= C && (dlogits == nullptr || ldd >= C), "softmax_xent: leading dimension smaller than C");
+    if (workspace == nullptr || workspace_bytes < plx_softmax_xent_workspace_bytes(M, C))
+        return plx::fail(PLX_ERR_WORKSPACE, "softmax_xent: workspace of %zu bytes needed, %zu given",
+                         plx_softmax_xent_workspace_bytes(M, C), workspace_bytes);
+    hipStream_t st = plx::as_stream(stream);
+
+    int lpr = 1;
+    while (lpr < 64 && lpr < C) lpr <<= 1;
+    int per = 1;
+    while ((int64_t)lpr * per < C) per <<= 1;
+
+    XentArgs a;
+    a.logits = logits;
+    a.labels = labels;
+    a.dlogits = dlogits;
+    a.partials = static_cast<float *>(workspace);
+    a.ld = ld;
+    a.ldd = ldd;
+    a.M = M;
+    a.C = C;
+    a.num_nodes = num_nodes;
+    a.num_classes = num_classes;
+    a.row_offset = row_offset;
+    a.scale = gscale / (float)num_nodes;
+
+    const int64_t rows_per_block = 4 * (64 / lpr);
+    const unsigned blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, rows_per_block), kXentMaxBlocks));
+    int rc = -1;
+    switch (lpr) {
+        case 1: rc = launch_xent<1>(a, per, blocks, st); break;
+        case 2: rc = launch_xent<2>(a, per, blocks, st); break;
+        case 4: rc = launch_xent<4>(a, per, blocks, st); break;
+        case 8: rc = launch_xent<8>(a, per, blocks, st); break;
+        case 16: rc = launch_xent<16>(a, per, blocks, st); break;
+        case 32: rc = launch_xent<32>(a, per, blocks, st); break;
+        default: rc = launch_xent<64>(a, per, blocks, st); break;
+    }
+    if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "softmax_xent: no kernel for C=%lld", (long long)C);
+    PLX_LAUNCH_CHECK("softmax_xent_kernel");
+    xent_finish_kernel<<<1, 256, 0, st>>>(a.partials, (int)blocks, 1.0 / (double)num_nodes, loss);
+    PLX_LAUNCH_CHECK("xent_finish_kernel");
+    return PLX_OK;
+}
+
+}  // extern "C"

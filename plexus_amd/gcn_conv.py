@@ -1,0 +1,158 @@
+"""GCN layer: counterpart of plexus/gcn_conv.py at one rank, on hand-written gfx950 kernels.
+
+Forward  (plexus/gcn_conv.py:137-219):  AGG = A.H ; OUT = AGG.W
+Backward (plexus/gcn_conv.py:222-296):  GRAD_W = AGG^T.G ; GRAD_AGG = G.W^T ; GRAD_H = A^T.GRAD_AGG
+
+Every collective of the reference is the identity at one rank and is not issued.  The aggregation is
+always done first, as in the reference.  Optionally the ReLU that the reference's model applies after
+the layer (examples/train.py:77-78) is fused: forward into the epilogue of the OUT product, backward as
+a mask applied while GRAD_OUT is read.
+"""
+import math
+
+import torch
+from torch.nn import Parameter
+
+from . import ops
+from . import plexus as plx
+from .utils.general import pad_dimension
+from .utils.timers import get_timers
+
+
+def chunk_bounds(num_rows, max_rows_per_chunk=1000000):
+    """Row ranges of the blocked aggregation (plexus/gcn_conv.py:77-91)."""
+    num_chunks = (num_rows + max_rows_per_chunk - 1) // max_rows_per_chunk
+    rows_per_chunk = num_rows // num_chunks
+    return [
+        (i * rows_per_chunk, num_rows if i == num_chunks - 1 else (i + 1) * rows_per_chunk)
+        for i in range(num_chunks)
+    ]
+
+
+class GCNConvFunction(torch.autograd.Function):
+    """Forward and backward of one GCN layer.
+
+    Takes the reference's twelve positional inputs (plexus/gcn_conv.py:137-151); the three process
+    groups and the two gather flags are accepted and unused at one rank.  ``fuse_relu`` is an addition.
+    """
+
+    @staticmethod
+    def forward(
+        ctx,
+        x,
+        edge_index,
+        edge_index_t,
+        weight,
+        local_features_shape,
+        local_weight_shape,
+        all_gather_group=None,
+        aggregation_all_reduce_group=None,
+        combination_all_reduce_group=None,
+        gather_features=False,
+        gather_weights=False,
+        layer_num=0,
+        fuse_relu=False,
+    ):
+        timers = get_timers()
+        timers.start("gcn conv fwd")
+        A = ops.as_csr(edge_index)
+        At = ops.as_csr(edge_index_t)
+
+        # layer-0 features arrive flat (plexus/gcn_conv.py:176-180)
+        H = x.detach().reshape(local_features_shape)
+
+        timers.start("AGG = A * H")
+        AGG = ops.spmm(A, H)
+        timers.stop("AGG = A * H")
+
+        W = weight.detach().reshape(local_weight_shape)
+        timers.start("OUT = AGG * W")
+        OUT = ops.gemm_nn(AGG, W, relu=fuse_relu)
+        timers.stop("OUT = AGG * W")
+
+        # the reference saves AGG, weight and the transposed adjacency (plexus/gcn_conv.py:194)
+        ctx.save_for_backward(AGG, weight, OUT if fuse_relu else None)
+        ctx.adj_t = At
+        ctx.local_weight_shape = tuple(local_weight_shape)
+        ctx.x_shape = x.shape
+        ctx.layer_num = layer_num
+        ctx.fuse_relu = fuse_relu
+        timers.stop("gcn conv fwd")
+        return OUT
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        timers = get_timers()
+        timers.start("gcn conv bwd")
+        agg, weight, out = ctx.saved_tensors
+        W = weight.detach().reshape(ctx.local_weight_shape)
+        mask = out if ctx.fuse_relu else None
+        grad_output = grad_output.contiguous()
+
+        grad_weight = None
+        if ctx.needs_input_grad[3]:
+            timers.start("GRAD_W = AGG.T * GRAD_OUT")
+            grad_weight = ops.gemm_tn(agg, grad_output, mask=mask).reshape(weight.shape)
+            timers.stop("GRAD_W = AGG.T * GRAD_OUT")
+
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            timers.start("GRAD_AGG = GRAD_OUT * W.T")
+            grad_agg = ops.gemm_nt(grad_output, W, mask=mask)
+            timers.stop("GRAD_AGG = GRAD_OUT * W.T")
+
+            timers.start("GRAD_H = A.T * GRAD_AGG")
+            grad_x = ops.spmm(ctx.adj_t, grad_agg)
+            timers.stop("GRAD_H = A.T * GRAD_AGG")
+            grad_x = grad_x.reshape(ctx.x_shape)  # flat again for layer 0 (plexus/gcn_conv.py:271)
+
+        timers.stop("gcn conv bwd")
+        return (grad_x, None, None, grad_weight) + (None,) * 9
+
+
+class GCNConv(torch.nn.Module):
+    """Drop-in for plexus.gcn_conv.GCNConv (plexus/gcn_conv.py:299-411) on one GPU.
+
+    ``weight`` is a flat fp32 Parameter of ``in_channels * out_channels`` elements holding the
+    row-major (in, out) matrix, as the reference stores it.  It is drawn with
+    ``kaiming_uniform_(a=sqrt(5))`` on an (in, out) tensor (plexus/gcn_conv.py:332-333) -- on the host
+    generator, so that a seed reproduces the same weights on any device -- or taken from ``weight``.
+    """
+
+    def __init__(self, in_channels, out_channels, layer_num, weight=None, fuse_relu=False, device=None, **kwargs):
+        super().__init__()
+        self.layer_num = layer_num
+        self.gather_features = layer_num == 0
+        self.gather_weights = True
+        # group sizes are all 1: padding is the identity (plexus/utils/general.py:20-23)
+        self.in_channels = pad_dimension(in_channels, 1, 1)
+        self.out_channels = pad_dimension(out_channels, 1)
+        self.local_in_channels = self.in_channels
+        self.local_out_channels = self.out_channels
+        self.fuse_relu = fuse_relu
+        if device is None:
+            device = "cuda" if torch.cuda.is_available() else "cpu"
+        if weight is None:
+            full_weight = torch.empty(in_channels, out_channels)
+            torch.nn.init.kaiming_uniform_(full_weight, a=math.sqrt(5))
+        else:
+            full_weight = torch.as_tensor(weight, dtype=torch.float32).reshape(in_channels, out_channels)
+        self.weight = Parameter(full_weight.reshape(-1).clone().to(device), requires_grad=True)
+
+    def forward(self, x, edge_index_shards):
+        edge_index, edge_index_t = edge_index_shards[self.layer_num % len(edge_index_shards)]
+        return GCNConvFunction.apply(
+            x,
+            edge_index,
+            edge_index_t,
+            self.weight,
+            (edge_index.shape[1], self.local_in_channels),
+            (self.local_in_channels, self.local_out_channels),
+            None,
+            None,
+            None,
+            self.gather_features,
+            self.gather_weights,
+            self.layer_num,
+            self.fuse_relu,
+        )

@@ -1,0 +1,291 @@
+"""Tensor-level front end of the C ABI: argument checks, output allocation, stream plumbing.
+
+PyTorch is used for device memory and streams only; every computation below is a call into
+libplexus_hip.so on the current HIP stream.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import PLX_GEMM_RELU, check
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise _lib.PlexusHipError(
+                "plexus_amd runs on the GPU only: got a tensor on %s (there is no CPU path)" % t.device
+            )
+
+
+def _rowmajor(t: torch.Tensor) -> torch.Tensor:
+    """A 2-D tensor whose rows are contiguous (any row pitch); copies only if it has to."""
+    if t.dim() != 2:
+        raise ValueError("expected a 2-D tensor, got shape %s" % (tuple(t.shape),))
+    if t.stride(1) != 1 and t.shape[1] > 1:
+        return t.contiguous()
+    if t.shape[1] == 1 and t.stride(0) < 1:
+        return t.contiguous()
+    if t.shape[0] > 1 and t.stride(0) < t.shape[1]:
+        return t.contiguous()
+    return t
+
+
+def _ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+class CsrMatrix:
+    """A CSR matrix prepared for the SpMM kernel: int32 indices, fp32 values and the row plan.
+
+    Built from a torch sparse-CSR tensor (``from_torch``) or from raw arrays.  The plan (row binning
+    and the split of long rows into segments) is computed once; the int32 arrays are owned here and
+    outlive it.
+    """
+
+    def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, val: torch.Tensor, shape, seg_len: int = 0):
+        _need_gpu(rowptr, col, val)
+        m, k = int(shape[0]), int(shape[1])
+        nnz = int(col.numel())
+        if rowptr.numel() != m + 1:
+            raise ValueError("rowptr has %d entries for %d rows" % (rowptr.numel(), m))
+        if val.numel() != nnz:
+            raise ValueError("col and val differ in length")
+        lib = _lib.load()
+        if rowptr.dtype == torch.int64 or col.dtype == torch.int64:
+            if nnz >= 2**31 or max(m, k) >= 2**31 - 1:
+                raise ValueError("matrix too large for int32 indexing")
+            rp64 = rowptr.to(torch.int64).contiguous()
+            ci64 = col.to(torch.int64).contiguous()
+            rp32 = torch.empty(m + 1, dtype=torch.int32, device=val.device)
+            ci32 = torch.empty(nnz, dtype=torch.int32, device=val.device)
+            check(
+                lib.plx_csr_narrow_i64(m, nnz, rp64.data_ptr(), ci64.data_ptr(), rp32.data_ptr(), ci32.data_ptr(), _stream()),
+                "plx_csr_narrow_i64",
+            )
+            rowptr, col = rp32, ci32
+        self.rowptr = rowptr.to(torch.int32).contiguous()
+        self.col = col.to(torch.int32).contiguous()
+        self.val = val.to(torch.float32).contiguous()
+        self.shape = (m, k)
+        self.nnz = nnz
+        self.device = val.device
+        self._plan = _lib.C.c_void_p()
+        check(
+            lib.plx_spmm_plan_create(
+                _lib.C.byref(self._plan), m, k, nnz, self.rowptr.data_ptr(), self.col.data_ptr() if nnz else None,
+                int(seg_len), _stream(),
+            ),
+            "plx_spmm_plan_create",
+        )
+        self._ws: Optional[torch.Tensor] = None
+
+    @classmethod
+    def from_torch(cls, a: torch.Tensor, seg_len: int = 0) -> "CsrMatrix":
+        if a.layout != torch.sparse_csr:
+            raise ValueError("expected a sparse CSR tensor, got layout %s" % a.layout)
+        return cls(a.crow_indices(), a.col_indices(), a.values(), a.shape, seg_len)
+
+    def __del__(self):
+        plan = getattr(self, "_plan", None)
+        if plan is not None and plan.value:
+            try:
+                _lib.load().plx_spmm_plan_destroy(plan)
+            except Exception:
+                pass
+            self._plan = None
+
+    @property
+    def n_long_rows(self) -> int:
+        return int(_lib.load().plx_spmm_plan_info(self._plan, 3))
+
+    @property
+    def n_segments(self) -> int:
+        return int(_lib.load().plx_spmm_plan_info(self._plan, 4))
+
+    def size(self, dim: int) -> int:
+        return self.shape[dim]
+
+    def _workspace(self, d: int):
+        need = int(_lib.load().plx_spmm_workspace_bytes(self._plan, d))
+        if need == 0:
+            return None, 0
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self._ws, need
+
+    def to_torch(self) -> torch.Tensor:
+        return torch.sparse_csr_tensor(
+            self.rowptr.to(torch.int64), self.col.to(torch.int64), self.val, size=self.shape, device=self.device
+        )
+
+
+def as_csr(a, seg_len: int = 0) -> CsrMatrix:
+    """CsrMatrix of ``a``; a torch CSR tensor is converted once and the result is cached on it."""
+    if isinstance(a, CsrMatrix):
+        return a
+    cached = getattr(a, "_plexus_amd_csr", None)
+    if cached is None:
+        cached = CsrMatrix.from_torch(a, seg_len)
+        try:
+            a._plexus_amd_csr = cached
+        except Exception:
+            pass
+    return cached
+
+
+def spmm(a, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Y = A.H (fp32 or bf16 H; fp32 accumulation)."""
+    a = as_csr(a)
+    _need_gpu(h)
+    h = _rowmajor(h)
+    m, k = a.shape
+    if h.shape[0] != k:
+        raise ValueError("spmm: A is %dx%d but H has %d rows" % (m, k, h.shape[0]))
+    d = h.shape[1]
+    if out is None:
+        out = torch.empty((m, d), dtype=h.dtype, device=h.device)
+    ws, ws_bytes = a._workspace(d)
+    lib = _lib.load()
+    fn = {torch.float32: lib.plx_spmm_csr_f32, torch.bfloat16: lib.plx_spmm_csr_bf16}.get(h.dtype)
+    if fn is None:
+        raise TypeError("spmm: unsupported dtype %s" % h.dtype)
+    if out.dtype != h.dtype:
+        raise TypeError("spmm: out dtype differs from H")
+    check(
+        fn(a._plan, a.val.data_ptr(), h.data_ptr(), _ld(h), d, out.data_ptr(), _ld(out),
+           ws.data_ptr() if ws is not None else None, ws_bytes, _stream()),
+        "plx_spmm_csr",
+    )
+    return out
+
+
+def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False) -> torch.Tensor:
+    """C = A.B, optionally max(C, 0)."""
+    _need_gpu(a, b)
+    a, b = _rowmajor(a), _rowmajor(b)
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2:
+        raise ValueError("gemm_nn: inner dimensions differ (%d vs %d)" % (k, k2))
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    check(
+        _lib.load().plx_gemm_nn_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                    PLX_GEMM_RELU if relu else 0, _stream()),
+        "plx_gemm_nn_f32",
+    )
+    return c
+
+
+def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = (A * [mask > 0]).B^T with B stored [N x K]."""
+    _need_gpu(a, b, mask)
+    a, b = _rowmajor(a), _rowmajor(b)
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise ValueError("gemm_nt: inner dimensions differ (%d vs %d)" % (k, k2))
+    if mask is not None:
+        mask = _rowmajor(mask)
+        if mask.shape != a.shape:
+            raise ValueError("gemm_nt: mask shape differs from A")
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    check(
+        _lib.load().plx_gemm_nt_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                    mask.data_ptr() if mask is not None else None,
+                                    _ld(mask) if mask is not None else 0, _stream()),
+        "plx_gemm_nt_f32",
+    )
+    return c
+
+
+def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C[K x N] = A[M x K]^T.(B * [mask > 0])[M x N]."""
+    _need_gpu(a, b, mask)
+    a, b = _rowmajor(a), _rowmajor(b)
+    m, k = a.shape
+    m2, n = b.shape
+    if m != m2:
+        raise ValueError("gemm_tn: row counts differ (%d vs %d)" % (m, m2))
+    if mask is not None:
+        mask = _rowmajor(mask)
+        if mask.shape != b.shape:
+            raise ValueError("gemm_tn: mask shape differs from B")
+    lib = _lib.load()
+    c = torch.empty((k, n), dtype=torch.float32, device=a.device)
+    need = int(lib.plx_gemm_tn_workspace_bytes(m, n, k))
+    ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need else None
+    check(
+        lib.plx_gemm_tn_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                            mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                            ws.data_ptr() if ws is not None else None, need, _stream()),
+        "plx_gemm_tn_f32",
+    )
+    return c
+
+
+def relu(x: torch.Tensor) -> torch.Tensor:
+    _need_gpu(x)
+    x = _rowmajor(x)
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    check(_lib.load().plx_relu_f32(x.shape[0], x.shape[1], x.data_ptr(), _ld(x), y.data_ptr(), _ld(y), _stream()), "plx_relu_f32")
+    return y
+
+
+def relu_bwd(dy: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    _need_gpu(dy, y)
+    dy, y = _rowmajor(dy), _rowmajor(y)
+    dx = torch.empty(dy.shape, dtype=torch.float32, device=dy.device)
+    check(
+        _lib.load().plx_relu_bwd_f32(dy.shape[0], dy.shape[1], dy.data_ptr(), _ld(dy), y.data_ptr(), _ld(y),
+                                     dx.data_ptr(), _ld(dx), _stream()),
+        "plx_relu_bwd_f32",
+    )
+    return dx
+
+
+def softmax_xent(logits: torch.Tensor, labels: torch.Tensor, num_nodes: int, num_classes: int, row_offset: int = 0,
+                 gscale: float = 1.0, want_grad: bool = True):
+    """(loss[1], dlogits or None) of the masked row-softmax cross-entropy."""
+    _need_gpu(logits, labels)
+    logits = _rowmajor(logits)
+    if labels.dtype != torch.int64:
+        labels = labels.to(torch.int64)
+    labels = labels.contiguous()
+    m, c = logits.shape
+    if labels.numel() != m:
+        raise ValueError("softmax_xent: %d labels for %d rows" % (labels.numel(), m))
+    lib = _lib.load()
+    loss = torch.empty(1, dtype=torch.float32, device=logits.device)
+    dlogits = torch.empty((m, c), dtype=torch.float32, device=logits.device) if want_grad else None
+    need = int(lib.plx_softmax_xent_workspace_bytes(m, c))
+    ws = torch.empty(need, dtype=torch.uint8, device=logits.device)
+    check(
+        lib.plx_softmax_xent_f32(m, c, logits.data_ptr(), _ld(logits), labels.data_ptr(), int(num_nodes),
+                                 int(num_classes), int(row_offset), float(gscale), loss.data_ptr(),
+                                 dlogits.data_ptr() if want_grad else None, _ld(dlogits) if want_grad else c,
+                                 ws.data_ptr(), need, _stream()),
+        "plx_softmax_xent_f32",
+    )
+    return loss, dlogits
+
+
+def gcn_norm_csr(a: CsrMatrix) -> torch.Tensor:
+    """Values of D^-1/2 A D^-1/2 for a square CSR matrix that already holds its self loops."""
+    if a.shape[0] != a.shape[1]:
+        raise ValueError("gcn_norm_csr: square matrix required")
+    out = torch.empty_like(a.val)
+    dinv = torch.empty(a.shape[0], dtype=torch.float32, device=a.device)
+    check(
+        _lib.load().plx_gcn_norm_csr_f32(a.shape[0], a.rowptr.data_ptr(), a.col.data_ptr(), a.val.data_ptr(),
+                                         out.data_ptr(), dinv.data_ptr(), _stream()),
+        "plx_gcn_norm_csr_f32",
+    )
+    return out

@@ -1,0 +1,65 @@
+"""Model and epoch loop of the path: counterpart of examples/train.py:55-112,155-193.
+
+``Net`` stacks GCNConv layers with ReLU after every layer but the last, no bias.  Unlike the reference
+(which keeps the layers in a plain list, so the optimizer never sees the weights) the layers are
+registered, and the optimizer updates the weights and the input features as the reference's serial
+validator does (benchmarking/pyg_serial.py:100-104).
+"""
+import torch
+import torch.nn.functional as F
+
+from .cross_entropy import parallel_cross_entropy
+from .gcn_conv import GCNConv
+from .utils.timers import get_timers
+
+
+class Net(torch.nn.Module):
+    def __init__(self, num_gcn_layers, input_size, hidden_size, output_size, weights=None, fuse_relu=True):
+        super().__init__()
+        self.num_gcn_layers = num_gcn_layers
+        self.fuse_relu = fuse_relu
+        dims = [input_size] + [hidden_size] * (num_gcn_layers - 1) + [output_size]
+        self.layers = torch.nn.ModuleList()
+        for i in range(num_gcn_layers):
+            last = i == num_gcn_layers - 1
+            self.layers.append(
+                GCNConv(dims[i], dims[i + 1], i, weight=None if weights is None else weights[i],
+                        fuse_relu=fuse_relu and not last)
+            )
+
+    def forward(self, x, edge_index_shards):
+        for i in range(self.num_gcn_layers):
+            x = self.layers[i](x, edge_index_shards)
+            if i != self.num_gcn_layers - 1 and not self.fuse_relu:
+                x = F.relu(x)
+        return x
+
+
+def train(model, optimizer, features_local, adj_shards, labels, num_nodes, num_classes):
+    """One epoch: examples/train.py:83-112."""
+    model.train()
+    optimizer.zero_grad()
+    output = model(features_local, adj_shards)
+    loss = parallel_cross_entropy(output, labels, model.num_gcn_layers, num_nodes, num_classes)
+    loss.backward()
+    optimizer.step()
+    return loss
+
+
+def make_optimizer(model, features, lr=3e-3, weight_decay=0.0):
+    """AdamW over the weights and the input features (examples/train.py:155-159)."""
+    return torch.optim.AdamW(list(model.parameters()) + [features], lr=lr, weight_decay=weight_decay)
+
+
+def run_epochs(model, optimizer, features, adj_shards, labels, num_nodes, num_classes, num_epochs, log=None):
+    """Epoch loop with the reference's per-epoch timer and log line (examples/train.py:164-193)."""
+    losses = []
+    timers = get_timers()
+    for i in range(num_epochs):
+        timers.start("epoch " + str(i))
+        loss = train(model, optimizer, features, adj_shards, labels, num_nodes, num_classes)
+        timers.stop("epoch " + str(i))
+        losses.append(float(loss))
+        if log is not None:
+            log("Epoch: {:03d}, Train Loss: {:.4f}".format(i, losses[-1]))
+    return losses

@@ -1,0 +1,359 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI, on the real GPU.
+
+fp32 bar: max|x - ref| / max|ref| <= 1e-5 per output tensor; bf16 storage: <= 2e-2.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import BF16_TOL, FP32_TOL, rel_err
+from oracle import oracle_c
+from oracle import plexus_oracle as po
+from plexus_amd import ops
+from plexus_amd.utils import synthetic as S
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def graph_small(kind="uniform", n=500, pairs=4000, seed=0, **kw):
+    return S.build_graph(n, kind, 0, seed=seed, device="cpu", exact_pairs=pairs, **kw)
+
+
+def to_dev(g, transpose=False, seg_len=0):
+    if transpose:
+        return ops.CsrMatrix(g.rowptr_t.to(DEV), g.col_t.to(DEV), g.val_t.to(DEV), (g.shape[1], g.shape[0]), seg_len)
+    return ops.CsrMatrix(g.rowptr.to(DEV), g.col.to(DEV), g.val.to(DEV), g.shape, seg_len)
+
+
+def oracle_spmm64(g, h, transpose=False):
+    if transpose:
+        return oracle_c.csr_spmm(g.rowptr_t.numpy(), g.col_t.numpy(), g.val_t.numpy(), h.numpy())
+    return oracle_c.csr_spmm(g.rowptr.numpy(), g.col.numpy(), g.val.numpy(), h.numpy())
+
+
+@pytest.mark.parametrize("d", [1, 2, 3, 4, 7, 16, 47, 64, 100, 128, 130, 256, 602, 1433, 2050])
+def test_spmm_widths(d):
+    say("spmm width D=%d" % d)
+    g = graph_small(n=700, pairs=6000, seed=d)
+    h = torch.randn(700, d, generator=torch.Generator().manual_seed(d))
+    a = to_dev(g)
+    y = ops.spmm(a, h.to(DEV)).cpu()
+    ref_t = po.spmm(g.torch_csr(), h)  # the reference's operator on the host
+    ref64 = oracle_spmm64(g, h)
+    assert rel_err(y, ref64) <= FP32_TOL
+    assert rel_err(y, ref_t) <= FP32_TOL
+
+
+@pytest.mark.parametrize("seg_len", [4, 64, 1024])
+@pytest.mark.parametrize("d", [8, 128, 602])
+def test_spmm_power_law_with_split_rows(seg_len, d):
+    say("spmm chung-lu seg_len=%d D=%d" % (seg_len, d))
+    g = S.build_graph(3000, "chunglu", 40000, seed=1, device="cpu", gamma=2.1)
+    assert g.degree_stats()["max_row_nnz"] > 1024
+    h = torch.randn(3000, d, generator=torch.Generator().manual_seed(2))
+    for transpose in (False, True):
+        a = to_dev(g, transpose, seg_len)
+        assert a.n_long_rows > 0 and a.n_segments >= 2 * a.n_long_rows
+        y = ops.spmm(a, h.to(DEV)).cpu()
+        assert rel_err(y, oracle_spmm64(g, h, transpose)) <= FP32_TOL
+
+
+def test_spmm_edge_cases():
+    say("spmm edge cases")
+    # empty matrix rows, a matrix with no entries, a single hub row, rectangular block, padded ld
+    m, k = 300, 200
+    rowptr = torch.zeros(m + 1, dtype=torch.int64)
+    col = torch.zeros(0, dtype=torch.int64)
+    val = torch.zeros(0)
+    a = ops.CsrMatrix(rowptr.to(DEV), col.to(DEV), val.to(DEV), (m, k))
+    y = ops.spmm(a, torch.randn(k, 20, device=DEV))
+    assert y.shape == (m, 20) and (y == 0).all()
+    # hub: row 5 holds every column twice over the seg_len, all other rows empty
+    gen = torch.Generator().manual_seed(0)
+    counts = torch.zeros(m, dtype=torch.int64)
+    counts[5] = k
+    counts[299] = 3
+    rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(counts, 0)])
+    col = torch.cat([torch.arange(k), torch.tensor([0, 7, 199])])
+    val = torch.rand(k + 3, generator=gen)
+    h = torch.randn(k, 36, generator=gen)
+    a = ops.CsrMatrix(rowptr.to(DEV), col.to(DEV), val.to(DEV), (m, k), seg_len=16)
+    y = ops.spmm(a, h.to(DEV)).cpu()
+    ref = oracle_c.csr_spmm(rowptr.numpy(), col.numpy(), val.numpy(), h.numpy())
+    assert rel_err(y, ref) <= FP32_TOL
+    assert (y[:5] == 0).all() and (y[6:299] == 0).all()
+    # H and Y with a leading dimension larger than D (a column slab of a wider matrix)
+    wide = torch.randn(k, 64, generator=gen)
+    out_wide = torch.full((m, 80), 7.0, device=DEV)
+    hd = wide.to(DEV)[:, 8:44]
+    ops.spmm(a, hd, out=out_wide[:, 4:40])
+    ref = oracle_c.csr_spmm(rowptr.numpy(), col.numpy(), val.numpy(), wide[:, 8:44].contiguous().numpy())
+    assert rel_err(out_wide[:, 4:40].cpu(), ref) <= FP32_TOL
+    assert (out_wide[:, :4] == 7).all() and (out_wide[:, 40:] == 7).all()
+    # zero rows
+    a0 = ops.CsrMatrix(torch.zeros(1, dtype=torch.int64, device=DEV), col[:0].to(DEV), val[:0].to(DEV), (0, k))
+    assert ops.spmm(a0, h.to(DEV)).shape == (0, 36)
+
+
+def test_spmm_int64_torch_csr_and_chunked_equivalence():
+    say("spmm from torch CSR tensor; chunked == unchunked")
+    g = graph_small(n=900, pairs=9000, seed=3)
+    a_t = g.torch_csr().to(DEV)
+    h = torch.randn(900, 32, generator=torch.Generator().manual_seed(1))
+    y = ops.spmm(a_t, h.to(DEV)).cpu()
+    assert getattr(a_t, "_plexus_amd_csr", None) is not None  # converted once, cached
+    assert rel_err(y, po.spmm(g.torch_csr(), h)) <= FP32_TOL
+    # row-chunked aggregation of the reference (gcn_conv.py:67-128) gives the same rows
+    ref_chunked = po.chunked_spmm(g.torch_csr(), h, max_rows_per_chunk=250)
+    assert rel_err(y, ref_chunked) <= FP32_TOL
+
+
+def test_spmm_bf16():
+    say("spmm bf16 storage")
+    g = S.build_graph(2000, "chunglu", 30000, seed=4, device="cpu")
+    for d in (256, 64, 100, 6):
+        h = torch.randn(2000, d, generator=torch.Generator().manual_seed(d)).to(torch.bfloat16)
+        a = to_dev(g, seg_len=128)
+        y = ops.spmm(a, h.to(DEV))
+        assert y.dtype == torch.bfloat16
+        ref = oracle_spmm64(g, h.float())  # fp32 math on bf16-rounded inputs
+        assert rel_err(y.float().cpu(), ref) <= BF16_TOL
+        # accumulation is fp32: the only error is the final rounding, 2^-9 relative per element
+        assert rel_err(y.float().cpu(), ref) <= 2.0 ** -8
+
+
+GEMM_SHAPES = [(1, 1, 1), (5, 3, 2), (127, 16, 33), (128, 32, 32), (300, 47, 128), (1000, 128, 100), (513, 128, 128),
+               (260, 7, 16), (200, 16, 1433), (150, 256, 256), (64, 130, 70)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_gemm_nn(m, n, k):
+    say("gemm_nn %dx%dx%d" % (m, n, k))
+    gen = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=gen)
+    b = torch.randn(k, n, generator=gen)
+    c = ops.gemm_nn(a.to(DEV), b.to(DEV)).cpu()
+    ref = oracle_c.gemm(a.numpy(), b.numpy())
+    assert rel_err(c, ref) <= FP32_TOL
+    assert rel_err(c, torch.mm(a, b)) <= FP32_TOL  # the reference's operator
+    cr = ops.gemm_nn(a.to(DEV), b.to(DEV), relu=True).cpu()
+    assert rel_err(cr, np.maximum(ref, 0)) <= FP32_TOL and (cr >= 0).all()
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_gemm_nt_and_mask(m, n, k):
+    say("gemm_nt %dx%dx%d" % (m, n, k))
+    gen = torch.Generator().manual_seed(m * 3 + n + k)
+    g = torch.randn(m, k, generator=gen)
+    w = torch.randn(n, k, generator=gen)
+    c = ops.gemm_nt(g.to(DEV), w.to(DEV)).cpu()
+    assert rel_err(c, oracle_c.gemm(g.numpy(), w.numpy(), tb=True)) <= FP32_TOL
+    assert rel_err(c, torch.mm(g, torch.t(w))) <= FP32_TOL
+    act = torch.relu(torch.randn(m, k, generator=gen))
+    cm = ops.gemm_nt(g.to(DEV), w.to(DEV), mask=act.to(DEV)).cpu()
+    ref = oracle_c.gemm((g * (act > 0)).numpy(), w.numpy(), tb=True)
+    assert rel_err(cm, ref) <= FP32_TOL
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(70000, 128, 100), (40000, 47, 128)])
+def test_gemm_tn_and_mask(m, n, k):
+    say("gemm_tn %dx%dx%d" % (m, n, k))
+    gen = torch.Generator().manual_seed(m * 5 + n + k)
+    a = torch.randn(m, k, generator=gen)
+    g = torch.randn(m, n, generator=gen)
+    c = ops.gemm_tn(a.to(DEV), g.to(DEV)).cpu()
+    assert c.shape == (k, n)
+    ref = oracle_c.gemm(a.numpy(), g.numpy(), ta=True)
+    assert rel_err(c, ref) <= FP32_TOL
+    act = torch.relu(torch.randn(m, n, generator=gen))
+    cm = ops.gemm_tn(a.to(DEV), g.to(DEV), mask=act.to(DEV)).cpu()
+    assert rel_err(cm, oracle_c.gemm(a.numpy(), (g * (act > 0)).numpy(), ta=True)) <= FP32_TOL
+    # run-to-run bit reproducibility (no atomics, fixed order)
+    assert torch.equal(c, ops.gemm_tn(a.to(DEV), g.to(DEV)).cpu())
+
+
+def test_gemm_strided_views_and_tuned_matmul():
+    say("gemm with leading dimensions; tuned_matmul routing")
+    from plexus_amd.utils.matmul_tuning import tuned_matmul
+
+    gen = torch.Generator().manual_seed(0)
+    big = torch.randn(300, 90, generator=gen)
+    a = big.to(DEV)[:, 10:75]  # ld 90, width 65, unaligned start
+    b = torch.randn(65, 33, generator=gen)
+    assert rel_err(ops.gemm_nn(a, b.to(DEV)).cpu(), big[:, 10:75] @ b) <= FP32_TOL
+    agg = torch.randn(400, 24, generator=gen)
+    go = torch.randn(400, 12, generator=gen)
+    w = torch.randn(24, 12, generator=gen)
+    assert rel_err(tuned_matmul(torch.t(agg.to(DEV)), go.to(DEV), "AGG.T * GRAD_OUT 0").cpu(), agg.t() @ go) <= FP32_TOL
+    assert rel_err(tuned_matmul(go.to(DEV), torch.t(w.to(DEV)), "GRAD_OUT * W.T 0").cpu(), go @ w.t()) <= FP32_TOL
+    assert rel_err(tuned_matmul(agg.to(DEV), w.to(DEV), "AGG * W 0").cpu(), agg @ w) <= FP32_TOL
+
+
+def test_relu_kernels():
+    say("relu fwd/bwd")
+    gen = torch.Generator().manual_seed(0)
+    for shape in [(33, 7), (128, 128), (5, 1)]:
+        x = torch.randn(*shape, generator=gen)
+        dy = torch.randn(*shape, generator=gen)
+        y = ops.relu(x.to(DEV))
+        assert torch.equal(y.cpu(), torch.relu(x))
+        dx = ops.relu_bwd(dy.to(DEV), y)
+        assert torch.equal(dx.cpu(), dy * (x > 0))
+
+
+@pytest.mark.parametrize("m,c", [(1, 1), (10, 7), (1000, 47), (333, 64), (257, 100), (50, 1000), (4100, 16)])
+def test_softmax_xent(m, c):
+    say("softmax_xent %dx%d" % (m, c))
+    gen = torch.Generator().manual_seed(m + c)
+    logits = torch.randn(m, c, generator=gen) * 3
+    y = torch.randint(0, c, (m,), generator=gen)
+    loss, dl = ops.softmax_xent(logits.to(DEV), y.to(DEV), m, c)
+    rl, rs, ro = po.cross_entropy_forward(logits, y, m, c)  # the reference's operator chain on the host
+    rg = po.cross_entropy_backward(rs, ro.float(), m)
+    closs, cgrad = oracle_c.softmax_xent(logits.numpy(), y.numpy(), m, c)
+    assert abs(loss.item() - closs) <= FP32_TOL * abs(closs)
+    assert abs(loss.item() - rl.item()) <= FP32_TOL * abs(closs)
+    assert rel_err(dl.cpu(), cgrad) <= FP32_TOL
+    assert rel_err(dl.cpu(), rg) <= FP32_TOL
+    # library closed form: equals F.cross_entropy when every label is valid
+    assert abs(loss.item() - torch.nn.functional.cross_entropy(logits.double(), y).item()) <= FP32_TOL * abs(closs)
+
+
+def test_softmax_xent_special_cases_and_no_mutation():
+    say("softmax_xent masks, padding, gscale")
+    gen = torch.Generator().manual_seed(9)
+    m, c = 40, 12
+    logits = torch.randn(m, c, generator=gen)
+    y = torch.randint(0, 10, (m,), generator=gen)
+    y[3] = -1
+    y[7] = 11  # labelled with a padded class
+    y[9] = 50  # outside [0, C)
+    num_nodes, num_classes = 36, 10
+    ld, yd = logits.to(DEV), y.to(DEV)
+    keep_l, keep_y = ld.clone(), yd.clone()
+    loss, dl = ops.softmax_xent(ld, yd, num_nodes, num_classes, gscale=2.5)
+    assert torch.equal(ld, keep_l) and torch.equal(yd, keep_y)
+    closs, cgrad = oracle_c.softmax_xent(logits.numpy(), y.numpy(), num_nodes, num_classes, gscale=2.5)
+    assert abs(loss.item() - closs) <= FP32_TOL * abs(closs)
+    assert rel_err(dl.cpu(), cgrad) <= FP32_TOL
+    assert (dl[3] == 0).all()  # negative label: no gradient
+    assert (dl[:, 10:] == 0)[y != 11].all()  # padded classes carry no probability
+    assert (dl[36:].cpu()[torch.arange(4), y[36:]] < 0).all() and loss.item() > 4 * 20.7 / 36
+    # row offset shifts the padded-row test
+    loss2, _ = ops.softmax_xent(ld, yd, num_nodes, num_classes, row_offset=30)
+    assert loss2.item() > loss.item()
+
+
+def test_gcn_norm_kernel():
+    say("gcn_norm_csr")
+    g = S.build_graph(1500, "chunglu", 12000, seed=5, device="cpu")
+    ones = torch.ones_like(g.val)
+    a = ops.CsrMatrix(g.rowptr.to(DEV), g.col.to(DEV), ones.to(DEV), g.shape)
+    v = ops.gcn_norm_csr(a).cpu()
+    assert rel_err(v, po.gcn_norm_csr_values(g.rowptr, g.col, ones)) <= FP32_TOL
+    assert rel_err(v, oracle_c.gcn_norm_csr(g.rowptr.numpy(), g.col.numpy(), ones.numpy())) <= FP32_TOL
+    assert rel_err(v, g.val) <= FP32_TOL
+
+
+def test_layer_forward_backward_matches_oracle():
+    say("GCNConv layer fwd+bwd, fused and unfused ReLU")
+    from plexus_amd.gcn_conv import GCNConv
+
+    n, din, dout = 1200, 100, 47
+    g = S.build_graph(n, "chunglu", 15000, seed=6, device="cpu")
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n * din, generator=gen)  # flat, as layer 0 receives it
+    w = po.kaiming_uniform_weight(din, dout, gen)
+    go = torch.randn(n, dout, generator=gen)
+    out_ref, agg_ref = po.gcn_conv_forward(x, g.torch_csr(), w, (n, din), (din, dout))
+    gx_ref, gw_ref = po.gcn_conv_backward(go, agg_ref, w, g.torch_csr(True), (din, dout), flatten_grad_x=True)
+
+    shards = [(to_dev(g), to_dev(g, True))]
+    layer = GCNConv(din, dout, 0, weight=w)
+    xd = x.to(DEV).requires_grad_()
+    out = layer(xd, shards)
+    out.backward(go.to(DEV))
+    assert rel_err(out, out_ref) <= FP32_TOL
+    assert xd.grad.shape == x.shape and rel_err(xd.grad, gx_ref) <= FP32_TOL
+    assert layer.weight.grad.shape == w.shape and rel_err(layer.weight.grad, gw_ref) <= FP32_TOL
+
+    # fused ReLU: forward max(OUT, 0); backward masks GRAD_OUT by OUT > 0
+    layer2 = GCNConv(din, dout, 1, weight=w, fuse_relu=True)
+    xd2 = x.reshape(n, din).to(DEV).requires_grad_()
+    out2 = layer2(xd2, shards)
+    out2.backward(go.to(DEV))
+    gmask = go * (out_ref > 0)
+    gx2_ref, gw2_ref = po.gcn_conv_backward(gmask, agg_ref, w, g.torch_csr(True), (din, dout))
+    assert rel_err(out2, torch.relu(out_ref)) <= FP32_TOL
+    assert rel_err(xd2.grad, gx2_ref) <= FP32_TOL and rel_err(layer2.weight.grad, gw2_ref) <= FP32_TOL
+
+
+@pytest.mark.parametrize("fuse_relu", [True, False])
+def test_config1_ten_epoch_loss_curve(fuse_relu):
+    """2-layer GCN of the CPU-runnable configuration: ten AdamW epochs against the oracle's."""
+    say("config 1, 10 epochs, fuse_relu=%s" % fuse_relu)
+    from plexus_amd.train import Net, make_optimizer, run_epochs
+
+    g, x, y, dims = S.config1(device="cpu", seed=0)
+    weights = S.glorot_weights(dims, seed=0)
+    n = g.shape[0]
+    ref_losses, ref_x, ref_w = po.train_epochs(x, weights, dims, [(g.torch_csr(), g.torch_csr(True))], y, n, 7, epochs=10)
+    ref64, _, _ = po.train_epochs(x.double(), [w.double() for w in weights], dims,
+                                  [(g.torch_csr().double(), g.torch_csr(True).double())], y, n, 7, epochs=10)
+
+    model = Net(2, dims[0], dims[1], dims[2], weights=weights, fuse_relu=fuse_relu)
+    feats = x.reshape(-1).to(DEV).requires_grad_()
+    opt = make_optimizer(model, feats)
+    shards = [(g.torch_csr().to(DEV), g.torch_csr(True).to(DEV))]
+    losses = run_epochs(model, opt, feats, shards, y.to(DEV), n, 7, 10)
+    print("gpu   ", ["%.6f" % v for v in losses], flush=True)
+    print("oracle", ["%.6f" % v for v in ref_losses], flush=True)
+    for l, r, r64 in zip(losses, ref_losses, ref64):
+        assert abs(l - r64) <= FP32_TOL * abs(r64) or abs(l - r) <= FP32_TOL * abs(r)
+    assert losses[-1] < losses[0]
+    assert rel_err(feats, ref_x) <= 1e-4  # ten optimizer steps amplify rounding; the loss is the gate
+    for layer, w in zip(model.layers, ref_w):
+        assert rel_err(layer.weight, w) <= 1e-4
+
+
+def test_scaled_config3_properties_and_sampled_rows():
+    """A tenth of the 2.45 M-node power-law configuration: size-independent properties of the SpMM
+    and a comparison of sampled rows against the fp64-accumulating oracle."""
+    say("config 3 at 1/10 scale: properties")
+    g = S.config3_graph(DEV, seed=0, scale=0.1)
+    n = g.shape[0]
+    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
+    at = ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (n, n))
+    print(g.degree_stats(), "long rows", a.n_long_rows, "segments", a.n_segments, flush=True)
+    h = S.normal_features(n, 128, DEV, seed=1)
+    gm = S.normal_features(n, 128, DEV, seed=2)
+    y = ops.spmm(a, h)
+    # A.1 = row sums
+    ones = torch.ones(n, 4, device=DEV)
+    rows = torch.repeat_interleave(torch.arange(n, device=DEV), g.rowptr[1:] - g.rowptr[:-1])
+    rowsum = torch.zeros(n, dtype=torch.float64, device=DEV).index_add_(0, rows, g.val.double())
+    assert rel_err(ops.spmm(a, ones)[:, 0], rowsum) <= FP32_TOL
+    # adjoint identity <A.H, G> = <H, A^T.G>
+    lhs = (y.double() * gm.double()).sum().item()
+    rhs = (h.double() * ops.spmm(at, gm).double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), (y.double().norm() * gm.double().norm()).item() * 1e-3)
+    # linearity
+    y2 = ops.spmm(a, 2.0 * h + gm)
+    assert rel_err(y2, 2.0 * y.double() + ops.spmm(a, gm).double()) <= FP32_TOL
+    # bit reproducibility
+    assert torch.equal(y, ops.spmm(a, h))
+    # sampled rows (the longest, the shortest and random ones) against the oracle
+    deg = (g.rowptr[1:] - g.rowptr[:-1]).cpu()
+    pick = torch.cat([torch.topk(deg, 8).indices, torch.topk(-deg, 8).indices,
+                      torch.randint(0, n, (200,), generator=torch.Generator().manual_seed(0))])
+    rp, ci, va = g.rowptr.cpu(), g.col.cpu(), g.val.cpu()
+    sub_counts = deg[pick]
+    sub_rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(sub_counts, 0)])
+    idx = torch.cat([torch.arange(rp[r], rp[r + 1]) for r in pick.tolist()])
+    ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci[idx].numpy(), va[idx].numpy(), h.cpu().numpy())
+    assert rel_err(y[pick.to(DEV)].cpu(), ref) <= FP32_TOL

@@ -1,0 +1,300 @@
+"""Pins the CPU oracle (oracle/) without the reference: the reference has no tests or golden vectors
+for this path, so each oracle function is checked against something the mathematics fixes --
+dense products, scipy, brute-force loops, library closed forms, autograd, published known answers."""
+import math
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+import torch.nn.functional as F
+
+from oracle import oracle_c
+from oracle import plexus_oracle as po
+from plexus_amd.utils import synthetic as S
+
+
+def small_graph(n=97, pairs=400, seed=3, with_empty_rows=True):
+    g = torch.Generator().manual_seed(seed)
+    src = torch.randint(0, n, (pairs,), generator=g)
+    dst = torch.randint(0, n, (pairs,), generator=g)
+    if with_empty_rows:
+        keep = (src % 7 != 0)
+        src, dst = src[keep], dst[keep]
+    w = torch.rand(src.numel(), generator=g) + 0.1
+    a = torch.sparse_coo_tensor(torch.stack([src, dst]), w, (n, n)).coalesce()
+    return a.to_sparse_csr()
+
+
+def brute_spmm(crow, col, val, h):
+    m = len(crow) - 1
+    y = np.zeros((m, h.shape[1]), dtype=np.float64)
+    for r in range(m):
+        for j in range(crow[r], crow[r + 1]):
+            for d in range(h.shape[1]):
+                y[r, d] += float(val[j]) * float(h[col[j], d])
+    return y
+
+
+def test_spmm_oracle_vs_dense_scipy_bruteforce():
+    a = small_graph()
+    h = torch.randn(97, 13, generator=torch.Generator().manual_seed(1))
+    y = po.spmm(a, h)
+    dense = a.to_dense().double() @ h.double()
+    assert torch.allclose(y.double(), dense, rtol=0, atol=1e-5)
+    crow, col, val = a.crow_indices().numpy(), a.col_indices().numpy(), a.values().numpy()
+    ys = sp.csr_matrix((val.astype(np.float64), col, crow), shape=(97, 97)) @ h.double().numpy()
+    assert np.allclose(dense.numpy(), ys, atol=1e-12)
+    yb = brute_spmm(crow, col, val, h.numpy())
+    assert np.allclose(dense.numpy(), yb, atol=1e-12)
+    # the C restatement: fp64 accumulation, fp32 accumulation, and all-fp64
+    assert np.allclose(oracle_c.csr_spmm(crow, col, val, h.numpy(), acc64=True), dense.numpy(), atol=2e-6)
+    assert np.allclose(oracle_c.csr_spmm(crow, col, val, h.numpy(), acc64=False), dense.numpy(), atol=1e-5)
+    assert np.allclose(oracle_c.csr_spmm(crow, col, val.astype(np.float64), h.double().numpy()), dense.numpy(), atol=1e-12)
+
+
+def test_spmm_oracle_invariants():
+    a = small_graph(n=120, pairs=900, seed=5)
+    n = 120
+    g = torch.Generator().manual_seed(2)
+    # A.1 = row sums ; empty row -> zero row
+    ones = torch.ones(n, 3)
+    y = po.spmm(a, ones)
+    crow = a.crow_indices()
+    rowsum = torch.zeros(n).index_add_(0, torch.repeat_interleave(torch.arange(n), crow[1:] - crow[:-1]), a.values())
+    assert torch.allclose(y[:, 0], rowsum, atol=1e-5)
+    empty = (crow[1:] - crow[:-1]) == 0
+    assert empty.any() and (y[empty] == 0).all()
+    # adjoint identity <A.H, G> = <H, A^T.G> with the separately materialised transpose
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    h = torch.randn(n, 6, generator=g, dtype=torch.float64)
+    gg = torch.randn(n, 6, generator=g, dtype=torch.float64)
+    a64, a_t64 = a.double(), a_t.double()
+    lhs = (po.spmm(a64, h) * gg).sum()
+    rhs = (h * po.spmm(a_t64, gg)).sum()
+    assert abs(lhs - rhs) < 1e-9 * abs(lhs)
+    # permutation equivariance (P A Q^T)(Q H) = P (A H)
+    p, q = torch.randperm(n, generator=g), torch.randperm(n, generator=g)
+    dense = a64.to_dense()
+    paq = torch.zeros_like(dense)
+    paq[p[:, None], q[None, :]] = dense
+    qh = torch.zeros_like(h)
+    qh[q] = h
+    ref = torch.zeros_like(h)
+    ref[p] = po.spmm(a64, h)
+    assert torch.allclose(po.spmm(paq.to_sparse_csr(), qh), ref, atol=1e-12)
+
+
+def test_chunked_spmm_equals_unchunked():
+    a = small_graph(n=103, pairs=700, seed=8)
+    h = torch.randn(103, 5, generator=torch.Generator().manual_seed(4))
+    assert po.chunk_bounds(2449029) == [(0, 816343), (816343, 1632686), (1632686, 2449029)]
+    assert po.chunk_bounds(10, 4) == [(0, 3), (3, 6), (6, 10)]
+    assert torch.equal(po.chunked_spmm(a, h, max_rows_per_chunk=10), po.spmm(a, h))
+
+
+def test_gemm_c_oracle_vs_numpy():
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((37, 21)).astype(np.float32)
+    b = rng.standard_normal((21, 11)).astype(np.float32)
+    assert np.allclose(oracle_c.gemm(a, b), a.astype(np.float64) @ b.astype(np.float64), atol=1e-5)
+    g = rng.standard_normal((37, 11)).astype(np.float32)
+    assert np.allclose(oracle_c.gemm(a, g, ta=True), a.astype(np.float64).T @ g, atol=1e-5)
+    w = rng.standard_normal((21, 11)).astype(np.float32)
+    assert np.allclose(oracle_c.gemm(g, w, tb=True), g.astype(np.float64) @ w.astype(np.float64).T, atol=1e-5)
+
+
+def test_layer_backward_formulas_vs_autograd():
+    """The hand formulas of gcn_conv.py:236-266 equal autograd over the plain-operator forward."""
+    n, din, dout = 60, 9, 5
+    a = small_graph(n=n, pairs=300, seed=11).double()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(n * din, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(din * dout, generator=g, dtype=torch.float64, requires_grad=True)
+    out, agg = po.gcn_conv_forward(x, a, w, (n, din), (din, dout))
+    go = torch.randn(n, dout, generator=g, dtype=torch.float64)
+    gx_ref, gw_ref = torch.autograd.grad(out, [x, w], go)
+    gx, gw = po.gcn_conv_backward(go, agg.detach(), w.detach(), a_t, (din, dout), flatten_grad_x=True)
+    assert torch.allclose(gx, gx_ref, atol=1e-12) and gx.shape == x.shape
+    assert torch.allclose(gw, gw_ref, atol=1e-12) and gw.shape == w.shape
+    # and the forward equals the dense product
+    ref = (a.to_dense() @ x.detach().reshape(n, din)) @ w.detach().reshape(din, dout)
+    assert torch.allclose(out.detach(), ref, atol=1e-12)
+
+
+def test_cross_entropy_equals_library_mean_loss():
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(50, 11, generator=g, dtype=torch.float64)
+    y = torch.randint(0, 11, (50,), generator=g)
+    loss, softmax, onehot = po.cross_entropy_forward(logits, y, 50, 11)
+    lg = logits.clone().requires_grad_()
+    ref = F.cross_entropy(lg, y)
+    assert abs(loss - ref) < 1e-12
+    (gref,) = torch.autograd.grad(ref, lg)
+    grad = po.cross_entropy_backward(softmax, onehot.double(), 50)
+    assert torch.allclose(grad, gref, atol=1e-14)
+    assert torch.allclose(grad.sum(1), torch.zeros(50, dtype=torch.float64), atol=1e-15)
+    # inputs untouched
+    assert torch.equal(logits, lg.detach())
+    # C restatement agrees (fp32 logits)
+    l32 = logits.float()
+    closs, cgrad = oracle_c.softmax_xent(l32.numpy(), y.numpy(), 50, 11)
+    ref32 = F.cross_entropy(l32.double(), y)
+    assert abs(closs - ref32) < 1e-9
+    assert np.allclose(cgrad, po.cross_entropy_backward(*[t.double() for t in po.cross_entropy_forward(l32.double(), y, 50, 11)[1:]], 50).numpy(), atol=1e-8)
+
+
+def test_cross_entropy_special_cases():
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(8, 6, generator=g, dtype=torch.float64)
+    y = torch.tensor([0, 1, -1, 3, 5, 2, 0, 4])
+    num_nodes, num_classes = 6, 5  # rows 6,7 are padded; class 5 is padded
+    loss, softmax, onehot = po.cross_entropy_forward(logits, y, num_nodes, num_classes)
+    grad = po.cross_entropy_backward(softmax, onehot.double(), num_nodes)
+    # label < 0: zero loss, zero gradient row
+    assert (softmax[2] == 0).all() and (grad[2] == 0).all()
+    # padded class has probability 0 everywhere
+    assert (softmax[:, 5] == 0).all()
+    # rows past num_nodes: softmax zero; label 0 / 4 is valid so each adds -log(1e-9)
+    assert (softmax[6:] == 0).all()
+    # row 4 is labelled with the padded class: probability 0 -> -log(1e-9) as well
+    valid = [0, 1, 3, 5]
+    sm = torch.softmax(logits[:, :5], dim=1)
+    expect = sum(-math.log(sm[i, y[i]]) for i in valid) + 3 * (-math.log(1e-9))
+    assert abs(loss * num_nodes - expect) < 1e-10
+    assert abs(-math.log(1e-9) - 20.7233) < 1e-4
+    # valid rows: gradient rows sum to zero
+    assert torch.allclose(grad[valid].sum(1), torch.zeros(4, dtype=torch.float64), atol=1e-15)
+    closs, cgrad = oracle_c.softmax_xent(logits.float().numpy(), y.numpy(), num_nodes, num_classes)
+    l32, s32, o32 = po.cross_entropy_forward(logits.float().double(), y, num_nodes, num_classes)
+    assert abs(closs - l32) < 1e-9
+    assert np.allclose(cgrad, po.cross_entropy_backward(s32, o32.double(), num_nodes).numpy(), atol=1e-8)
+
+
+def test_gcn_norm_closed_forms():
+    # ring of n nodes, each linked to its k nearest on both sides: (2k)-regular -> every entry 1 / (2k + 1)
+    n, k = 30, 2
+    src = torch.arange(n).repeat_interleave(2 * k)
+    off = torch.tensor([-2, -1, 1, 2]).repeat(n)
+    dst = (src + off) % n
+    ei, w = po.gcn_norm(torch.stack([src, dst]), n)
+    assert ei.shape[1] == n * (2 * k + 1)
+    assert torch.allclose(w, torch.full_like(w, 1.0 / (2 * k + 1)))
+    # general symmetric graph: dense formula D^-1/2 (A + I) D^-1/2, symmetric result
+    g = S.build_graph(40, "uniform", 0, seed=1, permute=False, exact_pairs=90)
+    dense = g.torch_csr().to_dense().double()
+    adj = (dense != 0).double()
+    d = adj.sum(1)
+    ref = adj / torch.sqrt(d[:, None] * d[None, :])
+    assert torch.allclose(dense, ref, atol=1e-7)
+    assert torch.equal(dense, dense.t())
+    # CSR-values variant and the C restatement reproduce it from unit values
+    ones = torch.ones_like(g.val)
+    v = po.gcn_norm_csr_values(g.rowptr, g.col, ones)
+    assert torch.allclose(v, g.val, atol=1e-7)
+    vc = oracle_c.gcn_norm_csr(g.rowptr.numpy(), g.col.numpy(), ones.numpy())
+    assert np.allclose(vc, g.val.numpy(), atol=1e-7)
+    # PyG-style edge-list variant agrees on the same graph without its loops
+    crow = g.rowptr
+    rows = torch.repeat_interleave(torch.arange(40), crow[1:] - crow[:-1])
+    nl = rows != g.col
+    ei2, w2 = po.gcn_norm(torch.stack([rows[nl], g.col[nl]]), 40)
+    d2 = torch.zeros(40, 40, dtype=torch.float64)
+    d2[ei2[0], ei2[1]] = w2.double()
+    assert torch.allclose(d2, ref, atol=1e-7)
+
+
+def test_weight_init_bound():
+    w = po.kaiming_uniform_weight(100, 16, torch.Generator().manual_seed(0))
+    assert w.shape == (1600,)
+    assert w.abs().max() <= 1 / math.sqrt(16) and w.abs().max() > 0.24
+    assert abs(w.mean()) < 0.02
+    # same bound as torch's initialiser on an (in, out) tensor: fan_in = size(1)
+    t = torch.empty(100, 16)
+    torch.manual_seed(0)
+    torch.nn.init.kaiming_uniform_(t, a=math.sqrt(5))
+    assert t.abs().max() <= 1 / math.sqrt(16) and t.abs().max() > 0.24
+
+
+def test_philox_known_answers():
+    """Published Random123 known-answer vectors for philox4x32-10."""
+    kat = [
+        ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+        ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+        ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+         (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+    ]
+    for ctr, key, out in kat:
+        r = po.philox4x32_10(np.array([ctr], dtype=np.uint32), key)
+        assert tuple(int(v) for v in r[0]) == out
+    m = po.dropout_keep_mask(100000, seed=0, offset=3, p=0.5)
+    assert abs(m.mean() - 0.5) < 0.01
+    assert abs(po.dropout_keep_mask(100000, seed=0, offset=3, p=0.25).mean() - 0.75) < 0.01
+    assert po.dropout_keep_mask(1000, 1, 0, 0.0).all()
+
+
+def test_adamw_step_matches_torch():
+    g = torch.Generator().manual_seed(0)
+    p0 = [torch.randn(7, generator=g, dtype=torch.float64), torch.randn(3, 4, generator=g, dtype=torch.float64)]
+    params = [p.clone().requires_grad_() for p in p0]
+    opt = torch.optim.AdamW(params, lr=3e-3, weight_decay=0.0)
+    mine = [p.clone() for p in p0]
+    state = {}
+    for _ in range(4):
+        grads = [torch.randn(p.shape, generator=g, dtype=torch.float64) for p in p0]
+        for p, gr in zip(params, grads):
+            p.grad = gr.clone()
+        opt.step()
+        po.adamw_step(mine, grads, state, lr=3e-3)
+    for a, b in zip(mine, params):
+        assert torch.allclose(a, b.detach(), atol=1e-12)
+
+
+def test_epoch_loop_matches_autograd_training():
+    """OracleNet + hand backward + adamw_step equals the same model trained by torch autograd + AdamW."""
+    g, x, y, dims = S.config1()
+    n = 300
+    gs = S.build_graph(n, "uniform", 0, seed=2, permute=False, exact_pairs=1200)
+    a, a_t = gs.torch_csr().double(), gs.torch_csr(True).double()
+    dims = [12, 8, 5]
+    gen = torch.Generator().manual_seed(0)
+    x0 = torch.randn(n, dims[0], generator=gen, dtype=torch.float64)
+    labels = torch.randint(0, 5, (n,), generator=gen)
+    ws = [w.double() for w in S.glorot_weights(dims, seed=1)]
+    losses, xf, wf = po.train_epochs(x0, ws, dims, [(a, a_t)], labels, n, 5, epochs=4)
+
+    xs = x0.clone().reshape(-1).requires_grad_()
+    wt = [w.clone().requires_grad_() for w in ws]
+    opt = torch.optim.AdamW(wt + [xs], lr=3e-3, weight_decay=0.0)
+    ref_losses = []
+    for _ in range(4):
+        opt.zero_grad()
+        h = xs.reshape(n, dims[0])
+        for i, w in enumerate(wt):
+            h = torch.mm(torch.sparse.mm(a, h), w.reshape(dims[i], dims[i + 1]))
+            if i != len(wt) - 1:
+                h = F.relu(h)
+        loss = F.cross_entropy(h, labels)
+        loss.backward()
+        opt.step()
+        ref_losses.append(float(loss))
+    assert np.allclose(losses, ref_losses, atol=1e-12)
+    assert torch.allclose(xf, xs.detach(), atol=1e-12)
+    for a_, b_ in zip(wf, wt):
+        assert torch.allclose(a_, b_.detach(), atol=1e-12)
+    assert losses[-1] < losses[0]
+
+
+def test_csr_pair_construction_and_block():
+    """build_csr_pair follows the loader: mask, re-base, COO->CSR, transpose->CSR."""
+    gen = torch.Generator().manual_seed(0)
+    ei = torch.randint(0, 20, (2, 150), generator=gen)
+    ei = torch.unique(ei, dim=1)
+    w = torch.rand(ei.shape[1], generator=gen)
+    a, a_t = po.build_csr_pair(ei, w, (20, 20), row_range=(5, 15), col_range=(0, 10))
+    dense = torch.zeros(20, 20)
+    dense[ei[0], ei[1]] = w
+    assert torch.equal(a.to_dense(), dense[5:15, 0:10])
+    assert torch.equal(a_t.to_dense(), dense[5:15, 0:10].t())
+    assert po.pad_dimension(10, 4) == 12 and po.pad_dimension(12, 4) == 12 and po.pad_dimension(7, 2, 3) == 12
