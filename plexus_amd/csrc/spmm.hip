@@ -382,7 +382,7 @@ int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t l
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
     PLX_REQUIRE(D >= 0 && D < (1ll << 30), "spmm: bad feature width D=%lld", (long long)D);
     if (plan->M == 0 || D == 0) return PLX_OK;
-    PLX_REQUIRE(val && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
+    PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
     const size_t need = plx_spmm_workspace_bytes(plan, D);
