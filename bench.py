@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--spmm-only", action="store_true", help="time only the SpMM kernels")
     ap.add_argument("--spmm-iters", type=int, default=20)
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch a plain 1 GiB device copy (known size) to calibrate profiler byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives are implemented); --gpus %d is not "
@@ -89,6 +91,14 @@ def main():
     dims = [100, 128, 128, 47]
     print("# graph: %s, long rows %d, segments %d, generated in %.1f s" % (stats, a.n_long_rows, a.n_segments, gen_s),
           file=sys.stderr, flush=True)
+
+    if args.calib_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- the dominant kernel: SpMM at D = 128 (and D = 100 beside it) ----
     spmm = {}

@@ -142,6 +142,18 @@ int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, 
 int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, const float *val_in, float *val_out,
                          float *dinv, void *stream);
 
+/* ------------------------------------------------------------------------------------------
+ * AdamW step over one flat fp32 tensor, in one pass
+ *   replaces optimizer.step() of torch.optim.AdamW(lr, weight_decay) over the weights and the input
+ *   features, examples/train.py:155-159 and :110 (decoupled weight decay, bias-corrected moments,
+ *   no amsgrad):
+ *     p *= 1 - lr * weight_decay;  m += (g - m) (1 - beta1);  v = beta2 v + (1 - beta2) g^2;
+ *     p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
+ *   `step` is the 1-based count of this update.
+ * ---------------------------------------------------------------------------------------- */
+int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, float lr, float beta1,
+                  float beta2, float eps, float weight_decay, int64_t step, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libplexus_hip.so")
+# PLEXUS_HIP_LIB selects another build of the same ABI (e.g. a tuning variant)
+LIB_PATH = os.environ.get("PLEXUS_HIP_LIB") or os.path.join(_HERE, "libplexus_hip.so")
 
 _vp = C.c_void_p
 _i64 = C.c_int64
@@ -39,6 +40,7 @@ SIGNATURES = {
     "plx_softmax_xent_workspace_bytes": (_sz, [_i64, _i64]),
     "plx_softmax_xent_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "plx_gcn_norm_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "plx_adamw_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32, _f32, _i64, _vp]),
 }
 
 PLX_GEMM_RELU = 1

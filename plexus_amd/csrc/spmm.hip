@@ -302,25 +302,55 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
     }
 }
 
-// Y[row q] = sum over the segments of split row q, in segment order.
+// Y[row q] = sum over the segments of split row q.  A workgroup owns one split row and 64 of its
+// columns: 16 chains x 16 lanes, each lane a float4.  Chain c adds segments c, c + 16, ... in order;
+// the 16 chain sums are then added in chain order, so the summation order is fixed.
 template <typename TOUT>
 __global__ void __launch_bounds__(256) spmm_reduce_split_rows(const float *__restrict__ ws, int64_t ldws,
                                                               const int32_t *__restrict__ long_rows,
                                                               const int32_t *__restrict__ seg_first, int32_t D,
                                                               TOUT *__restrict__ Y, int64_t ldy)
 {
+    __shared__ float4 part[16][16];
     const int q = blockIdx.x;
-    const int d = blockIdx.y * blockDim.x + threadIdx.x;
-    if (d >= D) return;
+    const int chain = threadIdx.x >> 4;
+    const int l = threadIdx.x & 15;
+    const int d = blockIdx.y * 64 + l * 4;
     const int s0 = seg_first[q];
     const int s1 = seg_first[q + 1];
-    float s = 0.f;
-    for (int i = s0; i < s1; ++i) s += ws[(int64_t)i * ldws + d];
-    TOUT *dst = Y + (int64_t)long_rows[q] * ldy + d;
-    if constexpr (sizeof(TOUT) == 4)
-        *dst = s;
-    else
-        *dst = (uint16_t)f32_to_bf16(s);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d < D) {  // ldws is a multiple of 4, so the float4 at d stays inside the padded workspace row
+        for (int i = s0 + chain; i < s1; i += 16) {
+            const float4 t = *reinterpret_cast<const float4 *>(ws + (int64_t)i * ldws + d);
+            acc.x += t.x;
+            acc.y += t.y;
+            acc.z += t.z;
+            acc.w += t.w;
+        }
+    }
+    part[chain][l] = acc;
+    __syncthreads();
+    if (chain == 0 && d < D) {
+        float4 s = part[0][l];
+#pragma unroll
+        for (int c = 1; c < 16; ++c) {
+            s.x += part[c][l].x;
+            s.y += part[c][l].y;
+            s.z += part[c][l].z;
+            s.w += part[c][l].w;
+        }
+        const float v[4] = {s.x, s.y, s.z, s.w};
+        TOUT *dst = Y + (int64_t)long_rows[q] * ldy + d;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (d + e < D) {
+                if constexpr (sizeof(TOUT) == 4)
+                    dst[e] = v[e];
+                else
+                    dst[e] = (uint16_t)f32_to_bf16(v[e]);
+            }
+        }
+    }
 }
 
 __global__ void narrow_i64_kernel(int64_t n, const int64_t *__restrict__ src, int32_t *__restrict__ dst)
@@ -439,9 +469,8 @@ int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t l
     PLX_LAUNCH_CHECK("spmm_csr_kernel");
 
     if (plan->n_long > 0) {
-        const int bs = (int)std::min<int64_t>(256, plx::ceil_div(D, 64) * 64);
-        dim3 rgrid((unsigned)plan->n_long, (unsigned)plx::ceil_div(D, bs), 1);
-        spmm_reduce_split_rows<T><<<rgrid, bs, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)D, Y, ldy);
+        dim3 rgrid((unsigned)plan->n_long, (unsigned)plx::ceil_div(D, 64), 1);
+        spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)D, Y, ldy);
         PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
     }
     return PLX_OK;

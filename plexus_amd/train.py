@@ -10,6 +10,7 @@ import torch.nn.functional as F
 
 from .cross_entropy import parallel_cross_entropy
 from .gcn_conv import GCNConv
+from .optim import AdamW
 from .utils.timers import get_timers
 
 
@@ -46,9 +47,15 @@ def train(model, optimizer, features_local, adj_shards, labels, num_nodes, num_c
     return loss
 
 
-def make_optimizer(model, features, lr=3e-3, weight_decay=0.0):
-    """AdamW over the weights and the input features (examples/train.py:155-159)."""
-    return torch.optim.AdamW(list(model.parameters()) + [features], lr=lr, weight_decay=weight_decay)
+def make_optimizer(model, features, lr=3e-3, weight_decay=0.0, fused=True):
+    """AdamW over the weights and the input features (examples/train.py:155-159).
+
+    ``fused`` selects the one-pass kernel of this package; otherwise torch's own optimizer is used.
+    """
+    params = list(model.parameters()) + [features]
+    if fused:
+        return AdamW(params, lr=lr, weight_decay=weight_decay)
+    return torch.optim.AdamW(params, lr=lr, weight_decay=weight_decay)
 
 
 def run_epochs(model, optimizer, features, adj_shards, labels, num_nodes, num_classes, num_epochs, log=None):

@@ -357,3 +357,28 @@ def test_scaled_config3_properties_and_sampled_rows():
     idx = torch.cat([torch.arange(rp[r], rp[r + 1]) for r in pick.tolist()])
     ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci[idx].numpy(), va[idx].numpy(), h.cpu().numpy())
     assert rel_err(y[pick.to(DEV)].cpu(), ref) <= FP32_TOL
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_fused_adamw_matches_torch_and_oracle(n):
+    say("fused AdamW n=%d" % n)
+    from plexus_amd.optim import AdamW
+
+    gen = torch.Generator().manual_seed(n)
+    p0 = torch.randn(n, generator=gen)
+    grads = [torch.randn(n, generator=gen) * (10.0 ** (i - 2)) for i in range(5)]
+    for wd in (0.0, 0.01):
+        p = p0.clone().to(DEV).requires_grad_()
+        opt = AdamW([p], lr=3e-3, weight_decay=wd)
+        ref = p0.clone().double().requires_grad_()
+        ropt = torch.optim.AdamW([ref], lr=3e-3, weight_decay=wd)
+        mine = [p0.clone().double()]
+        state = {}
+        for g in grads:
+            p.grad = g.to(DEV)
+            opt.step()
+            ref.grad = g.double()
+            ropt.step()
+            po.adamw_step(mine, [g.double()], state, lr=3e-3, weight_decay=wd)
+        assert rel_err(p, ref) <= FP32_TOL
+        assert rel_err(p, mine[0]) <= FP32_TOL
