@@ -25,6 +25,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 FP32_VECTOR_TFLOPS = 157.3
+# Bytes moved between L2 and the memory side per SpMM launch at D = 128 on the full-size workload, from
+# rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain
+# 1 GiB copy: 2.000 and 1.000); the summary is profiles/spmm_csr_config3_fp32_pmc.txt.
+MEASURED_SPMM_TRAFFIC_BYTES = {(2449029, 126149029, 128): 53.9e9}
 
 
 def spmm_bytes(m, k, nnz, d, elem=4):
@@ -190,7 +194,8 @@ def main():
         "epoch_ms": epoch_ms,
         "loss_first_last": [losses[0], losses[-1]] if losses else None,
         "roofline": {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": dom["alg_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": dom["alg_GBps"] / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_SPMM_TRAFFIC_BYTES.get((n, nnz, 128)),
                      "kernel": "spmm_csr_kernel (A.H, D=128)", "alg_bytes_per_launch": dom["alg_bytes"],
                      "avg_launch_ms": dom["ms"]},
         "cpu_baseline": cpu,
