@@ -256,14 +256,18 @@ class OracleNet:
         self._saved = saved
         return h
 
-    def backward(self, grad_logits):
+    def backward(self, grad_logits, masks=None):
+        """``masks[i]`` (optional) replaces the ReLU mask ``pre_i > 0`` of layer i: a pre-activation within
+        rounding of zero may take either sign in two fp32 summation orders, and a caller comparing backward
+        passes can pin the mask to the one the other implementation used."""
         g = grad_logits
         grads_w = [None] * len(self.weights)
         n_layers = len(self.weights)
         for i in reversed(range(n_layers)):
             agg, a_t, wshape, pre = self._saved[i]
             if i != n_layers - 1:
-                g = g * (pre > 0).to(g.dtype)
+                mask = (pre > 0) if masks is None or masks[i] is None else masks[i]
+                g = g * mask.to(g.dtype)
             g, grads_w[i] = gcn_conv_backward(g, agg, self.weights[i], a_t, wshape, flatten_grad_x=(i == 0))
         return g, grads_w
 

@@ -91,6 +91,83 @@ __global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
     if (threadIdx.x == 0) p.partials[blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
 }
 
+// Narrow rows (C up to a few hundred): a workgroup stages a tile of R consecutive rows in LDS with
+// coalesced loads, one lane then owns one row (row stride C | 1, so lanes hit distinct banks), and the
+// gradient tile goes back with coalesced stores.  Every lane is busy whatever C is, which the
+// group-per-row kernel above cannot offer for widths like 47.
+__global__ void __launch_bounds__(256) softmax_xent_tiled_kernel(const XentArgs p, int R, int CP)
+{
+    extern __shared__ float tile[];
+    __shared__ float wsum[4];
+    const int C = (int)p.C;
+    const int cv = (int)min(p.C, p.num_classes);
+    const int64_t n_tiles = (p.M + R - 1) / R;
+    const int step_r = 256 / C, step_c = 256 % C;
+    float loss_acc = 0.f;
+    for (int64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+        const int64_t row0 = t * R;
+        const int rows = (int)min((int64_t)R, p.M - row0);
+        const int count = rows * C;
+        // stage: element i of the tile is (i / C, i % C); (r, c) advance without divisions
+        int r = (int)threadIdx.x / C, c = (int)threadIdx.x % C;
+        for (int i = threadIdx.x; i < count; i += 256) {
+            tile[r * CP + c] = p.logits[(row0 + r) * p.ld + c];
+            r += step_r;
+            c += step_c;
+            if (c >= C) {
+                c -= C;
+                ++r;
+            }
+        }
+        __syncthreads();
+        if ((int)threadIdx.x < rows) {
+            float *x = tile + threadIdx.x * CP;
+            const int64_t row = row0 + threadIdx.x;
+            float mx = -INFINITY;
+            for (int k = 0; k < cv; ++k) mx = fmaxf(mx, x[k]);
+            float den = 0.f;
+            for (int k = 0; k < cv; ++k) {
+                const float e = expf(x[k] - mx);
+                x[k] = e;
+                den += e;
+            }
+            const int64_t y = p.labels[row];
+            const bool invalid_node = (p.row_offset + row >= p.num_nodes) || (y < 0);
+            const bool label_ok = (y >= 0) && (y < p.C);
+            const float inv = invalid_node ? 0.f : 1.f / den;
+            float py = 0.f;
+            for (int k = 0; k < C; ++k) {
+                const float prob = k < cv ? x[k] * inv : 0.f;
+                const bool hit = label_ok && k == (int)y;
+                if (hit) py = prob;
+                x[k] = (prob - (hit ? 1.f : 0.f)) * p.scale;
+            }
+            if (label_ok) loss_acc += -logf(fmaxf(py, 1e-9f));
+        }
+        __syncthreads();
+        if (p.dlogits != nullptr) {
+            r = (int)threadIdx.x / C;
+            c = (int)threadIdx.x % C;
+            for (int i = threadIdx.x; i < count; i += 256) {
+                p.dlogits[(row0 + r) * p.ldd + c] = tile[r * CP + c];
+                r += step_r;
+                c += step_c;
+                if (c >= C) {
+                    c -= C;
+                    ++r;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) loss_acc += __shfl_xor(loss_acc, o, 64);
+    if (lane == 0) wsum[threadIdx.x >> 6] = loss_acc;
+    __syncthreads();
+    if (threadIdx.x == 0) p.partials[blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+}
+
 __global__ void __launch_bounds__(256) xent_finish_kernel(const float *__restrict__ partials, int n, double inv_nodes,
                                                           float *__restrict__ loss)
 {
@@ -109,13 +186,19 @@ __global__ void __launch_bounds__(256) xent_finish_kernel(const float *__restric
 template <int LPR>
 int launch_xent(const XentArgs &a, int per, unsigned blocks, hipStream_t st)
 {
-    switch (per) {
-        case 1: softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a); return 0;
-        case 2: softmax_xent_kernel<LPR, 2><<<blocks, 256, 0, st>>>(a); return 0;
-        case 4: softmax_xent_kernel<LPR, 4><<<blocks, 256, 0, st>>>(a); return 0;
-        case 8: softmax_xent_kernel<LPR, 8><<<blocks, 256, 0, st>>>(a); return 0;
-        case 16: softmax_xent_kernel<LPR, 16><<<blocks, 256, 0, st>>>(a); return 0;
-        default: return -1;
+    if constexpr (LPR < 64) {
+        if (per != 1) return -1;
+        softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a);
+        return 0;
+    } else {
+        switch (per) {
+            case 1: softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a); return 0;
+            case 2: softmax_xent_kernel<LPR, 2><<<blocks, 256, 0, st>>>(a); return 0;
+            case 4: softmax_xent_kernel<LPR, 4><<<blocks, 256, 0, st>>>(a); return 0;
+            case 8: softmax_xent_kernel<LPR, 8><<<blocks, 256, 0, st>>>(a); return 0;
+            case 16: softmax_xent_kernel<LPR, 16><<<blocks, 256, 0, st>>>(a); return 0;
+            default: return -1;
+        }
     }
 }
 
@@ -165,20 +248,25 @@ int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, 
     a.row_offset = row_offset;
     a.scale = gscale / (float)num_nodes;
 
-    const int64_t rows_per_block = 4 * (64 / lpr);
-    const unsigned blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, rows_per_block), kXentMaxBlocks));
-    int rc = -1;
-    switch (lpr) {
-        case 1: rc = launch_xent<1>(a, per, blocks, st); break;
-        case 2: rc = launch_xent<2>(a, per, blocks, st); break;
-        case 4: rc = launch_xent<4>(a, per, blocks, st); break;
-        case 8: rc = launch_xent<8>(a, per, blocks, st); break;
-        case 16: rc = launch_xent<16>(a, per, blocks, st); break;
-        case 32: rc = launch_xent<32>(a, per, blocks, st); break;
-        default: rc = launch_xent<64>(a, per, blocks, st); break;
+    unsigned blocks;
+    if (C >= 2 && C <= 190) {
+        const int CP = (int)C | 1;
+        const int R = C <= 47 ? 256 : (C <= 95 ? 128 : 64);  // R * CP * 4 <= 49,152 bytes of LDS
+        blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, R), kXentMaxBlocks));
+        softmax_xent_tiled_kernel<<<blocks, 256, (size_t)R * CP * sizeof(float), st>>>(a, R, CP);
+        PLX_LAUNCH_CHECK("softmax_xent_tiled_kernel");
+    } else {
+        const int64_t rows_per_block = 4 * (64 / lpr);
+        blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, rows_per_block), kXentMaxBlocks));
+        int rc = -1;
+        switch (lpr) {
+            case 1: rc = launch_xent<1>(a, per, blocks, st); break;
+            case 64: rc = launch_xent<64>(a, per, blocks, st); break;
+            default: break;
+        }
+        if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "softmax_xent: no kernel for C=%lld", (long long)C);
+        PLX_LAUNCH_CHECK("softmax_xent_kernel");
     }
-    if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "softmax_xent: no kernel for C=%lld", (long long)C);
-    PLX_LAUNCH_CHECK("softmax_xent_kernel");
     xent_finish_kernel<<<1, 256, 0, st>>>(a.partials, (int)blocks, 1.0 / (double)num_nodes, loss);
     PLX_LAUNCH_CHECK("xent_finish_kernel");
     return PLX_OK;

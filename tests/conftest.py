@@ -33,3 +33,18 @@ def lib():
     from plexus_amd import _lib
 
     return _lib.load()
+
+
+def assert_parity(x, ref32, ref64, tol=FP32_TOL, what=""):
+    """fp32 gate with the fp64 oracle as arbiter.
+
+    Passes when x is within `tol` of the fp32 oracle (the reference's own operators on the host) or of the
+    fp64 oracle; and, where a long fp32 chain makes the two oracles themselves differ by more than `tol`,
+    when x is no further from the fp64 result than the reference's fp32 operators are.
+    """
+    e32 = rel_err(x, ref32)
+    e64 = rel_err(x, ref64)
+    ref_gap = rel_err(ref32, ref64)
+    assert e32 <= tol or e64 <= tol or e64 <= ref_gap, (
+        "%s: rel err vs fp32 oracle %.3e, vs fp64 oracle %.3e, fp32-vs-fp64 oracle gap %.3e" % (what, e32, e64, ref_gap)
+    )

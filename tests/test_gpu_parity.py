@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import BF16_TOL, FP32_TOL, rel_err
+from conftest import BF16_TOL, FP32_TOL, assert_parity, rel_err
 from oracle import oracle_c
 from oracle import plexus_oracle as po
 from plexus_amd import ops
@@ -382,3 +382,73 @@ def test_fused_adamw_matches_torch_and_oracle(n):
             po.adamw_step(mine, [g.double()], state, lr=3e-3, weight_decay=wd)
         assert rel_err(p, ref) <= FP32_TOL
         assert rel_err(p, mine[0]) <= FP32_TOL
+
+
+def test_scaled_config2_rmat_spmm_wide_and_narrow():
+    """SpMM-only configuration (R-MAT 0.57/0.19/0.19/0.05) at 1/50 scale, widths 602 and 128."""
+    say("config 2 at 1/50 scale, D=602 and D=128")
+    g = S.config2_graph(DEV, seed=0, scale=0.02)
+    n = g.shape[0]
+    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
+    print(g.degree_stats(), "long rows", a.n_long_rows, flush=True)
+    rp, ci, va = g.rowptr.cpu().numpy(), g.col.cpu().numpy(), g.val.cpu().numpy()
+    for d in (602, 128):
+        h = S.normal_features(n, d, DEV, seed=d)
+        y = ops.spmm(a, h)
+        ref = oracle_c.csr_spmm(rp, ci, va, h.cpu().numpy())
+        assert rel_err(y, ref) <= FP32_TOL
+        ref_t = po.spmm(torch.sparse_csr_tensor(g.rowptr.cpu(), g.col.cpu(), g.val.cpu(), size=g.shape), h.cpu())
+        assert rel_err(y, ref_t) <= FP32_TOL
+
+
+def test_scaled_config4_rank_block_layers():
+    """One rank's block of a 2x2x2 grid at 1/64 scale: rectangular CSR block and its transpose, a
+    feature slab that is a column slice of a wider matrix (ld != D), three layers fwd+bwd, no collectives."""
+    say("config 4 block at 1/64 scale")
+    from plexus_amd.gcn_conv import GCNConv
+
+    g = S.config4_block(DEV, seed=0, scale=1.0 / 64)
+    m, k = g.shape
+    assert m == k  # rows [0, N/2) x cols [0, N/2) of a doubly permuted matrix: not symmetric
+    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
+    at = ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (k, m))
+    a_cpu = torch.sparse_csr_tensor(g.rowptr.cpu(), g.col.cpu(), g.val.cpu(), size=g.shape)
+    at_cpu = torch.sparse_csr_tensor(g.rowptr_t.cpu(), g.col_t.cpu(), g.val_t.cpu(), size=(k, m))
+    assert not torch.equal(g.rowptr, g.rowptr_t)
+    gen = torch.Generator().manual_seed(0)
+    wide = torch.randn(k, 128, generator=gen)
+    slab = wide[:, 64:128]  # this rank's half of the feature columns
+    dims = [64, 64, 64, 24]
+    ws = [po.kaiming_uniform_weight(dims[i], dims[i + 1], gen) for i in range(3)]
+    go = torch.randn(m, dims[-1], generator=gen)
+
+    # oracle: three layers with ReLU between, backward by the reference's formulas
+    layers = [GCNConv(dims[i], dims[i + 1], i + 1, weight=ws[i], fuse_relu=(i < 2)) for i in range(3)]
+    x = wide.to(DEV)[:, 64:128].requires_grad_()  # non-contiguous view: row pitch 128, width 64
+    hcur = x
+    acts = []
+    for layer in layers:
+        hcur = layer(hcur, [(a, at)])
+        acts.append(hcur)
+    hcur.backward(go.to(DEV))
+
+    # oracle: three layers with ReLU between, backward by the reference's formulas.  The ReLU masks of
+    # the backward pass are pinned to the ones the GPU forward produced: a pre-activation within rounding
+    # of zero can take either sign in two fp32 summation orders (the forward outputs are compared on
+    # their own, and the masks may differ in a handful of such elements only).
+    net = po.OracleNet(ws, dims)
+    out_ref = net.forward(slab.contiguous(), [(a_cpu, at_cpu)])
+    net64 = po.OracleNet([w.double() for w in ws], dims)
+    out64 = net64.forward(slab.contiguous().double(), [(a_cpu.double(), at_cpu.double())])
+    masks = [(acts[0] > 0).cpu(), (acts[1] > 0).cpu(), None]
+    for i in range(2):
+        flips = int((masks[i] != (net64._saved[i][3] > 0)).sum())
+        print("layer %d: %d ReLU mask elements differ from the fp64 oracle" % (i, flips), flush=True)
+        assert flips <= 4
+        assert rel_err(acts[i], torch.relu(net._saved[i][3])) <= FP32_TOL
+    gx_ref, gws_ref = net.backward(go, masks)
+    gx64, gws64 = net64.backward(go.double(), masks)
+    assert_parity(hcur, out_ref, out64, what="OUT")
+    assert_parity(x.grad, gx_ref.reshape(k, 64), gx64.reshape(k, 64), what="grad_x")
+    for i, layer in enumerate(layers):
+        assert_parity(layer.weight.grad, gws_ref[i], gws64[i], what="grad_w[%d]" % i)
