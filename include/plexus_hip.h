@@ -37,7 +37,8 @@ typedef enum plx_status {
 } plx_status;
 
 /* epilogue / prologue flags of the GEMM entry points */
-#define PLX_GEMM_RELU 1u /* C = max(C, 0) (examples/train.py:77-78 fused into the producer) */
+#define PLX_GEMM_RELU 1u    /* C = max(C, 0) (examples/train.py:77-78 fused into the producer) */
+#define PLX_GEMM_DROPOUT 2u /* after the ReLU: zero with probability p, scale the rest by 1 / (1 - p) */
 
 int plx_version(void);
 const char *plx_error_string(int status);
@@ -110,6 +111,31 @@ int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
                     float *C, int64_t ldc, const float *mask, int64_t ldmask, void *workspace,
                     size_t workspace_bytes, void *stream);
 
+/* ---- bf16 storage, fp32 accumulation (raw uint16 bit patterns; the reference has no reduced-precision
+ *      path, these follow the same call sites as the fp32 entry points above) ----
+ *
+ * C[M x N] = epilogue(alpha * (A ⊙ [mask > 0])[M x K] . B[N x K]^T), C bf16.
+ *   forward  OUT = AGG . W: pass B = W^T stored [N_out x K_in] (plx_cast_f32_bf16 with transpose = 1 makes it
+ *   from the fp32 weight), flags PLX_GEMM_RELU and/or PLX_GEMM_DROPOUT;
+ *   backward GRAD_AGG = GRAD_OUT . W^T: pass B = W stored [K_in x N_out], mask = the layer's output,
+ *   alpha = 1 / (1 - p) when the forward applied dropout.
+ * Dropout is counter-based so that a host can regenerate the mask: element e (row-major linear index
+ * r * N + c) is kept iff 16-bit lane (e % 8) of Philox-4x32-10(counter = (e / 8, offset), key = seed) is
+ * >= round(p * 65536); lane i is the low (i even) or high (i odd) half of output word i / 2. */
+int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                     uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, unsigned flags,
+                     float dropout_p, uint64_t seed, uint64_t offset, void *stream);
+
+/* C[K x N] (fp32) = alpha * A[M x K]^T . (B ⊙ [mask > 0])[M x N]      GRAD_W = AGG^T . GRAD_OUT */
+size_t plx_gemm_tn_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                     float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* Y = bf16(X) (transpose = 0, Y is [M x N]) or bf16(X^T) (transpose = 1, Y is [N x M]); X is [M x N] fp32. */
+int plx_cast_f32_bf16(int64_t M, int64_t N, const float *X, int64_t ldx, uint16_t *Y, int64_t ldy, int transpose,
+                      void *stream);
+
 /* Y = max(X, 0) and dX = dY ⊙ [Y > 0] for callers that keep F.relu outside the layer
  * (examples/train.py:77-78). */
 int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream);
@@ -132,6 +158,10 @@ size_t plx_softmax_xent_workspace_bytes(int64_t M, int64_t C);
 int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
                          int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
                          float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream);
+/* bf16 logits and gradient, fp32 math and fp32 loss */
+int plx_softmax_xent_bf16(int64_t M, int64_t C, const uint16_t *logits, int64_t ld, const int64_t *labels,
+                          int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
+                          uint16_t *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Symmetric GCN normalisation of a CSR matrix that already holds its self loops
@@ -153,6 +183,11 @@ int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, c
  * ---------------------------------------------------------------------------------------- */
 int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, float lr, float beta1,
                   float beta2, float eps, float weight_decay, int64_t step, void *stream);
+/* same update with a bf16 gradient (fp32 parameter and moments); optionally also writes bf16(param) to
+ * param_bf16 (may be NULL) so that the next forward needs no separate cast pass */
+int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, float lr,
+                            float beta1, float beta2, float eps, float weight_decay, int64_t step, uint16_t *param_bf16,
+                            void *stream);
 
 #ifdef __cplusplus
 }

@@ -338,14 +338,83 @@ def philox4x32_10(counter: np.ndarray, key: Tuple[int, int]) -> np.ndarray:
 
 
 def dropout_keep_mask(n_elems: int, seed: int, offset: int, p: float) -> np.ndarray:
-    """Keep-mask of element e: word (e % 4) of Philox(counter=(e//4, offset, 0, 0), key=seed) >= p * 2^32."""
-    n4 = (n_elems + 3) // 4
-    ctr = np.zeros((n4, 4), dtype=np.uint32)
-    idx = np.arange(n4, dtype=np.uint64)
+    """Keep-mask of the fused dropout (not in the reference; counter-based so host and device agree).
+
+    Element e (row-major linear index) uses call q = e // 8 of Philox-4x32-10 with counter
+    (q, offset) and key seed; its 16-bit lane is the low (e even) or high (e odd) half of output word
+    (e % 8) // 2; the element is kept iff lane >= round(p * 65536).
+    """
+    n8 = (n_elems + 7) // 8
+    ctr = np.zeros((n8, 4), dtype=np.uint32)
+    idx = np.arange(n8, dtype=np.uint64)
     ctr[:, 0] = (idx & np.uint64(0xFFFFFFFF)).astype(np.uint32)
     ctr[:, 1] = (idx >> np.uint64(32)).astype(np.uint32)
     ctr[:, 2] = np.uint32(offset & 0xFFFFFFFF)
     ctr[:, 3] = np.uint32((offset >> 32) & 0xFFFFFFFF)
-    r = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)).reshape(-1)[:n_elems]
-    thresh = np.uint64(min(int(p * 4294967296.0), 4294967295))
-    return r.astype(np.uint64) >= thresh
+    words = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))  # (n8, 4)
+    lanes = np.empty((n8, 8), dtype=np.uint32)
+    lanes[:, 0::2] = words & np.uint32(0xFFFF)
+    lanes[:, 1::2] = words >> np.uint32(16)
+    thresh = min(int(round(p * 65536.0)), 65535)
+    return lanes.reshape(-1)[:n_elems] >= np.uint32(thresh)
+
+
+# --------------------------------------------------------------------------
+# bf16 storage with fp32 accumulation (not in the reference): the fp32 operator sequence above with
+# every STORED tensor rounded to bf16, which is what the device path keeps in memory
+# --------------------------------------------------------------------------
+def rb(t: torch.Tensor) -> torch.Tensor:
+    """Round to bf16 and back (round-to-nearest-even), keeping the working dtype."""
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
+class OracleNetBf16:
+    """OracleNet with bf16-stored activations, optional dropout after each ReLU, fp32 weights.
+
+    forward:  AGG = rb(A.H); OUT = rb(dropout(relu(AGG . rb(W))))          (last layer: no ReLU / dropout)
+    backward: G' = G * [OUT > 0] / (1 - p); GRAD_W = AGG^T . G' (fp32, not rounded);
+              GRAD_AGG = rb(G' . rb(W)^T); GRAD_H = rb(A^T . GRAD_AGG)
+    ``offsets[i]`` is the dropout offset of layer i for this forward pass.
+    """
+
+    def __init__(self, weights, dims, dropout_p=0.0, seed=0):
+        self.weights = [w.clone() for w in weights]
+        self.dims = list(dims)
+        self.p = dropout_p
+        self.seed = seed
+
+    def forward(self, x, adj_shards, offsets=None):
+        saved = []
+        h = rb(x)
+        n_layers = len(self.weights)
+        for i, w in enumerate(self.weights):
+            a, a_t = adj_shards[i % len(adj_shards)]
+            agg = rb(torch.sparse.mm(a, h.reshape(a.shape[1], self.dims[i])))
+            out = torch.mm(agg, rb(w.reshape(self.dims[i], self.dims[i + 1])))
+            last = i == n_layers - 1
+            if not last:
+                out = F.relu(out)
+                if self.p > 0.0:
+                    keep = dropout_keep_mask(out.numel(), self.seed, offsets[i], self.p).reshape(out.shape)
+                    out = out * torch.from_numpy(keep).to(out.dtype) / (1.0 - self.p)
+            out = rb(out)
+            saved.append((agg, a_t, out, last))
+            h = out
+        self._saved = saved
+        return h
+
+    def backward(self, grad_logits):
+        g = rb(grad_logits)
+        grads_w = [None] * len(self.weights)
+        for i in reversed(range(len(self.weights))):
+            agg, a_t, out, last = self._saved[i]
+            w = rb(self.weights[i].reshape(self.dims[i], self.dims[i + 1]))
+            if not last:
+                g = g * (out > 0).to(g.dtype)
+                scale = 1.0 / (1.0 - self.p) if self.p > 0.0 else 1.0
+            else:
+                scale = 1.0
+            grads_w[i] = (scale * torch.mm(torch.t(agg), g)).reshape(-1)
+            grad_agg = rb(scale * torch.mm(g, torch.t(w)))
+            g = rb(torch.sparse.mm(a_t, grad_agg))
+        return g, grads_w

@@ -41,9 +41,17 @@ SIGNATURES = {
     "plx_softmax_xent_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "plx_gcn_norm_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "plx_adamw_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32, _f32, _i64, _vp]),
+    "plx_adamw_f32_grad_bf16": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32, _f32, _i64, _vp, _vp]),
+    "plx_gemm_nt_bf16": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _u32, _f32,
+                                   C.c_uint64, C.c_uint64, _vp]),
+    "plx_gemm_tn_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_gemm_tn_bf16": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz, _vp]),
+    "plx_cast_f32_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, C.c_int, _vp]),
+    "plx_softmax_xent_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
 }
 
 PLX_GEMM_RELU = 1
+PLX_GEMM_DROPOUT = 2
 
 _lib = None
 

@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdint>
 
+#include "bf16.h"
 #include "common.h"
 
 namespace {
@@ -110,6 +111,27 @@ __global__ void __launch_bounds__(256) adamw_kernel(int64_t n, float *__restrict
     }
 }
 
+// AdamW with a bf16 gradient; optionally refreshes a bf16 copy of the parameter in the same pass
+__global__ void __launch_bounds__(256) adamw_grad_bf16_kernel(int64_t n, float *__restrict__ p, const uint16_t *__restrict__ g,
+                                                              float *__restrict__ m, float *__restrict__ v, float decay,
+                                                              float one_minus_b1, float b2, float one_minus_b2,
+                                                              float step_size, float inv_bc2_sqrt, float eps,
+                                                              uint16_t *__restrict__ p16)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float ge = plx::bf16_to_f32(g[i]);
+        const float me = m[i] + (ge - m[i]) * one_minus_b1;
+        const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
+        const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
+        const float pe = p[i] * decay - step_size * (me / denom);
+        p[i] = pe;
+        m[i] = me;
+        v[i] = ve;
+        if (p16 != nullptr) p16[i] = (uint16_t)plx::f32_to_bf16(pe);
+    }
+}
+
 int relu_common(bool bwd, int64_t M, int64_t N, const float *in, int64_t ldi, const float *ref, int64_t ldr, float *out,
                 int64_t ldo, void *stream)
 {
@@ -174,6 +196,23 @@ int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, fl
         adamw_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2, 1.0f - beta2,
                                                     step_size, inv_bc2_sqrt, eps);
     PLX_LAUNCH_CHECK("adamw_kernel");
+    return PLX_OK;
+}
+
+int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, float lr,
+                            float beta1, float beta2, float eps, float weight_decay, int64_t step, uint16_t *param_bf16,
+                            void *stream)
+{
+    PLX_REQUIRE(n >= 0 && step >= 1, "adamw: bad size or step (n=%lld step=%lld)", (long long)n, (long long)step);
+    if (n == 0) return PLX_OK;
+    PLX_REQUIRE(param && grad && exp_avg && exp_avg_sq, "adamw: NULL operand");
+    const double bc1 = 1.0 - std::pow((double)beta1, (double)step);
+    const double bc2 = 1.0 - std::pow((double)beta2, (double)step);
+    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(n, 256), 256 * 32);
+    adamw_grad_bf16_kernel<<<blocks, 256, 0, plx::as_stream(stream)>>>(n, param, grad, exp_avg, exp_avg_sq, 1.0f - lr * weight_decay,
+                                                                      1.0f - beta1, beta2, 1.0f - beta2, (float)((double)lr / bc1),
+                                                                      (float)(1.0 / std::sqrt(bc2)), eps, param_bf16);
+    PLX_LAUNCH_CHECK("adamw_grad_bf16_kernel");
     return PLX_OK;
 }
 

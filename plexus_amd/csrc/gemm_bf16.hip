@@ -1,0 +1,535 @@
+// Dense products of the GCN layer with bf16 storage and fp32 accumulation (v_mfma_f32_32x32x16_bf16).
+//
+//   NT  C[M x N] (bf16) = epilogue(alpha * (A*mask)[M x K] . B[N x K]^T)
+//         forward  OUT      = AGG . W        with B = W^T stored [N_out x K_in]  (+ ReLU, + dropout)
+//         backward GRAD_AGG = GRAD_OUT . W^T with B = W   stored [K_in x N_out]  (+ ReLU/dropout mask, alpha = 1/(1-p))
+//   TN  C[K x N] (fp32) = alpha * A[M x K]^T . (B*mask)[M x N]          GRAD_W = AGG^T . GRAD_OUT
+//
+// With bf16 storage these tall-skinny products are bound by HBM, not by the matrix cores (the MFMA
+// rate is 16x the fp32 one), so the kernels are built around wide memory accesses:
+//   * operands are fetched as 16-byte vectors (8 bf16) along contiguous memory;
+//   * an MFMA lane needs 8 consecutive contraction indices of one row/column.  For NT both operands
+//     are already contraction-contiguous ("x-major" LDS tiles, one 128-bit LDS read per fragment).  For
+//     TN the contraction runs over the rows of both operands, so tiles are transposed on their way into
+//     LDS: a thread loads the same 8 columns of two consecutive rows and writes eight 32-bit words
+//     (row pair packed) down a column of the transposed tile;
+//   * the NT output goes through LDS so that every lane stores 16 bytes of one output row; the dropout
+//     generator (Philox-4x32-10) is called once per 8 consecutive elements there.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+
+#include "bf16.h"
+#include "common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128;      // output rows per workgroup
+constexpr int kBK = 64;       // contraction chunk (bf16 elements)
+constexpr int kS = kBK + 8;   // LDS row stride in bf16 elements: 144 bytes, keeps 128-bit reads conflict-free
+constexpr int kThreads = 256;
+
+struct Bf16Args {
+    const uint16_t *A;
+    const uint16_t *B;
+    const uint16_t *mask;
+    void *C;
+    int64_t lda, ldb, ldc, ldmask;
+    int64_t M, N, K;
+    float alpha;
+    unsigned flags;
+    uint32_t thresh16;   // keep iff 16-bit lane >= thresh16
+    float keep_scale;    // 1 / (1 - p)
+    uint32_t seed_lo, seed_hi, off_lo, off_hi;
+    int a_vec, b_vec, c_vec, m_vec;
+    // TN only
+    int64_t rows_per_split;
+    float *ws;
+    int64_t ws_ld, ws_slab;
+};
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// 8 consecutive bf16 of a row, zero beyond `valid` elements; 16-byte load when allowed
+__device__ __forceinline__ uint4 load8(const uint16_t *q, int valid, int vec_ok)
+{
+    if (valid >= 8 && vec_ok) return *reinterpret_cast<const uint4 *>(q);
+    uint32_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) e[i] = i < valid ? (uint32_t)q[i] : 0u;
+    return make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+}
+
+__device__ __forceinline__ uint32_t mask2(uint32_t v, uint32_t m)
+{
+    const uint32_t lo = plx::bf16_positive(m & 0xffffu) ? 0x0000ffffu : 0u;
+    const uint32_t hi = plx::bf16_positive(m >> 16) ? 0xffff0000u : 0u;
+    return v & (lo | hi);
+}
+
+__device__ __forceinline__ uint4 mask8(uint4 v, uint4 m) { return make_uint4(mask2(v.x, m.x), mask2(v.y, m.y), mask2(v.z, m.z), mask2(v.w, m.w)); }
+
+// ------------------------------------------------------------------------------------------------
+// NT: C = epilogue(alpha * (A*mask) . B^T), A [M x K], B [N x K], both contraction-contiguous
+// ------------------------------------------------------------------------------------------------
+template <int TN, bool MASKED>
+__global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr int kAVec = kBM * kBK / 8 / kThreads;                       // 16-byte vectors per thread, A tile
+    constexpr int kBVec = (BN * kBK / 8 + kThreads - 1) / kThreads;       // B tile
+    constexpr int kTile = (kBM + BN) * kS;                                // bf16 elements per buffer
+    constexpr int kCS = BN + 4;                                           // fp32 row stride of the staged output
+    static_assert(4 * 32 * kCS * 4 <= 2 * kTile * 2, "staged output must fit the operand buffers");
+
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kTile];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    const int64_t row0 = (int64_t)blockIdx.x * kBM;
+    const int64_t col0 = (int64_t)blockIdx.y * BN;
+
+    uint4 ra[kAVec], rb[kBVec];
+    auto fetch = [&](int64_t k0) {
+#pragma unroll
+        for (int p = 0; p < kAVec; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            const int64_t r = row0 + idx / 8;
+            const int64_t k = k0 + (idx % 8) * 8;
+            uint4 v = zero4();
+            if (r < g.M && k < g.K) {
+                const int valid = (int)min((int64_t)8, g.K - k);
+                v = load8(g.A + r * g.lda + k, valid, g.a_vec);
+                if constexpr (MASKED) v = mask8(v, load8(g.mask + r * g.ldmask + k, valid, g.m_vec));
+            }
+            ra[p] = v;
+        }
+#pragma unroll
+        for (int p = 0; p < kBVec; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            const int64_t n = col0 + idx / 8;
+            const int64_t k = k0 + (idx % 8) * 8;
+            uint4 v = zero4();
+            if (idx < BN * 8 && n < g.N && k < g.K) v = load8(g.B + n * g.ldb + k, (int)min((int64_t)8, g.K - k), g.b_vec);
+            rb[p] = v;
+        }
+    };
+    auto stash = [&](int buf) {
+        uint16_t *as = lds + buf * kTile;
+        uint16_t *bs = as + kBM * kS;
+#pragma unroll
+        for (int p = 0; p < kAVec; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            *reinterpret_cast<uint4 *>(as + (idx / 8) * kS + (idx % 8) * 8) = ra[p];
+        }
+#pragma unroll
+        for (int p = 0; p < kBVec; ++p) {
+            const int idx = p * kThreads + threadIdx.x;
+            if (idx < BN * 8) *reinterpret_cast<uint4 *>(bs + (idx / 8) * kS + (idx % 8) * 8) = rb[p];
+        }
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    int buf = 0;
+    if (g.K > 0) {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t k0 = 0; k0 < g.K; k0 += kBK) {
+        const bool more = k0 + kBK < g.K;
+        if (more) fetch(k0 + kBK);
+        const uint16_t *as = lds + buf * kTile;
+        const uint16_t *bs = as + kBM * kS;
+#pragma unroll
+        for (int s = 0; s < kBK / 16; ++s) {
+            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(as + (wave * 32 + li) * kS + 16 * s + 8 * h);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(bs + (t * 32 + li) * kS + 16 * s + 8 * h);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // stage the wavefront's 32 x BN fp32 tile in LDS (register v of a lane is row 8 (v / 4) + 4 h + v % 4,
+    // column lane % 32 of each 32 x 32 tile), then hand out 8 consecutive columns of one row per lane
+    float *cs = reinterpret_cast<float *>(lds) + wave * 32 * kCS;
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) cs[(8 * (v / 4) + 4 * h + (v % 4)) * kCS + t * 32 + li] = acc[t][v];
+    __syncthreads();
+
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+    const bool drop = (g.flags & PLX_GEMM_DROPOUT) != 0;
+    uint16_t *C = static_cast<uint16_t *>(g.C);
+    constexpr int kVecPerRow = BN / 8;
+#pragma unroll
+    for (int it = 0; it < 32 * kVecPerRow / 64; ++it) {
+        const int id = it * 64 + lane;
+        const int rl = id / kVecPerRow;
+        const int cq = id % kVecPerRow;
+        const int64_t r = row0 + wave * 32 + rl;
+        const int64_t c = col0 + cq * 8;
+        if (r >= g.M || c >= g.N) continue;
+        const float4 lo = *reinterpret_cast<const float4 *>(cs + rl * kCS + cq * 8);
+        const float4 hi = *reinterpret_cast<const float4 *>(cs + rl * kCS + cq * 8 + 4);
+        float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x[e] *= g.alpha;
+            if (relu) x[e] = fmaxf(x[e], 0.f);
+        }
+        const int valid = (int)min((int64_t)8, g.N - c);
+        if (drop) {
+            const uint64_t e0 = (uint64_t)r * (uint64_t)g.N + (uint64_t)c;
+            if ((e0 & 7u) == 0) {
+                const uint64_t q = e0 >> 3;
+                const plx::Philox4 rnd = plx::philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), g.off_lo, g.off_hi, g.seed_lo, g.seed_hi);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = plx::dropout_lane16(rnd, e) >= g.thresh16 ? x[e] * g.keep_scale : 0.f;
+            } else {
+                for (int e = 0; e < valid; ++e) {
+                    const uint64_t ee = e0 + e;
+                    const uint64_t q = ee >> 3;
+                    const plx::Philox4 rnd = plx::philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), g.off_lo, g.off_hi, g.seed_lo, g.seed_hi);
+                    x[e] = plx::dropout_lane16(rnd, (int)(ee & 7u)) >= g.thresh16 ? x[e] * g.keep_scale : 0.f;
+                }
+            }
+        }
+        uint16_t *dst = C + r * g.ldc + c;
+        if (valid == 8 && g.c_vec) {
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(plx::pack_bf16x2(x[0], x[1]), plx::pack_bf16x2(x[2], x[3]),
+                                                         plx::pack_bf16x2(x[4], x[5]), plx::pack_bf16x2(x[6], x[7]));
+        } else {
+            for (int e = 0; e < valid; ++e) dst[e] = (uint16_t)plx::f32_to_bf16(x[e]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// TN: C[K x N] (fp32) = alpha * A[M x K]^T . (B*mask)[M x N]; contraction over the rows of both
+// ------------------------------------------------------------------------------------------------
+template <int TN, bool MASKED>
+__global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr int kAItems = 32 * (kBM / 8) / kThreads;                      // (row pair, 8-column vector) items per thread
+    constexpr int kBItems = (32 * (BN / 8) + kThreads - 1) / kThreads;
+    constexpr int kTile = (kBM + BN) * kS;
+
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kTile];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    const int64_t row0 = (int64_t)blockIdx.y * kBM;  // rows of C = columns of A
+    const int64_t col0 = (int64_t)blockIdx.z * BN;   // columns of C = columns of B
+    const int64_t mbeg = (int64_t)blockIdx.x * g.rows_per_split;
+    const int64_t mend = min(mbeg + g.rows_per_split, g.M);
+
+    uint4 ra[kAItems][2], rb[kBItems][2];
+    auto fetch = [&](int64_t m0) {
+#pragma unroll
+        for (int p = 0; p < kAItems; ++p) {
+            const int item = p * kThreads + threadIdx.x;
+            const int mp = item % 32, cq = item / 32;
+            const int64_t c = row0 + cq * 8;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int64_t m = m0 + 2 * mp + j;
+                uint4 v = zero4();
+                if (m < mend && c < g.K) v = load8(g.A + m * g.lda + c, (int)min((int64_t)8, g.K - c), g.a_vec);
+                ra[p][j] = v;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < kBItems; ++p) {
+            const int item = p * kThreads + threadIdx.x;
+            const int mp = item % 32, cq = item / 32;
+            const int64_t c = col0 + cq * 8;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int64_t m = m0 + 2 * mp + j;
+                uint4 v = zero4();
+                if (cq < BN / 8 && m < mend && c < g.N) {
+                    const int valid = (int)min((int64_t)8, g.N - c);
+                    v = load8(g.B + m * g.ldb + c, valid, g.b_vec);
+                    if constexpr (MASKED) v = mask8(v, load8(g.mask + m * g.ldmask + c, valid, g.m_vec));
+                }
+                rb[p][j] = v;
+            }
+        }
+    };
+    // transposed stash: word e of the pair holds (row 2 mp, row 2 mp + 1) of column 8 cq + e
+    auto stash_pair = [&](uint16_t *t, int mp, int cq, const uint4 &r0, const uint4 &r1) {
+        const uint32_t a[4] = {r0.x, r0.y, r0.z, r0.w};
+        const uint32_t b[4] = {r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t lo = (e & 1) ? (a[e >> 1] >> 16) : (a[e >> 1] & 0xffffu);
+            const uint32_t hi = (e & 1) ? (b[e >> 1] >> 16) : (b[e >> 1] & 0xffffu);
+            *reinterpret_cast<uint32_t *>(t + (cq * 8 + e) * kS + 2 * mp) = lo | (hi << 16);
+        }
+    };
+    auto stash = [&](int buf) {
+        uint16_t *at = lds + buf * kTile;
+        uint16_t *bt = at + kBM * kS;
+#pragma unroll
+        for (int p = 0; p < kAItems; ++p) {
+            const int item = p * kThreads + threadIdx.x;
+            stash_pair(at, item % 32, item / 32, ra[p][0], ra[p][1]);
+        }
+#pragma unroll
+        for (int p = 0; p < kBItems; ++p) {
+            const int item = p * kThreads + threadIdx.x;
+            if (item / 32 < BN / 8) stash_pair(bt, item % 32, item / 32, rb[p][0], rb[p][1]);
+        }
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    int buf = 0;
+    if (mbeg < mend) {
+        fetch(mbeg);
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t m0 = mbeg; m0 < mend; m0 += kBK) {
+        const bool more = m0 + kBK < mend;
+        if (more) fetch(m0 + kBK);
+        const uint16_t *at = lds + buf * kTile;
+        const uint16_t *bt = at + kBM * kS;
+#pragma unroll
+        for (int s = 0; s < kBK / 16; ++s) {
+            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(at + (wave * 32 + li) * kS + 16 * s + 8 * h);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(bt + (t * 32 + li) * kS + 16 * s + 8 * h);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    float *out;
+    int64_t ldo;
+    float scale;
+    if (g.ws != nullptr) {
+        out = g.ws + (int64_t)blockIdx.x * g.ws_slab;
+        ldo = g.ws_ld;
+        scale = 1.f;  // alpha is applied when the partial tiles are added
+    } else {
+        out = static_cast<float *>(g.C);
+        ldo = g.ldc;
+        scale = g.alpha;
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int64_t c = col0 + t * 32 + li;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t r = row0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+            if (c < g.N && r < g.K) out[r * ldo + c] = acc[t][v] * scale;
+        }
+    }
+}
+
+// C[e] = alpha * sum over splits of ws[s][e]; four interleaved chains, added in chain order
+__global__ void __launch_bounds__(256) gemm_bf16_tn_reduce(const float *__restrict__ ws, int64_t ws_ld, int64_t ws_slab,
+                                                           int splits, int64_t rows, int64_t cols, float alpha,
+                                                           float *__restrict__ C, int64_t ldc)
+{
+    __shared__ float part[4][64];
+    const int e_local = threadIdx.x & 63;
+    const int chain = threadIdx.x >> 6;
+    const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
+    const int64_t total = rows * cols;
+    float s = 0.f;
+    int64_t r = 0, c = 0;
+    if (e < total) {
+        r = e / cols;
+        c = e % cols;
+        const float *p = ws + r * ws_ld + c;
+        for (int i = chain; i < splits; i += 4) s += p[(int64_t)i * ws_slab];
+    }
+    part[chain][e_local] = s;
+    __syncthreads();
+    if (chain == 0 && e < total)
+        C[r * ldc + c] = alpha * (((part[0][e_local] + part[1][e_local]) + part[2][e_local]) + part[3][e_local]);
+}
+
+// Y = bf16(X) or bf16(X^T): 32 x 32 tiles through LDS so that both sides are accessed along rows
+__global__ void __launch_bounds__(256) cast_f32_bf16_kernel(int64_t M, int64_t N, const float *__restrict__ X, int64_t ldx,
+                                                            uint16_t *__restrict__ Y, int64_t ldy, int transpose)
+{
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    const int64_t r0 = (int64_t)blockIdx.x * 32, c0 = (int64_t)blockIdx.y * 32;
+    for (int j = ty; j < 32; j += 8) {
+        const int64_t r = r0 + j, c = c0 + tx;
+        tile[j][tx] = (r < M && c < N) ? X[r * ldx + c] : 0.f;
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        if (transpose) {
+            const int64_t r = c0 + j, c = r0 + tx;  // Y is [N x M]
+            if (r < N && c < M) Y[r * ldy + c] = (uint16_t)plx::f32_to_bf16(tile[tx][j]);
+        } else {
+            const int64_t r = r0 + j, c = c0 + tx;
+            if (r < M && c < N) Y[r * ldy + c] = (uint16_t)plx::f32_to_bf16(tile[j][tx]);
+        }
+    }
+}
+
+int vec16(const void *p, int64_t ld) { return (p == nullptr || (reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 8 == 0)) ? 1 : 0; }
+int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
+
+int64_t tn_splits(int64_t M, int64_t N, int64_t K)
+{
+    const int64_t tiles = plx::ceil_div(K, kBM) * plx::ceil_div(N, 32 * pick_tn(N));
+    const int64_t want = std::max<int64_t>(1, 1024 / tiles);
+    const int64_t by_rows = std::max<int64_t>(1, M / 512);
+    return std::max<int64_t>(1, std::min(want, by_rows));
+}
+
+template <bool MASKED>
+void launch_nt(const Bf16Args &g, int tn, dim3 grid, hipStream_t st)
+{
+    switch (tn) {
+        case 1: gemm_bf16_nt_kernel<1, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_bf16_nt_kernel<2, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_bf16_nt_kernel<4, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+    }
+}
+
+template <bool MASKED>
+void launch_tn(const Bf16Args &g, int tn, dim3 grid, hipStream_t st)
+{
+    switch (tn) {
+        case 1: gemm_bf16_tn_kernel<1, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_bf16_tn_kernel<2, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_bf16_tn_kernel<4, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                     uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, unsigned flags,
+                     float dropout_p, uint64_t seed, uint64_t offset, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_bf16: negative dimension");
+    PLX_REQUIRE(N < (1ll << 30) && K < (1ll << 30), "gemm_nt_bf16: dimension too large");
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(C != nullptr, "gemm_nt_bf16: NULL output");
+    PLX_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "gemm_nt_bf16: NULL operand");
+    PLX_REQUIRE(lda >= K && ldb >= K && ldc >= N, "gemm_nt_bf16: leading dimension too small");
+    PLX_REQUIRE(mask == nullptr || ldmask >= K, "gemm_nt_bf16: mask leading dimension too small");
+    PLX_REQUIRE(!(flags & PLX_GEMM_DROPOUT) || (dropout_p >= 0.f && dropout_p < 1.f), "gemm_nt_bf16: dropout p=%g outside [0, 1)",
+                (double)dropout_p);
+    Bf16Args g{};
+    g.A = A; g.B = B; g.mask = mask; g.C = C;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
+    g.M = M; g.N = N; g.K = K;
+    g.alpha = alpha; g.flags = flags;
+    g.thresh16 = (uint32_t)std::min<long long>(65535, llroundf(dropout_p * 65536.f));
+    g.keep_scale = 1.f / (1.f - dropout_p);
+    g.seed_lo = (uint32_t)seed; g.seed_hi = (uint32_t)(seed >> 32);
+    g.off_lo = (uint32_t)offset; g.off_hi = (uint32_t)(offset >> 32);
+    g.a_vec = vec16(A, lda); g.b_vec = vec16(B, ldb); g.c_vec = vec16(C, ldc); g.m_vec = vec16(mask, ldmask);
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
+    if (mask != nullptr) launch_nt<true>(g, tn, grid, plx::as_stream(stream));
+    else launch_nt<false>(g, tn, grid, plx::as_stream(stream));
+    PLX_LAUNCH_CHECK("gemm_bf16_nt_kernel");
+    return PLX_OK;
+}
+
+size_t plx_gemm_tn_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t splits = tn_splits(M, N, K);
+    if (splits <= 1) return 0;
+    const int64_t ld = (N + 3) / 4 * 4;
+    return (size_t)splits * (size_t)K * (size_t)ld * sizeof(float);
+}
+
+int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                     float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, void *workspace,
+                     size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_tn_bf16: negative dimension");
+    if (K == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(C != nullptr, "gemm_tn_bf16: NULL output");
+    PLX_REQUIRE(M == 0 || (A != nullptr && B != nullptr), "gemm_tn_bf16: NULL operand");
+    PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_tn_bf16: leading dimension too small");
+    PLX_REQUIRE(mask == nullptr || ldmask >= N, "gemm_tn_bf16: mask leading dimension too small");
+    hipStream_t st = plx::as_stream(stream);
+    const int64_t splits = tn_splits(std::max<int64_t>(M, 1), N, K);
+    const size_t need = plx_gemm_tn_bf16_workspace_bytes(M, N, K);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
+        return plx::fail(PLX_ERR_WORKSPACE, "gemm_tn_bf16: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    Bf16Args g{};
+    g.A = A; g.B = B; g.mask = mask; g.C = C;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
+    g.M = M; g.N = N; g.K = K; g.alpha = alpha;
+    g.a_vec = vec16(A, lda); g.b_vec = vec16(B, ldb); g.m_vec = vec16(mask, ldmask);
+    g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;
+    const int64_t used = plx::ceil_div(std::max<int64_t>(M, 1), g.rows_per_split);
+    if (splits > 1) {
+        g.ws = static_cast<float *>(workspace);
+        g.ws_ld = (N + 3) / 4 * 4;
+        g.ws_slab = K * g.ws_ld;
+    }
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
+    if (mask != nullptr) launch_tn<true>(g, tn, grid, st);
+    else launch_tn<false>(g, tn, grid, st);
+    PLX_LAUNCH_CHECK("gemm_bf16_tn_kernel");
+    if (splits > 1) {
+        gemm_bf16_tn_reduce<<<(unsigned)plx::ceil_div(K * N, 64), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, alpha, C, ldc);
+        PLX_LAUNCH_CHECK("gemm_bf16_tn_reduce");
+    }
+    return PLX_OK;
+}
+
+int plx_cast_f32_bf16(int64_t M, int64_t N, const float *X, int64_t ldx, uint16_t *Y, int64_t ldy, int transpose, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0, "cast_f32_bf16: negative shape");
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(X && Y, "cast_f32_bf16: NULL operand");
+    PLX_REQUIRE(ldx >= N && ldy >= (transpose ? M : N), "cast_f32_bf16: leading dimension too small");
+    PLX_REQUIRE(N <= 32ll * 65535, "cast_f32_bf16: too many columns");
+    dim3 grid((unsigned)plx::ceil_div(M, 32), (unsigned)plx::ceil_div(N, 32), 1);
+    cast_f32_bf16_kernel<<<grid, 256, 0, plx::as_stream(stream)>>>(M, N, X, ldx, Y, ldy, transpose);
+    PLX_LAUNCH_CHECK("cast_f32_bf16_kernel");
+    return PLX_OK;
+}
+
+}  // extern "C"

@@ -12,6 +12,7 @@
 #include <cmath>
 #include <cstdint>
 
+#include "bf16.h"
 #include "common.h"
 
 namespace {
@@ -19,17 +20,35 @@ namespace {
 constexpr int kXentMaxBlocks = 4096;
 constexpr int kMaxPerLane = 16;  // classes per lane kept in registers: C <= 64 * 16
 
+// element access for fp32 (float) or bf16 (uint16_t bit pattern) storage; the arithmetic is fp32
+template <typename T>
+__device__ __forceinline__ float ld_elem(const void *base, int64_t i)
+{
+    if constexpr (sizeof(T) == 4)
+        return static_cast<const float *>(base)[i];
+    else
+        return plx::bf16_to_f32(static_cast<const uint16_t *>(base)[i]);
+}
+template <typename T>
+__device__ __forceinline__ void st_elem(void *base, int64_t i, float v)
+{
+    if constexpr (sizeof(T) == 4)
+        static_cast<float *>(base)[i] = v;
+    else
+        static_cast<uint16_t *>(base)[i] = (uint16_t)plx::f32_to_bf16(v);
+}
+
 struct XentArgs {
-    const float *logits;
+    const void *logits;
     const int64_t *labels;
-    float *dlogits;
+    void *dlogits;
     float *partials;
     int64_t ld, ldd;
     int64_t M, C, num_nodes, num_classes, row_offset;
     float scale;  // gscale / num_nodes
 };
 
-template <int LPR, int PER>
+template <typename T, int LPR, int PER>
 __global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
 {
     constexpr int RPW = 64 / LPR;  // rows per wavefront
@@ -46,13 +65,13 @@ __global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
     for (int64_t gb = blockIdx.x; gb < n_groups; gb += gridDim.x) {
         const int64_t r = gb * rows_per_block + wave * RPW + grp;
         const bool row_ok = r < p.M;
-        const float *x = p.logits + (row_ok ? r : 0) * p.ld;
+        const int64_t xoff = (row_ok ? r : 0) * p.ld;
         float v[PER];
         float mx = -INFINITY;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             const int64_t c = t + (int64_t)k * LPR;
-            v[k] = (row_ok && c < cv) ? x[c] : -INFINITY;
+            v[k] = (row_ok && c < cv) ? ld_elem<T>(p.logits, xoff + c) : -INFINITY;
             mx = fmaxf(mx, v[k]);
         }
 #pragma unroll
@@ -77,7 +96,7 @@ __global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
             const float prob = v[k] * inv;
             const bool hit = label_ok && c == y;
             if (hit) py = prob;
-            if (row_ok && c < p.C && p.dlogits != nullptr) p.dlogits[r * p.ldd + c] = (prob - (hit ? 1.f : 0.f)) * p.scale;
+            if (row_ok && c < p.C && p.dlogits != nullptr) st_elem<T>(p.dlogits, r * p.ldd + c, (prob - (hit ? 1.f : 0.f)) * p.scale);
         }
 #pragma unroll
         for (int o = LPR / 2; o > 0; o >>= 1) py += __shfl_xor(py, o, 64);  // one lane holds it, the rest 0
@@ -95,6 +114,7 @@ __global__ void __launch_bounds__(256) softmax_xent_kernel(const XentArgs p)
 // coalesced loads, one lane then owns one row (row stride C | 1, so lanes hit distinct banks), and the
 // gradient tile goes back with coalesced stores.  Every lane is busy whatever C is, which the
 // group-per-row kernel above cannot offer for widths like 47.
+template <typename T>
 __global__ void __launch_bounds__(256) softmax_xent_tiled_kernel(const XentArgs p, int R, int CP)
 {
     extern __shared__ float tile[];
@@ -111,7 +131,7 @@ __global__ void __launch_bounds__(256) softmax_xent_tiled_kernel(const XentArgs 
         // stage: element i of the tile is (i / C, i % C); (r, c) advance without divisions
         int r = (int)threadIdx.x / C, c = (int)threadIdx.x % C;
         for (int i = threadIdx.x; i < count; i += 256) {
-            tile[r * CP + c] = p.logits[(row0 + r) * p.ld + c];
+            tile[r * CP + c] = ld_elem<T>(p.logits, (row0 + r) * p.ld + c);
             r += step_r;
             c += step_c;
             if (c >= C) {
@@ -149,7 +169,7 @@ __global__ void __launch_bounds__(256) softmax_xent_tiled_kernel(const XentArgs 
             r = (int)threadIdx.x / C;
             c = (int)threadIdx.x % C;
             for (int i = threadIdx.x; i < count; i += 256) {
-                p.dlogits[(row0 + r) * p.ldd + c] = tile[r * CP + c];
+                st_elem<T>(p.dlogits, (row0 + r) * p.ldd + c, tile[r * CP + c]);
                 r += step_r;
                 c += step_c;
                 if (c >= C) {
@@ -183,20 +203,20 @@ __global__ void __launch_bounds__(256) xent_finish_kernel(const float *__restric
     if (threadIdx.x == 0) *loss = (float)(part[0] * inv_nodes);
 }
 
-template <int LPR>
+template <typename T, int LPR>
 int launch_xent(const XentArgs &a, int per, unsigned blocks, hipStream_t st)
 {
     if constexpr (LPR < 64) {
         if (per != 1) return -1;
-        softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a);
+        softmax_xent_kernel<T, LPR, 1><<<blocks, 256, 0, st>>>(a);
         return 0;
     } else {
         switch (per) {
-            case 1: softmax_xent_kernel<LPR, 1><<<blocks, 256, 0, st>>>(a); return 0;
-            case 2: softmax_xent_kernel<LPR, 2><<<blocks, 256, 0, st>>>(a); return 0;
-            case 4: softmax_xent_kernel<LPR, 4><<<blocks, 256, 0, st>>>(a); return 0;
-            case 8: softmax_xent_kernel<LPR, 8><<<blocks, 256, 0, st>>>(a); return 0;
-            case 16: softmax_xent_kernel<LPR, 16><<<blocks, 256, 0, st>>>(a); return 0;
+            case 1: softmax_xent_kernel<T, LPR, 1><<<blocks, 256, 0, st>>>(a); return 0;
+            case 2: softmax_xent_kernel<T, LPR, 2><<<blocks, 256, 0, st>>>(a); return 0;
+            case 4: softmax_xent_kernel<T, LPR, 4><<<blocks, 256, 0, st>>>(a); return 0;
+            case 8: softmax_xent_kernel<T, LPR, 8><<<blocks, 256, 0, st>>>(a); return 0;
+            case 16: softmax_xent_kernel<T, LPR, 16><<<blocks, 256, 0, st>>>(a); return 0;
             default: return -1;
         }
     }
@@ -213,9 +233,13 @@ size_t plx_softmax_xent_workspace_bytes(int64_t M, int64_t C)
     return (size_t)kXentMaxBlocks * sizeof(float);
 }
 
-int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
-                         int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
-                         float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream)
+}  // extern "C"
+
+namespace {
+template <typename T>
+int softmax_xent_impl(int64_t M, int64_t C, const T *logits, int64_t ld, const int64_t *labels, int64_t num_nodes,
+                      int64_t num_classes, int64_t row_offset, float gscale, float *loss, T *dlogits, int64_t ldd,
+                      void *workspace, size_t workspace_bytes, void *stream)
 {
     PLX_REQUIRE(M >= 0 && C >= 1, "softmax_xent: bad shape M=%lld C=%lld", (long long)M, (long long)C);
     PLX_REQUIRE(C <= 64 * kMaxPerLane, "softmax_xent: at most %d classes are supported, got %lld", 64 * kMaxPerLane,
@@ -253,15 +277,15 @@ int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, 
         const int CP = (int)C | 1;
         const int R = C <= 47 ? 256 : (C <= 95 ? 128 : 64);  // R * CP * 4 <= 49,152 bytes of LDS
         blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, R), kXentMaxBlocks));
-        softmax_xent_tiled_kernel<<<blocks, 256, (size_t)R * CP * sizeof(float), st>>>(a, R, CP);
+        softmax_xent_tiled_kernel<T><<<blocks, 256, (size_t)R * CP * sizeof(float), st>>>(a, R, CP);
         PLX_LAUNCH_CHECK("softmax_xent_tiled_kernel");
     } else {
         const int64_t rows_per_block = 4 * (64 / lpr);
         blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, rows_per_block), kXentMaxBlocks));
         int rc = -1;
         switch (lpr) {
-            case 1: rc = launch_xent<1>(a, per, blocks, st); break;
-            case 64: rc = launch_xent<64>(a, per, blocks, st); break;
+            case 1: rc = launch_xent<T, 1>(a, per, blocks, st); break;
+            case 64: rc = launch_xent<T, 64>(a, per, blocks, st); break;
             default: break;
         }
         if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "softmax_xent: no kernel for C=%lld", (long long)C);
@@ -270,6 +294,26 @@ int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, 
     xent_finish_kernel<<<1, 256, 0, st>>>(a.partials, (int)blocks, 1.0 / (double)num_nodes, loss);
     PLX_LAUNCH_CHECK("xent_finish_kernel");
     return PLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
+                         int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
+                         float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return softmax_xent_impl<float>(M, C, logits, ld, labels, num_nodes, num_classes, row_offset, gscale, loss, dlogits, ldd,
+                                    workspace, workspace_bytes, stream);
+}
+
+int plx_softmax_xent_bf16(int64_t M, int64_t C, const uint16_t *logits, int64_t ld, const int64_t *labels,
+                          int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
+                          uint16_t *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return softmax_xent_impl<uint16_t>(M, C, logits, ld, labels, num_nodes, num_classes, row_offset, gscale, loss, dlogits,
+                                       ldd, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

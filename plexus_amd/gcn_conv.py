@@ -33,7 +33,9 @@ class GCNConvFunction(torch.autograd.Function):
     """Forward and backward of one GCN layer.
 
     Takes the reference's twelve positional inputs (plexus/gcn_conv.py:137-151); the three process
-    groups and the two gather flags are accepted and unused at one rank.  ``fuse_relu`` is an addition.
+    groups and the two gather flags are accepted and unused at one rank.  ``fuse_relu`` and the dropout
+    triple are additions.  The storage type follows ``x``: fp32 (the reference's) or bf16 with fp32
+    accumulation; the weight is always the fp32 parameter.
     """
 
     @staticmethod
@@ -52,11 +54,17 @@ class GCNConvFunction(torch.autograd.Function):
         gather_weights=False,
         layer_num=0,
         fuse_relu=False,
+        dropout_p=0.0,
+        dropout_seed=0,
+        dropout_offset=0,
     ):
         timers = get_timers()
         timers.start("gcn conv fwd")
         A = ops.as_csr(edge_index)
         At = ops.as_csr(edge_index_t)
+        bf16 = x.dtype == torch.bfloat16
+        if dropout_p > 0.0 and not (bf16 and fuse_relu):
+            raise ValueError("fused dropout needs bf16 storage and fuse_relu=True")
 
         # layer-0 features arrive flat (plexus/gcn_conv.py:176-180)
         H = x.detach().reshape(local_features_shape)
@@ -67,7 +75,11 @@ class GCNConvFunction(torch.autograd.Function):
 
         W = weight.detach().reshape(local_weight_shape)
         timers.start("OUT = AGG * W")
-        OUT = ops.gemm_nn(AGG, W, relu=fuse_relu)
+        if bf16:
+            OUT = ops.gemm_nt_bf16(AGG, ops.cast_bf16(W, transpose=True), relu=fuse_relu, dropout_p=dropout_p,
+                                   seed=dropout_seed, offset=dropout_offset)
+        else:
+            OUT = ops.gemm_nn(AGG, W, relu=fuse_relu)
         timers.stop("OUT = AGG * W")
 
         # the reference saves AGG, weight and the transposed adjacency (plexus/gcn_conv.py:194)
@@ -77,6 +89,8 @@ class GCNConvFunction(torch.autograd.Function):
         ctx.x_shape = x.shape
         ctx.layer_num = layer_num
         ctx.fuse_relu = fuse_relu
+        ctx.bf16 = bf16
+        ctx.grad_scale = 1.0 / (1.0 - dropout_p) if dropout_p > 0.0 else 1.0
         timers.stop("gcn conv fwd")
         return OUT
 
@@ -92,13 +106,20 @@ class GCNConvFunction(torch.autograd.Function):
         grad_weight = None
         if ctx.needs_input_grad[3]:
             timers.start("GRAD_W = AGG.T * GRAD_OUT")
-            grad_weight = ops.gemm_tn(agg, grad_output, mask=mask).reshape(weight.shape)
+            if ctx.bf16:
+                grad_weight = ops.gemm_tn_bf16(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
+            else:
+                grad_weight = ops.gemm_tn(agg, grad_output, mask=mask)
+            grad_weight = grad_weight.reshape(weight.shape)
             timers.stop("GRAD_W = AGG.T * GRAD_OUT")
 
         grad_x = None
         if ctx.needs_input_grad[0]:
             timers.start("GRAD_AGG = GRAD_OUT * W.T")
-            grad_agg = ops.gemm_nt(grad_output, W, mask=mask)
+            if ctx.bf16:
+                grad_agg = ops.gemm_nt_bf16(grad_output, ops.cast_bf16(W), mask=mask, alpha=ctx.grad_scale)
+            else:
+                grad_agg = ops.gemm_nt(grad_output, W, mask=mask)
             timers.stop("GRAD_AGG = GRAD_OUT * W.T")
 
             timers.start("GRAD_H = A.T * GRAD_AGG")
@@ -107,7 +128,7 @@ class GCNConvFunction(torch.autograd.Function):
             grad_x = grad_x.reshape(ctx.x_shape)  # flat again for layer 0 (plexus/gcn_conv.py:271)
 
         timers.stop("gcn conv bwd")
-        return (grad_x, None, None, grad_weight) + (None,) * 9
+        return (grad_x, None, None, grad_weight) + (None,) * 12
 
 
 class GCNConv(torch.nn.Module):
@@ -117,9 +138,15 @@ class GCNConv(torch.nn.Module):
     row-major (in, out) matrix, as the reference stores it.  It is drawn with
     ``kaiming_uniform_(a=sqrt(5))`` on an (in, out) tensor (plexus/gcn_conv.py:332-333) -- on the host
     generator, so that a seed reproduces the same weights on any device -- or taken from ``weight``.
+
+    Additions: ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (bf16 storage only) drops
+    activations after the ReLU in training mode with a counter-based generator keyed by ``dropout_seed``;
+    every training forward uses a fresh offset (``layer_num + 64 * call count``).  The storage type
+    follows the input tensor.
     """
 
-    def __init__(self, in_channels, out_channels, layer_num, weight=None, fuse_relu=False, device=None, **kwargs):
+    def __init__(self, in_channels, out_channels, layer_num, weight=None, fuse_relu=False, dropout=0.0, dropout_seed=0,
+                 device=None, **kwargs):
         super().__init__()
         self.layer_num = layer_num
         self.gather_features = layer_num == 0
@@ -130,6 +157,9 @@ class GCNConv(torch.nn.Module):
         self.local_in_channels = self.in_channels
         self.local_out_channels = self.out_channels
         self.fuse_relu = fuse_relu
+        self.dropout = float(dropout)
+        self.dropout_seed = int(dropout_seed)
+        self.forward_calls = 0
         if device is None:
             device = "cuda" if torch.cuda.is_available() else "cpu"
         if weight is None:
@@ -139,8 +169,16 @@ class GCNConv(torch.nn.Module):
             full_weight = torch.as_tensor(weight, dtype=torch.float32).reshape(in_channels, out_channels)
         self.weight = Parameter(full_weight.reshape(-1).clone().to(device), requires_grad=True)
 
+    def next_dropout_offset(self):
+        """Offset the next training forward will use (the oracle regenerates the mask from it)."""
+        return self.layer_num + 64 * self.forward_calls
+
     def forward(self, x, edge_index_shards):
         edge_index, edge_index_t = edge_index_shards[self.layer_num % len(edge_index_shards)]
+        p = self.dropout if self.training else 0.0
+        offset = self.next_dropout_offset()
+        if p > 0.0:
+            self.forward_calls += 1
         return GCNConvFunction.apply(
             x,
             edge_index,
@@ -155,4 +193,7 @@ class GCNConv(torch.nn.Module):
             self.gather_weights,
             self.layer_num,
             self.fuse_relu,
+            p,
+            self.dropout_seed,
+            offset,
         )

@@ -10,7 +10,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from ._lib import PLX_GEMM_RELU, check
+from ._lib import PLX_GEMM_DROPOUT, PLX_GEMM_RELU, check
 
 
 def _stream() -> int:
@@ -231,6 +231,72 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
     return c
 
 
+def cast_bf16(x: torch.Tensor, transpose: bool = False) -> torch.Tensor:
+    """bf16(x) or bf16(x^T) of an fp32 matrix."""
+    _need_gpu(x)
+    x = _rowmajor(x)
+    if x.dtype != torch.float32:
+        raise TypeError("cast_bf16: fp32 input expected")
+    m, n = x.shape
+    y = torch.empty((n, m) if transpose else (m, n), dtype=torch.bfloat16, device=x.device)
+    check(_lib.load().plx_cast_f32_bf16(m, n, x.data_ptr(), _ld(x), y.data_ptr(), _ld(y), int(transpose), _stream()),
+          "plx_cast_f32_bf16")
+    return y
+
+
+def gemm_nt_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0,
+                 relu: bool = False, dropout_p: float = 0.0, seed: int = 0, offset: int = 0) -> torch.Tensor:
+    """bf16 C = epilogue(alpha * (A * [mask > 0]) . B^T), B stored [N x K]; optional ReLU then dropout."""
+    _need_gpu(a, b, mask)
+    a, b = _rowmajor(a), _rowmajor(b)
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise TypeError("gemm_nt_bf16: bf16 operands expected")
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise ValueError("gemm_nt_bf16: inner dimensions differ (%d vs %d)" % (k, k2))
+    if mask is not None:
+        mask = _rowmajor(mask)
+        if mask.shape != a.shape or mask.dtype != torch.bfloat16:
+            raise ValueError("gemm_nt_bf16: mask must be bf16 with the shape of A")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    flags = (PLX_GEMM_RELU if relu else 0) | (PLX_GEMM_DROPOUT if dropout_p > 0.0 else 0)
+    check(
+        _lib.load().plx_gemm_nt_bf16(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                     mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                                     float(alpha), flags, float(dropout_p), int(seed), int(offset), _stream()),
+        "plx_gemm_nt_bf16",
+    )
+    return c
+
+
+def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0) -> torch.Tensor:
+    """fp32 C[K x N] = alpha * A[M x K]^T . (B * [mask > 0])[M x N] from bf16 operands."""
+    _need_gpu(a, b, mask)
+    a, b = _rowmajor(a), _rowmajor(b)
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise TypeError("gemm_tn_bf16: bf16 operands expected")
+    m, k = a.shape
+    m2, n = b.shape
+    if m != m2:
+        raise ValueError("gemm_tn_bf16: row counts differ (%d vs %d)" % (m, m2))
+    if mask is not None:
+        mask = _rowmajor(mask)
+        if mask.shape != b.shape or mask.dtype != torch.bfloat16:
+            raise ValueError("gemm_tn_bf16: mask must be bf16 with the shape of B")
+    lib = _lib.load()
+    c = torch.empty((k, n), dtype=torch.float32, device=a.device)
+    need = int(lib.plx_gemm_tn_bf16_workspace_bytes(m, n, k))
+    ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need else None
+    check(
+        lib.plx_gemm_tn_bf16(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                             mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                             float(alpha), ws.data_ptr() if ws is not None else None, need, _stream()),
+        "plx_gemm_tn_bf16",
+    )
+    return c
+
+
 def relu(x: torch.Tensor) -> torch.Tensor:
     _need_gpu(x)
     x = _rowmajor(x)
@@ -263,16 +329,19 @@ def softmax_xent(logits: torch.Tensor, labels: torch.Tensor, num_nodes: int, num
     if labels.numel() != m:
         raise ValueError("softmax_xent: %d labels for %d rows" % (labels.numel(), m))
     lib = _lib.load()
+    fn = {torch.float32: lib.plx_softmax_xent_f32, torch.bfloat16: lib.plx_softmax_xent_bf16}.get(logits.dtype)
+    if fn is None:
+        raise TypeError("softmax_xent: unsupported dtype %s" % logits.dtype)
     loss = torch.empty(1, dtype=torch.float32, device=logits.device)
-    dlogits = torch.empty((m, c), dtype=torch.float32, device=logits.device) if want_grad else None
+    dlogits = torch.empty((m, c), dtype=logits.dtype, device=logits.device) if want_grad else None
     need = int(lib.plx_softmax_xent_workspace_bytes(m, c))
     ws = torch.empty(need, dtype=torch.uint8, device=logits.device)
     check(
-        lib.plx_softmax_xent_f32(m, c, logits.data_ptr(), _ld(logits), labels.data_ptr(), int(num_nodes),
+        fn(m, c, logits.data_ptr(), _ld(logits), labels.data_ptr(), int(num_nodes),
                                  int(num_classes), int(row_offset), float(gscale), loss.data_ptr(),
                                  dlogits.data_ptr() if want_grad else None, _ld(dlogits) if want_grad else c,
                                  ws.data_ptr(), need, _stream()),
-        "plx_softmax_xent_f32",
+        "plx_softmax_xent",
     )
     return loss, dlogits
 

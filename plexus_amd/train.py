@@ -15,7 +15,8 @@ from .utils.timers import get_timers
 
 
 class Net(torch.nn.Module):
-    def __init__(self, num_gcn_layers, input_size, hidden_size, output_size, weights=None, fuse_relu=True):
+    def __init__(self, num_gcn_layers, input_size, hidden_size, output_size, weights=None, fuse_relu=True, dropout=0.0,
+                 dropout_seed=0):
         super().__init__()
         self.num_gcn_layers = num_gcn_layers
         self.fuse_relu = fuse_relu
@@ -25,7 +26,7 @@ class Net(torch.nn.Module):
             last = i == num_gcn_layers - 1
             self.layers.append(
                 GCNConv(dims[i], dims[i + 1], i, weight=None if weights is None else weights[i],
-                        fuse_relu=fuse_relu and not last)
+                        fuse_relu=fuse_relu and not last, dropout=0.0 if last else dropout, dropout_seed=dropout_seed)
             )
 
     def forward(self, x, edge_index_shards):
@@ -47,12 +48,16 @@ def train(model, optimizer, features_local, adj_shards, labels, num_nodes, num_c
     return loss
 
 
-def make_optimizer(model, features, lr=3e-3, weight_decay=0.0, fused=True):
+def make_optimizer(model, features, lr=3e-3, weight_decay=0.0, fused=True, features_bf16=None):
     """AdamW over the weights and the input features (examples/train.py:155-159).
 
     ``fused`` selects the one-pass kernel of this package; otherwise torch's own optimizer is used.
+    With bf16 storage, ``features`` is the fp32 master copy and ``features_bf16`` the tensor the model
+    reads (its gradient drives the update and it is refreshed by the same kernel).
     """
     params = list(model.parameters()) + [features]
+    if features_bf16 is not None:
+        return AdamW(params, lr=lr, weight_decay=weight_decay, shadows=[(features, features_bf16)])
     if fused:
         return AdamW(params, lr=lr, weight_decay=weight_decay)
     return torch.optim.AdamW(params, lr=lr, weight_decay=weight_decay)

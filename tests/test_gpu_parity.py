@@ -452,3 +452,159 @@ def test_scaled_config4_rank_block_layers():
     assert_parity(x.grad, gx_ref.reshape(k, 64), gx64.reshape(k, 64), what="grad_x")
     for i, layer in enumerate(layers):
         assert_parity(layer.weight.grad, gws_ref[i], gws64[i], what="grad_w[%d]" % i)
+
+
+# ---------------------------------------------------------------------------------------------------
+# bf16 storage with fp32 accumulation; fused dropout
+# ---------------------------------------------------------------------------------------------------
+def bf(t):
+    return t.to(torch.bfloat16)
+
+
+BF16_GEMM_SHAPES = [(1, 1, 1), (5, 3, 2), (127, 16, 33), (128, 32, 64), (300, 47, 256), (1000, 256, 256), (513, 128, 100),
+                    (260, 7, 16), (150, 256, 264), (64, 130, 70)]
+
+
+def test_cast_bf16():
+    say("cast fp32 -> bf16, plain and transposed")
+    gen = torch.Generator().manual_seed(0)
+    for shape in [(1, 1), (33, 7), (256, 256), (100, 47), (5, 300)]:
+        x = torch.randn(*shape, generator=gen)
+        assert torch.equal(ops.cast_bf16(x.to(DEV)).cpu(), bf(x))
+        assert torch.equal(ops.cast_bf16(x.to(DEV), transpose=True).cpu(), bf(x.t().contiguous()))
+
+
+@pytest.mark.parametrize("m,n,k", BF16_GEMM_SHAPES)
+def test_gemm_nt_bf16(m, n, k):
+    say("gemm_nt_bf16 %dx%dx%d" % (m, n, k))
+    gen = torch.Generator().manual_seed(m + 7 * n + k)
+    a = bf(torch.randn(m, k, generator=gen))
+    b = bf(torch.randn(n, k, generator=gen))
+    ref = oracle_c.gemm(a.float().numpy(), b.float().numpy(), tb=True)  # fp64 accumulation of the bf16 inputs
+    c = ops.gemm_nt_bf16(a.to(DEV), b.to(DEV)).float().cpu()
+    assert rel_err(c, ref) <= 2.0 ** -8  # fp32 accumulation: only the final rounding to bf16 is left
+    # ReLU + mask + alpha
+    act = bf(torch.relu(torch.randn(m, k, generator=gen)))
+    cm = ops.gemm_nt_bf16(a.to(DEV), b.to(DEV), mask=act.to(DEV), alpha=2.0, relu=True).float().cpu()
+    refm = np.maximum(2.0 * oracle_c.gemm((a.float() * (act > 0)).numpy(), b.float().numpy(), tb=True), 0)
+    assert rel_err(cm, refm) <= 2.0 ** -8 and (cm >= 0).all()
+
+
+@pytest.mark.parametrize("m,n,k", [(300, 256, 64), (1000, 47, 128), (129, 100, 256), (64, 8, 8)])
+@pytest.mark.parametrize("p", [0.5, 0.25])
+def test_gemm_nt_bf16_dropout_mask_is_the_oracles(m, n, k, p):
+    say("fused dropout %dx%dx%d p=%g" % (m, n, k, p))
+    gen = torch.Generator().manual_seed(m + n)
+    a = bf(torch.rand(m, k, generator=gen) + 0.1)  # positive products: every kept element is > 0
+    b = bf(torch.rand(n, k, generator=gen) + 0.1)
+    seed, offset = 1234567890123, 77
+    c = ops.gemm_nt_bf16(a.to(DEV), b.to(DEV), relu=True, dropout_p=p, seed=seed, offset=offset).float().cpu()
+    keep = torch.from_numpy(po.dropout_keep_mask(m * n, seed, offset, p).reshape(m, n))
+    assert torch.equal(c > 0, keep)  # bit-exact mask
+    assert abs(keep.float().mean().item() - (1 - p)) < 0.02
+    ref = oracle_c.gemm(a.float().numpy(), b.float().numpy(), tb=True) * keep.numpy() / (1 - p)
+    assert rel_err(c, ref) <= 2.0 ** -8
+    # another offset gives another mask
+    c2 = ops.gemm_nt_bf16(a.to(DEV), b.to(DEV), relu=True, dropout_p=p, seed=seed, offset=offset + 1).float().cpu()
+    assert not torch.equal(c2 > 0, keep)
+
+
+@pytest.mark.parametrize("m,n,k", BF16_GEMM_SHAPES + [(70000, 256, 256), (40000, 47, 256)])
+def test_gemm_tn_bf16(m, n, k):
+    say("gemm_tn_bf16 %dx%dx%d" % (m, n, k))
+    gen = torch.Generator().manual_seed(m * 5 + n + k)
+    a = bf(torch.randn(m, k, generator=gen))
+    g = bf(torch.randn(m, n, generator=gen))
+    c = ops.gemm_tn_bf16(a.to(DEV), g.to(DEV)).cpu()
+    assert c.shape == (k, n) and c.dtype == torch.float32
+    ref = oracle_c.gemm(a.float().numpy(), g.float().numpy(), ta=True)
+    err = rel_err(c, ref)
+    print("rel err %.2e" % err, flush=True)
+    assert err <= FP32_TOL  # bf16 products are exact in fp32; only the fp32 summation order differs
+    act = bf(torch.relu(torch.randn(m, n, generator=gen)))
+    cm = ops.gemm_tn_bf16(a.to(DEV), g.to(DEV), mask=act.to(DEV), alpha=2.0).cpu()
+    assert rel_err(cm, 2.0 * oracle_c.gemm(a.float().numpy(), (g.float() * (act > 0)).numpy(), ta=True)) <= FP32_TOL
+    assert torch.equal(c, ops.gemm_tn_bf16(a.to(DEV), g.to(DEV)).cpu())  # bit-reproducible
+
+
+@pytest.mark.parametrize("m,c", [(10, 7), (1000, 47), (257, 100), (50, 1000)])
+def test_softmax_xent_bf16(m, c):
+    say("softmax_xent bf16 %dx%d" % (m, c))
+    gen = torch.Generator().manual_seed(m + c)
+    logits = bf(torch.randn(m, c, generator=gen) * 3)
+    y = torch.randint(0, c, (m,), generator=gen)
+    loss, dl = ops.softmax_xent(logits.to(DEV), y.to(DEV), m, c)
+    assert dl.dtype == torch.bfloat16
+    closs, cgrad = oracle_c.softmax_xent(logits.float().numpy(), y.numpy(), m, c)
+    assert abs(loss.item() - closs) <= FP32_TOL * abs(closs)  # the loss itself is fp32 math on the bf16 logits
+    assert rel_err(dl.float().cpu(), cgrad) <= 2.0 ** -8
+
+
+def test_adamw_bf16_gradient_and_shadow():
+    say("AdamW with bf16 gradient and bf16 shadow")
+    from plexus_amd.optim import AdamW
+
+    gen = torch.Generator().manual_seed(3)
+    n = 10007
+    master0 = torch.randn(n, generator=gen)
+    master = master0.clone().to(DEV)
+    shadow = bf(master).clone().requires_grad_()
+    opt = AdamW([master], lr=3e-3, weight_decay=0.0, shadows=[(master, shadow)])
+    mine = [master0.clone().double()]
+    state = {}
+    for i in range(4):
+        g = bf(torch.randn(n, generator=gen))
+        shadow.grad = g.to(DEV)
+        opt.step()
+        po.adamw_step(mine, [g.double()], state, lr=3e-3)
+        opt.zero_grad()
+        assert shadow.grad is None
+    assert rel_err(master, mine[0]) <= FP32_TOL
+    assert torch.equal(shadow.detach().cpu(), bf(master.cpu()))
+
+
+def test_bf16_three_layer_network_with_dropout():
+    """Wide-hidden bf16 configuration at 1/100 scale: 256-256-256-47, dropout 0.5 after each ReLU,
+    forward, loss and backward against the bf16-storage oracle."""
+    say("config 5 at 1/100 scale: bf16 storage, dropout 0.5")
+    from plexus_amd.cross_entropy import parallel_cross_entropy
+    from plexus_amd.train import Net
+
+    g = S.config3_graph("cpu", seed=1, scale=0.01)
+    n = g.shape[0]
+    dims = [256, 256, 256, 47]
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, dims[0], generator=gen)
+    y = torch.randint(0, 47, (n,), generator=gen)
+    ws = S.glorot_weights(dims, seed=2)
+    seed = 42
+
+    model = Net(3, dims[0], dims[1], dims[-1], weights=ws, fuse_relu=True, dropout=0.5, dropout_seed=seed)
+    model.train()
+    offsets = [layer.next_dropout_offset() for layer in model.layers]
+    shards = [(to_dev(g), to_dev(g, True))]
+    xd = bf(x).to(DEV).requires_grad_()
+    logits = model(xd, shards)
+    loss = parallel_cross_entropy(logits, y.to(DEV), 3, n, 47)
+    loss.backward()
+
+    net = po.OracleNetBf16(ws, dims, dropout_p=0.5, seed=seed)
+    ref_logits = net.forward(x, [(g.torch_csr(), g.torch_csr(True))], offsets)
+    ref_loss, sm, oh = po.cross_entropy_forward(ref_logits, y, n, 47)
+    gl = po.cross_entropy_backward(sm, oh.float(), n)
+    gx_ref, gws_ref = net.backward(gl)
+
+    assert logits.dtype == torch.bfloat16 and xd.grad.dtype == torch.bfloat16
+    assert rel_err(logits.float(), ref_logits) <= BF16_TOL
+    assert abs(loss.item() - ref_loss.item()) <= BF16_TOL * abs(ref_loss.item())
+    assert rel_err(xd.grad.float(), gx_ref.reshape(n, dims[0])) <= BF16_TOL
+    for layer, gw in zip(model.layers, gws_ref):
+        assert layer.weight.grad.dtype == torch.float32
+        assert rel_err(layer.weight.grad, gw) <= BF16_TOL
+    # eval mode: no dropout, deterministic
+    model.eval()
+    e1 = model(xd.detach(), shards)
+    e2 = model(xd.detach(), shards)
+    assert torch.equal(e1, e2)
+    net0 = po.OracleNetBf16(ws, dims, dropout_p=0.0)
+    assert rel_err(e1.float(), net0.forward(x, [(g.torch_csr(), g.torch_csr(True))])) <= BF16_TOL
