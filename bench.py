@@ -62,6 +62,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--spmm-only", action="store_true", help="time only the SpMM kernels")
     ap.add_argument("--spmm-iters", type=int, default=20)
+    ap.add_argument("--config", type=int, default=3, choices=[3, 5],
+                    help="3: fp32, 100-128-128-47 (default, the headline workload); 5: bf16 storage, 256-256-256-47, dropout 0.5")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy (known size) to calibrate profiler byte counters")
     args = ap.parse_args()
@@ -92,7 +94,11 @@ def main():
     torch.cuda.synchronize()
     gen_s = time.time() - t0
     nnz = g.nnz
-    dims = [100, 128, 128, 47]
+    bf16 = args.config == 5
+    dims = [256, 256, 256, 47] if bf16 else [100, 128, 128, 47]
+    dtype = torch.bfloat16 if bf16 else torch.float32
+    elem = 2 if bf16 else 4
+    d_main, d_side = (256, 128) if bf16 else (128, 100)
     print("# graph: %s, long rows %d, segments %d, generated in %.1f s" % (stats, a.n_long_rows, a.n_segments, gen_s),
           file=sys.stderr, flush=True)
 
@@ -106,28 +112,36 @@ def main():
 
     # ---- the dominant kernel: SpMM at D = 128 (and D = 100 beside it) ----
     spmm = {}
-    for d in (128, 100):
-        h = S.normal_features(n, d, dev, seed=d)
-        out = torch.empty(n, d, device=dev)
+    for d in (d_main, d_side):
+        h = S.normal_features(n, d, dev, seed=d, dtype=dtype)
+        out = torch.empty(n, d, device=dev, dtype=dtype)
         ms = time_gpu(lambda: ops.spmm(a, h, out=out), 5, args.spmm_iters)
-        b = spmm_bytes(n, n, nnz, d)
+        b = spmm_bytes(n, n, nnz, d, elem)
         flops = 2.0 * nnz * d
         spmm[d] = {"ms": ms, "alg_bytes": b, "alg_GBps": b / ms / 1e6, "GFLOPs": flops / ms / 1e6,
-                   "gather_GBps": (nnz * 8 + (n + 1) * 4 + nnz * d * 4 + n * d * 4) / ms / 1e6,
+                   "gather_GBps": (nnz * 8 + (n + 1) * 4 + nnz * d * elem + n * d * elem) / ms / 1e6,
                    "t_roof_ms": max(b / (HBM_PEAK_GBPS * 1e6), flops / (FP32_VECTOR_TFLOPS * 1e9))}
-        print("# spmm D=%d: %.3f ms, %.1f GB/s algorithmic, %.1f GFLOP/s" % (d, ms, spmm[d]["alg_GBps"], spmm[d]["GFLOPs"]),
+        print("# spmm D=%d %s: %.3f ms, %.1f GB/s algorithmic, %.1f GFLOP/s" % (d, "bf16" if bf16 else "fp32", ms, spmm[d]["alg_GBps"], spmm[d]["GFLOPs"]),
               file=sys.stderr, flush=True)
         del h, out
-    dom = spmm[128]
+    dom = spmm[d_main]
 
     # ---- the epoch ----
     epoch_ms = None
     losses = []
     if not args.spmm_only:
-        x = S.normal_features(n, dims[0], dev, seed=1).reshape(-1).requires_grad_()
         y = S.uniform_labels(n, dims[-1], dev, seed=2)
-        model = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True)
-        opt = make_optimizer(model, x)
+        if bf16:
+            # fp32 master features for the optimizer, bf16 copy read by the model and refreshed by the update
+            x_master = S.normal_features(n, dims[0], dev, seed=1).reshape(-1)
+            x = x_master.to(torch.bfloat16).requires_grad_()
+            model = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True, dropout=0.5,
+                        dropout_seed=0)
+            opt = make_optimizer(model, x_master, features_bf16=x)
+        else:
+            x = S.normal_features(n, dims[0], dev, seed=1).reshape(-1).requires_grad_()
+            model = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True)
+            opt = make_optimizer(model, x)
         shards = [(a, at)]
         for _ in range(args.warmup):
             losses.append(float(train(model, opt, x, shards, y, n, dims[-1])))
@@ -152,7 +166,7 @@ def main():
         from oracle import plexus_oracle as po
 
         a_cpu = torch.sparse_csr_tensor(g.rowptr.cpu(), g.col.cpu(), g.val.cpu(), size=g.shape)
-        h_cpu = S.normal_features(n, 128, dev, seed=128).cpu()
+        h_cpu = S.normal_features(n, d_main, dev, seed=d_main, dtype=dtype).float().cpu()  # bf16 config: fp32 math on bf16-rounded inputs
         po.spmm(a_cpu, h_cpu)  # warm-up
         reps = 2
         t2 = time.time()
@@ -160,11 +174,11 @@ def main():
             y_cpu = po.spmm(a_cpu, h_cpu)
         cpu_s = (time.time() - t2) / reps
         # the same product on the GPU must agree with it
-        y_gpu = ops.spmm(a, h_cpu.to(dev)).cpu()
+        y_gpu = ops.spmm(a, h_cpu.to(dev).to(dtype)).float().cpu()
         err = ((y_gpu.double() - y_cpu.double()).abs().max() / y_cpu.double().abs().max()).item()
         cpu = {"value": dom["alg_bytes"] / cpu_s / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": "the whole SpMM A.H of the workload at D=128 (torch.sparse.mm, fp32, %d timed runs)" % reps,
-               "ms": cpu_s * 1e3, "GFLOPs": 2.0 * nnz * 128 / cpu_s / 1e9, "host_cpus": os.cpu_count(),
+               "sample": "the whole SpMM A.H of the workload at D=%d (torch.sparse.mm, fp32, %d timed runs)" % (d_main, reps),
+               "ms": cpu_s * 1e3, "GFLOPs": 2.0 * nnz * d_main / cpu_s / 1e9, "host_cpus": os.cpu_count(),
                "max_rel_err_gpu_vs_cpu": err}
         print("# cpu: %.1f ms per SpMM on %d threads, gpu-vs-cpu max rel err %.2e" % (cpu_s * 1e3, cpu["cores"], err),
               file=sys.stderr, flush=True)
@@ -180,23 +194,26 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16" if bf16 else "f32",
         "data": "synthetic",
-        "config": {"workload": "config 3: 3-layer GCN 100-128-128-47 on a Chung-Lu(2.1) graph, N=%d, nnz=%d "
-                               "(value = SpMM A.H at D=128; step = one training epoch incl. AdamW)" % (n, nnz),
+        "config": {"workload": "config %d: 3-layer GCN %s on a Chung-Lu(2.1) graph, N=%d, nnz=%d "
+                               "(value = SpMM A.H at D=%d; step = one training epoch incl. AdamW%s)"
+                               % (args.config, "-".join(str(d) for d in dims), n, nnz, d_main,
+                                  ", bf16 storage, fp32 accumulate, dropout 0.5" if bf16 else ""),
                    "nodes": n, "nnz": nnz, "max_row_nnz": stats["max_row_nnz"], "scale": args.scale,
                    "split_rows": a.n_long_rows, "segments": a.n_segments},
         "spmm_ms": dom["ms"],
         "spmm_pct_of_hbm_peak": 100.0 * dom["alg_GBps"] / HBM_PEAK_GBPS,
         "spmm_GFLOPs": dom["GFLOPs"],
         "spmm_gather_model_GBps": dom["gather_GBps"],
-        "spmm_D100": spmm[100],
+        "spmm_D%d" % d_side: spmm[d_side],
         "epoch_ms": epoch_ms,
         "loss_first_last": [losses[0], losses[-1]] if losses else None,
         "roofline": {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": dom["alg_GBps"] / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_SPMM_TRAFFIC_BYTES.get((n, nnz, 128)),
-                     "kernel": "spmm_csr_kernel (A.H, D=128)", "alg_bytes_per_launch": dom["alg_bytes"],
+                     "traffic": None if bf16 else MEASURED_SPMM_TRAFFIC_BYTES.get((n, nnz, 128)),
+                     "kernel": "spmm_csr_kernel (A.H, D=%d, %s)" % (d_main, "bf16" if bf16 else "fp32"),
+                     "alg_bytes_per_launch": dom["alg_bytes"],
                      "avg_launch_ms": dom["ms"]},
         "cpu_baseline": cpu,
     }

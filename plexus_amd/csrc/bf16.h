@@ -19,7 +19,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16(float f)
     return u >> 16;
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f32_to_bf16(lo) | (f32_to_bf16(hi) << 16); }
+// two fp32 -> packed bf16 pair with the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even)
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const float2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
 // true where the bf16 value is > 0 (positive sign, non-zero magnitude)
 __device__ __forceinline__ bool bf16_positive(uint32_t bits16) { return (bits16 & 0x8000u) == 0 && (bits16 & 0x7fffu) != 0; }

@@ -77,14 +77,19 @@ __device__ __forceinline__ uint4 mask8(uint4 v, uint4 m) { return make_uint4(mas
 // ------------------------------------------------------------------------------------------------
 // NT: C = epilogue(alpha * (A*mask) . B^T), A [M x K], B [N x K], both contraction-contiguous
 // ------------------------------------------------------------------------------------------------
-template <int TN, bool MASKED>
+// VEC: every operand is 16-byte aligned with a leading dimension that is a multiple of 8 and K % 8 == 0,
+// so a tile is made of whole 16-byte vectors: no element-wise paths, and addressing is one 64-bit
+// multiply per thread and tile plus pointer steps (address arithmetic per vector would otherwise cost more
+// vector-ALU time than the MFMAs take).
+template <int TN, bool MASKED, bool VEC>
 __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g)
 {
     constexpr int BN = 32 * TN;
-    constexpr int kAVec = kBM * kBK / 8 / kThreads;                       // 16-byte vectors per thread, A tile
+    constexpr int kAVec = kBM * kBK / 8 / kThreads;                       // 16-byte vectors per thread and chunk, A tile
     constexpr int kBVec = (BN * kBK / 8 + kThreads - 1) / kThreads;       // B tile
     constexpr int kTile = (kBM + BN) * kS;                                // bf16 elements per buffer
     constexpr int kCS = BN + 4;                                           // fp32 row stride of the staged output
+    constexpr int kAhead = 4;                                             // chunks of A fetched in one go
     static_assert(4 * 32 * kCS * 4 <= 2 * kTile * 2, "staged output must fit the operand buffers");
 
     __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kTile];
@@ -93,47 +98,74 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
     const int wave = threadIdx.x >> 6;
     const int li = lane & 31;
     const int h = lane >> 5;
-    const int64_t row0 = (int64_t)blockIdx.x * kBM;
-    const int64_t col0 = (int64_t)blockIdx.y * BN;
 
-    uint4 ra[kAVec], rb[kBVec];
-    auto fetch = [&](int64_t k0) {
+    // Workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with
+    // its own L2; the column tiles of one row panel are therefore given to consecutive workgroups of the
+    // SAME XCD (ids b, b + 8, ...), so that the row panel of A is read from HBM once and from that L2 after.
+    const int64_t n_ct = (g.N + BN - 1) / BN;
+    const int64_t n_rp = (g.M + kBM - 1) / kBM;
+    const int64_t bid = blockIdx.x;
+    const int64_t xcd = bid % 8, slot = bid / 8;
+    const int64_t rp = (slot / n_ct) * 8 + xcd;
+    if (rp >= n_rp) return;
+    const int64_t row0 = rp * kBM;
+    const int64_t col0 = (slot % n_ct) * BN;
+
+    // thread (rt, kq) owns vector kq of rows rt, rt + 32, ... of a tile
+    const int rt = threadIdx.x >> 3;
+    const int kq = threadIdx.x & 7;
+    const uint16_t *pa = g.A + (row0 + rt) * g.lda + kq * 8;
+    const uint16_t *pm = MASKED ? g.mask + (row0 + rt) * g.ldmask + kq * 8 : nullptr;
+    const uint16_t *pb = g.B + (col0 + rt) * g.ldb + kq * 8;
+    const int a_rows = (int)min(max(g.M - row0 - rt, (int64_t)0), (int64_t)kBM);  // rows rt + 32 p with 32 p < a_rows exist
+    const int b_rows = (int)min(max(g.N - col0 - rt, (int64_t)0), (int64_t)BN);
+    const int K = (int)g.K;
+
+    // A is bound by HBM latency, not by the matrix cores (one chunk is 16 MFMAs): all loads of up to
+    // kAhead chunks are issued back to back before the first one is consumed.  B (the weight) comes from
+    // L2 and keeps the usual one-chunk-ahead prefetch.
+    uint4 ra[kAhead][kAVec], rb[kBVec];
+    auto fetch_a = [&](int k0, uint4(&dst)[kAVec]) {
+        const int k = k0 + kq * 8;
 #pragma unroll
         for (int p = 0; p < kAVec; ++p) {
-            const int idx = p * kThreads + threadIdx.x;
-            const int64_t r = row0 + idx / 8;
-            const int64_t k = k0 + (idx % 8) * 8;
             uint4 v = zero4();
-            if (r < g.M && k < g.K) {
-                const int valid = (int)min((int64_t)8, g.K - k);
-                v = load8(g.A + r * g.lda + k, valid, g.a_vec);
-                if constexpr (MASKED) v = mask8(v, load8(g.mask + r * g.ldmask + k, valid, g.m_vec));
+            if (32 * p < a_rows && k < K) {
+                if constexpr (VEC) {
+                    v = *reinterpret_cast<const uint4 *>(pa + (int64_t)(32 * p) * g.lda + k0);
+                    if constexpr (MASKED) v = mask8(v, *reinterpret_cast<const uint4 *>(pm + (int64_t)(32 * p) * g.ldmask + k0));
+                } else {
+                    const int valid = min(8, K - k);
+                    v = load8(pa + (int64_t)(32 * p) * g.lda + k0, valid, g.a_vec);
+                    if constexpr (MASKED) v = mask8(v, load8(pm + (int64_t)(32 * p) * g.ldmask + k0, valid, g.m_vec));
+                }
             }
-            ra[p] = v;
+            dst[p] = v;
         }
+    };
+    auto fetch_b = [&](int k0) {
+        const int k = k0 + kq * 8;
 #pragma unroll
         for (int p = 0; p < kBVec; ++p) {
-            const int idx = p * kThreads + threadIdx.x;
-            const int64_t n = col0 + idx / 8;
-            const int64_t k = k0 + (idx % 8) * 8;
             uint4 v = zero4();
-            if (idx < BN * 8 && n < g.N && k < g.K) v = load8(g.B + n * g.ldb + k, (int)min((int64_t)8, g.K - k), g.b_vec);
+            if (32 * p < b_rows && k < K) {
+                if constexpr (VEC)
+                    v = *reinterpret_cast<const uint4 *>(pb + (int64_t)(32 * p) * g.ldb + k0);
+                else
+                    v = load8(pb + (int64_t)(32 * p) * g.ldb + k0, min(8, K - k), g.b_vec);
+            }
             rb[p] = v;
         }
     };
-    auto stash = [&](int buf) {
-        uint16_t *as = lds + buf * kTile;
+    const int st_off = rt * kS + kq * 8;
+    auto stash = [&](int buf, const uint4(&a)[kAVec]) {
+        uint16_t *as = lds + buf * kTile + st_off;
         uint16_t *bs = as + kBM * kS;
 #pragma unroll
-        for (int p = 0; p < kAVec; ++p) {
-            const int idx = p * kThreads + threadIdx.x;
-            *reinterpret_cast<uint4 *>(as + (idx / 8) * kS + (idx % 8) * 8) = ra[p];
-        }
+        for (int p = 0; p < kAVec; ++p) *reinterpret_cast<uint4 *>(as + 32 * p * kS) = a[p];
 #pragma unroll
-        for (int p = 0; p < kBVec; ++p) {
-            const int idx = p * kThreads + threadIdx.x;
-            if (idx < BN * 8) *reinterpret_cast<uint4 *>(bs + (idx / 8) * kS + (idx % 8) * 8) = rb[p];
-        }
+        for (int p = 0; p < kBVec; ++p)
+            if (32 * p < BN) *reinterpret_cast<uint4 *>(bs + 32 * p * kS) = rb[p];
     };
 
     floatx16 acc[TN];
@@ -143,28 +175,33 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
         for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
     int buf = 0;
-    if (g.K > 0) {
-        fetch(0);
-        stash(0);
-    }
-    __syncthreads();
-    for (int64_t k0 = 0; k0 < g.K; k0 += kBK) {
-        const bool more = k0 + kBK < g.K;
-        if (more) fetch(k0 + kBK);
-        const uint16_t *as = lds + buf * kTile;
-        const uint16_t *bs = as + kBM * kS;
+    for (int kk = 0; kk < K; kk += kAhead * kBK) {
 #pragma unroll
-        for (int s = 0; s < kBK / 16; ++s) {
-            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(as + (wave * 32 + li) * kS + 16 * s + 8 * h);
-#pragma unroll
-            for (int t = 0; t < TN; ++t) {
-                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(bs + (t * 32 + li) * kS + 16 * s + 8 * h);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
-            }
-        }
-        if (more) stash(buf ^ 1);
+        for (int c = 0; c < kAhead; ++c) fetch_a(kk + c * kBK, ra[c]);  // chunks past K come back as zeros
+        fetch_b(kk);
+        stash(buf, ra[0]);
         __syncthreads();
-        buf ^= 1;
+#pragma unroll
+        for (int c = 0; c < kAhead; ++c) {
+            const int k0 = kk + c * kBK;
+            if (k0 >= K) break;
+            const bool more = (c + 1 < kAhead) && (k0 + kBK < K);
+            if (more) fetch_b(k0 + kBK);
+            const uint16_t *as = lds + buf * kTile;
+            const uint16_t *bs = as + kBM * kS;
+#pragma unroll
+            for (int s = 0; s < kBK / 16; ++s) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8 *>(as + (wave * 32 + li) * kS + 16 * s + 8 * h);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(bs + (t * 32 + li) * kS + 16 * s + 8 * h);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+                }
+            }
+            if (more) stash(buf ^ 1, ra[(c + 1) % kAhead]);
+            __syncthreads();
+            buf ^= 1;
+        }
     }
 
     // stage the wavefront's 32 x BN fp32 tile in LDS (register v of a lane is row 8 (v / 4) + 4 h + v % 4,
@@ -226,7 +263,7 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
 // ------------------------------------------------------------------------------------------------
 // TN: C[K x N] (fp32) = alpha * A[M x K]^T . (B*mask)[M x N]; contraction over the rows of both
 // ------------------------------------------------------------------------------------------------
-template <int TN, bool MASKED>
+template <int TN, bool MASKED, bool VEC>
 __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g)
 {
     constexpr int BN = 32 * TN;
@@ -245,38 +282,54 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
     const int64_t mbeg = (int64_t)blockIdx.x * g.rows_per_split;
     const int64_t mend = min(mbeg + g.rows_per_split, g.M);
 
+    // thread (mp, cq0) owns the row pair (2 mp, 2 mp + 1) and the column vectors cq0, cq0 + 8, ... of a chunk;
+    // pointers walk down the rows chunk by chunk, so a fetch costs pointer steps and 32-bit compares only
+    const int mp = threadIdx.x & 31;
+    const int cq0 = threadIdx.x >> 5;
+    const uint16_t *pa = g.A + (mbeg + 2 * mp) * g.lda + row0 + cq0 * 8;
+    const uint16_t *pb = g.B + (mbeg + 2 * mp) * g.ldb + col0 + cq0 * 8;
+    const uint16_t *pm = MASKED ? g.mask + (mbeg + 2 * mp) * g.ldmask + col0 + cq0 * 8 : nullptr;
+    const int a_cols = (int)min(max(g.K - row0 - cq0 * 8, (int64_t)0), (int64_t)kBM);  // columns 64 p + e with 64 p + e < a_cols exist
+    const int b_cols = (int)min(max(g.N - col0 - cq0 * 8, (int64_t)0), (int64_t)BN);
+
     uint4 ra[kAItems][2], rb[kBItems][2];
     auto fetch = [&](int64_t m0) {
+        const int rows_left = (int)min(mend - m0 - 2 * mp, (int64_t)2);  // 2: both rows of the pair exist
 #pragma unroll
         for (int p = 0; p < kAItems; ++p) {
-            const int item = p * kThreads + threadIdx.x;
-            const int mp = item % 32, cq = item / 32;
-            const int64_t c = row0 + cq * 8;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int64_t m = m0 + 2 * mp + j;
                 uint4 v = zero4();
-                if (m < mend && c < g.K) v = load8(g.A + m * g.lda + c, (int)min((int64_t)8, g.K - c), g.a_vec);
+                if (j < rows_left && 64 * p < a_cols) {
+                    if constexpr (VEC)
+                        v = *reinterpret_cast<const uint4 *>(pa + j * g.lda + 64 * p);
+                    else
+                        v = load8(pa + j * g.lda + 64 * p, min(8, a_cols - 64 * p), g.a_vec);
+                }
                 ra[p][j] = v;
             }
         }
 #pragma unroll
         for (int p = 0; p < kBItems; ++p) {
-            const int item = p * kThreads + threadIdx.x;
-            const int mp = item % 32, cq = item / 32;
-            const int64_t c = col0 + cq * 8;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int64_t m = m0 + 2 * mp + j;
                 uint4 v = zero4();
-                if (cq < BN / 8 && m < mend && c < g.N) {
-                    const int valid = (int)min((int64_t)8, g.N - c);
-                    v = load8(g.B + m * g.ldb + c, valid, g.b_vec);
-                    if constexpr (MASKED) v = mask8(v, load8(g.mask + m * g.ldmask + c, valid, g.m_vec));
+                if (j < rows_left && 64 * p < b_cols && 64 * p + cq0 * 8 < BN) {
+                    if constexpr (VEC) {
+                        v = *reinterpret_cast<const uint4 *>(pb + j * g.ldb + 64 * p);
+                        if constexpr (MASKED) v = mask8(v, *reinterpret_cast<const uint4 *>(pm + j * g.ldmask + 64 * p));
+                    } else {
+                        const int valid = min(8, b_cols - 64 * p);
+                        v = load8(pb + j * g.ldb + 64 * p, valid, g.b_vec);
+                        if constexpr (MASKED) v = mask8(v, load8(pm + j * g.ldmask + 64 * p, valid, g.m_vec));
+                    }
                 }
                 rb[p][j] = v;
             }
         }
+        pa += (int64_t)kBK * g.lda;
+        pb += (int64_t)kBK * g.ldb;
+        if constexpr (MASKED) pm += (int64_t)kBK * g.ldmask;
     };
     // transposed stash: word e of the pair holds (row 2 mp, row 2 mp + 1) of column 8 cq + e
     auto stash_pair = [&](uint16_t *t, int mp, int cq, const uint4 &r0, const uint4 &r1) {
@@ -293,15 +346,10 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
         uint16_t *at = lds + buf * kTile;
         uint16_t *bt = at + kBM * kS;
 #pragma unroll
-        for (int p = 0; p < kAItems; ++p) {
-            const int item = p * kThreads + threadIdx.x;
-            stash_pair(at, item % 32, item / 32, ra[p][0], ra[p][1]);
-        }
+        for (int p = 0; p < kAItems; ++p) stash_pair(at, mp, cq0 + 8 * p, ra[p][0], ra[p][1]);
 #pragma unroll
-        for (int p = 0; p < kBItems; ++p) {
-            const int item = p * kThreads + threadIdx.x;
-            if (item / 32 < BN / 8) stash_pair(bt, item % 32, item / 32, rb[p][0], rb[p][1]);
-        }
+        for (int p = 0; p < kBItems; ++p)
+            if (cq0 + 8 * p < BN / 8) stash_pair(bt, mp, cq0 + 8 * p, rb[p][0], rb[p][1]);
     };
 
     floatx16 acc[TN];
@@ -416,23 +464,23 @@ int64_t tn_splits(int64_t M, int64_t N, int64_t K)
     return std::max<int64_t>(1, std::min(want, by_rows));
 }
 
-template <bool MASKED>
+template <bool MASKED, bool VEC>
 void launch_nt(const Bf16Args &g, int tn, dim3 grid, hipStream_t st)
 {
     switch (tn) {
-        case 1: gemm_bf16_nt_kernel<1, MASKED><<<grid, kThreads, 0, st>>>(g); break;
-        case 2: gemm_bf16_nt_kernel<2, MASKED><<<grid, kThreads, 0, st>>>(g); break;
-        default: gemm_bf16_nt_kernel<4, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        case 1: gemm_bf16_nt_kernel<1, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_bf16_nt_kernel<2, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_bf16_nt_kernel<4, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
     }
 }
 
-template <bool MASKED>
+template <bool MASKED, bool VEC>
 void launch_tn(const Bf16Args &g, int tn, dim3 grid, hipStream_t st)
 {
     switch (tn) {
-        case 1: gemm_bf16_tn_kernel<1, MASKED><<<grid, kThreads, 0, st>>>(g); break;
-        case 2: gemm_bf16_tn_kernel<2, MASKED><<<grid, kThreads, 0, st>>>(g); break;
-        default: gemm_bf16_tn_kernel<4, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        case 1: gemm_bf16_tn_kernel<1, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_bf16_tn_kernel<2, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_bf16_tn_kernel<4, MASKED, VEC><<<grid, kThreads, 0, st>>>(g); break;
     }
 }
 
@@ -446,6 +494,7 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
 {
     PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_bf16: negative dimension");
     PLX_REQUIRE(N < (1ll << 30) && K < (1ll << 30), "gemm_nt_bf16: dimension too large");
+    PLX_REQUIRE(M < (1ll << 40), "gemm_nt_bf16: too many rows");
     if (M == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(C != nullptr, "gemm_nt_bf16: NULL output");
     PLX_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "gemm_nt_bf16: NULL operand");
@@ -464,9 +513,20 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     g.off_lo = (uint32_t)offset; g.off_hi = (uint32_t)(offset >> 32);
     g.a_vec = vec16(A, lda); g.b_vec = vec16(B, ldb); g.c_vec = vec16(C, ldc); g.m_vec = vec16(mask, ldmask);
     const int tn = pick_tn(N);
-    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
-    if (mask != nullptr) launch_nt<true>(g, tn, grid, plx::as_stream(stream));
-    else launch_nt<false>(g, tn, grid, plx::as_stream(stream));
+    // one workgroup per (row panel, column tile); row panels are rounded up to a multiple of 8 for the XCD mapping
+    const int64_t n_ct = plx::ceil_div(N, 32 * tn);
+    const int64_t blocks = plx::ceil_div(plx::ceil_div(M, kBM), 8) * 8 * n_ct;
+    PLX_REQUIRE(blocks < (1ll << 31), "gemm_nt_bf16: too many tiles");
+    dim3 grid((unsigned)blocks, 1, 1);
+    const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0;
+    hipStream_t st = plx::as_stream(stream);
+    if (mask != nullptr) {
+        if (vec) launch_nt<true, true>(g, tn, grid, st);
+        else launch_nt<true, false>(g, tn, grid, st);
+    } else {
+        if (vec) launch_nt<false, true>(g, tn, grid, st);
+        else launch_nt<false, false>(g, tn, grid, st);
+    }
     PLX_LAUNCH_CHECK("gemm_bf16_nt_kernel");
     return PLX_OK;
 }
@@ -509,8 +569,14 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     }
     const int tn = pick_tn(N);
     dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
-    if (mask != nullptr) launch_tn<true>(g, tn, grid, st);
-    else launch_tn<false>(g, tn, grid, st);
+    const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0 && N % 8 == 0;
+    if (mask != nullptr) {
+        if (vec) launch_tn<true, true>(g, tn, grid, st);
+        else launch_tn<true, false>(g, tn, grid, st);
+    } else {
+        if (vec) launch_tn<false, true>(g, tn, grid, st);
+        else launch_tn<false, false>(g, tn, grid, st);
+    }
     PLX_LAUNCH_CHECK("gemm_bf16_tn_kernel");
     if (splits > 1) {
         gemm_bf16_tn_reduce<<<(unsigned)plx::ceil_div(K * N, 64), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, alpha, C, ldc);

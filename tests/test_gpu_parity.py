@@ -321,11 +321,12 @@ def test_config1_ten_epoch_loss_curve(fuse_relu):
         assert rel_err(layer.weight, w) <= 1e-4
 
 
-def test_scaled_config3_properties_and_sampled_rows():
-    """A tenth of the 2.45 M-node power-law configuration: size-independent properties of the SpMM
-    and a comparison of sampled rows against the fp64-accumulating oracle."""
-    say("config 3 at 1/10 scale: properties")
-    g = S.config3_graph(DEV, seed=0, scale=0.1)
+@pytest.mark.parametrize("scale", [0.1, 1.0])
+def test_config3_properties_and_sampled_rows(scale):
+    """The 2.45 M-node power-law configuration (full size and a tenth of it): size-independent
+    properties of the SpMM and a comparison of sampled rows against the fp64-accumulating oracle."""
+    say("config 3 at scale %g: properties" % scale)
+    g = S.config3_graph(DEV, seed=0, scale=scale)
     n = g.shape[0]
     a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
     at = ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (n, n))
@@ -351,11 +352,12 @@ def test_scaled_config3_properties_and_sampled_rows():
     deg = (g.rowptr[1:] - g.rowptr[:-1]).cpu()
     pick = torch.cat([torch.topk(deg, 8).indices, torch.topk(-deg, 8).indices,
                       torch.randint(0, n, (200,), generator=torch.Generator().manual_seed(0))])
-    rp, ci, va = g.rowptr.cpu(), g.col.cpu(), g.val.cpu()
     sub_counts = deg[pick]
     sub_rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(sub_counts, 0)])
-    idx = torch.cat([torch.arange(rp[r], rp[r + 1]) for r in pick.tolist()])
-    ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci[idx].numpy(), va[idx].numpy(), h.cpu().numpy())
+    starts = g.rowptr[pick.to(DEV)]
+    idx = torch.repeat_interleave(starts - sub_rowptr[:-1].to(DEV), sub_counts.to(DEV)) + torch.arange(int(sub_rowptr[-1]), device=DEV)
+    ci, va = g.col[idx].cpu(), g.val[idx].cpu()  # only the sampled rows leave the device
+    ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci.numpy(), va.numpy(), h.cpu().numpy())
     assert rel_err(y[pick.to(DEV)].cpu(), ref) <= FP32_TOL
 
 
@@ -608,3 +610,28 @@ def test_bf16_three_layer_network_with_dropout():
     assert torch.equal(e1, e2)
     net0 = po.OracleNetBf16(ws, dims, dropout_p=0.0)
     assert rel_err(e1.float(), net0.forward(x, [(g.torch_csr(), g.torch_csr(True))])) <= BF16_TOL
+
+
+def test_internal_timers_use_the_reference_names():
+    say("timers")
+    import plexus_amd
+    from plexus_amd.gcn_conv import GCNConv
+    from plexus_amd.cross_entropy import parallel_cross_entropy
+    from plexus_amd.utils.timers import get_timers
+
+    plexus_amd.init(enable_internal_timers=True)
+    try:
+        get_timers().reset()
+        g = graph_small(n=300, pairs=2000, seed=1)
+        layer = GCNConv(12, 5, 0)
+        x = torch.randn(300 * 12, device=DEV, requires_grad=True)
+        y = torch.randint(0, 5, (300,), device=DEV)
+        loss = parallel_cross_entropy(layer(x, [(to_dev(g), to_dev(g, True))]), y, 1, 300, 5)
+        loss.backward()
+        times = get_timers().get_times()
+        for name in ["gcn conv fwd", "AGG = A * H", "OUT = AGG * W", "gcn conv bwd", "GRAD_W = AGG.T * GRAD_OUT",
+                     "GRAD_AGG = GRAD_OUT * W.T", "GRAD_H = A.T * GRAD_AGG", "cross entropy fwd", "cross entropy bwd"]:
+            assert name in times and times[name] >= 0.0
+    finally:
+        plexus_amd.init()
+        get_timers().reset()
