@@ -24,6 +24,10 @@
 
 #include "common.h"
 
+#ifndef PLX_GEMM_LEAN
+#define PLX_GEMM_LEAN 1  // 0: always use the general kernel (for A/B timing)
+#endif
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -259,6 +263,230 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Lean variant for aligned operands (every base 16-byte aligned, every leading dimension and the
+// contraction / column extents multiples of 4).  Same tiling and LDS layouts as gemm_f32_kernel; the
+// difference is the cost of a fetch: one 64-bit multiply per thread and tile, then pointer steps and
+// 32-bit compares.  In the general kernel the per-element guards and 64-bit address products amount to
+// ~8 vector-ALU instructions per MFMA, which is what keeps its MFMA pipe half idle.
+// ---------------------------------------------------------------------------------------------------
+template <int MODE, int TN, bool MASKED>
+__global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr bool kAX = (MODE != kTN);
+    constexpr bool kBX = (MODE == kNT);
+    constexpr int kAStride = kAX ? kXS : kBM;
+    constexpr int kBStride = kBX ? kXS : BN;
+    constexpr int kASize = kAX ? kBM * kXS : kBK * kBM;
+    constexpr int kBSize = kBX ? BN * kXS : kBK * BN;
+    // float4 per tile row and rows covered by one pass of the 256 threads
+    constexpr int kAV = (kAX ? kBK : kBM) / 4, kARows = kAX ? kBM : kBK, kAPass = kThreads / kAV;
+    constexpr int kBV = (kBX ? kBK : BN) / 4, kBRows = kBX ? BN : kBK, kBPass = kThreads / kBV;
+    constexpr int kAPer = (kARows + kAPass - 1) / kAPass, kBPer = (kBRows + kBPass - 1) / kBPass;
+
+    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+
+    int64_t row0, col0, kbeg, kend;
+    if constexpr (MODE == kTN) {
+        row0 = (int64_t)blockIdx.y * kBM;
+        col0 = (int64_t)blockIdx.z * BN;
+        kbeg = (int64_t)blockIdx.x * g.rows_per_split;
+        kend = min(kbeg + g.rows_per_split, g.M);
+    } else {
+        row0 = (int64_t)blockIdx.x * kBM;
+        col0 = (int64_t)blockIdx.y * BN;
+        kbeg = 0;
+        kend = g.K;
+    }
+
+    // thread coordinates inside the A and B tiles: (row of the first pass, float4 index in the row)
+    const int ar = threadIdx.x / kAV, av = (threadIdx.x % kAV) * 4;
+    const int br = threadIdx.x / kBV, bv = (threadIdx.x % kBV) * 4;
+    // source row / column of element (0, 0) of each tile at contraction offset kbeg, and the extents left
+    const float *pa, *pb, *pm = nullptr;
+    int64_t a_step, b_step, m_step = 0;  // pointer advance per pass (rows of the tile)
+    int64_t a_adv, b_adv, m_adv = 0;     // pointer advance per chunk
+    int a_rows_left, a_cols_left, b_rows_left, b_cols_left;  // relative to this thread's first element
+    if constexpr (MODE == kNN) {
+        pa = g.A + (row0 + ar) * g.lda + av;             a_step = (int64_t)kAPass * g.lda; a_adv = kBK;
+        pb = g.B + (int64_t)br * g.ldb + col0 + bv;      b_step = (int64_t)kBPass * g.ldb; b_adv = (int64_t)kBK * g.ldb;
+        a_rows_left = (int)min(max(g.M - row0 - ar, (int64_t)0), (int64_t)kBM);  a_cols_left = (int)min(g.K - av, (int64_t)1 << 30);
+        b_rows_left = (int)min(g.K - br, (int64_t)1 << 30);                       b_cols_left = (int)min(max(g.N - col0 - bv, (int64_t)0), (int64_t)BN);
+    } else if constexpr (MODE == kNT) {
+        pa = g.A + (row0 + ar) * g.lda + av;             a_step = (int64_t)kAPass * g.lda; a_adv = kBK;
+        if constexpr (MASKED) { pm = g.mask + (row0 + ar) * g.ldmask + av; m_step = (int64_t)kAPass * g.ldmask; m_adv = kBK; }
+        pb = g.B + (col0 + br) * g.ldb + bv;             b_step = (int64_t)kBPass * g.ldb; b_adv = kBK;
+        a_rows_left = (int)min(max(g.M - row0 - ar, (int64_t)0), (int64_t)kBM);  a_cols_left = (int)min(g.K - av, (int64_t)1 << 30);
+        b_rows_left = (int)min(max(g.N - col0 - br, (int64_t)0), (int64_t)BN);   b_cols_left = (int)min(g.K - bv, (int64_t)1 << 30);
+    } else {
+        pa = g.A + (kbeg + ar) * g.lda + row0 + av;      a_step = (int64_t)kAPass * g.lda; a_adv = (int64_t)kBK * g.lda;
+        pb = g.B + (kbeg + br) * g.ldb + col0 + bv;      b_step = (int64_t)kBPass * g.ldb; b_adv = (int64_t)kBK * g.ldb;
+        if constexpr (MASKED) { pm = g.mask + (kbeg + br) * g.ldmask + col0 + bv; m_step = (int64_t)kBPass * g.ldmask; m_adv = (int64_t)kBK * g.ldmask; }
+        a_rows_left = (int)min(kend - kbeg - ar, (int64_t)1 << 30);  a_cols_left = (int)min(max(g.K - row0 - av, (int64_t)0), (int64_t)kBM);
+        b_rows_left = (int)min(kend - kbeg - br, (int64_t)1 << 30);  b_cols_left = (int)min(max(g.N - col0 - bv, (int64_t)0), (int64_t)BN);
+    }
+    // which of (rows, cols) shrinks as the contraction advances
+    constexpr bool kAContrRows = (MODE == kTN);            // A tile rows are contraction indices (k-major)
+    constexpr bool kBContrRows = (MODE != kNT);            // B tile rows are contraction indices
+
+    float4 ra[kAPer], rb[kBPer];
+    auto fetch = [&]() {
+        {
+            const float *q = pa;
+            const float *mq = pm;
+#pragma unroll
+            for (int p = 0; p < kAPer; ++p) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (p * kAPass < a_rows_left && a_cols_left > 0 && (kARows % kAPass == 0 || ar + p * kAPass < kARows)) {
+                    v = *reinterpret_cast<const float4 *>(q);
+                    if constexpr (MASKED && MODE == kNT) {
+                        const float4 m = *reinterpret_cast<const float4 *>(mq);
+                        v.x = m.x > 0.f ? v.x : 0.f;
+                        v.y = m.y > 0.f ? v.y : 0.f;
+                        v.z = m.z > 0.f ? v.z : 0.f;
+                        v.w = m.w > 0.f ? v.w : 0.f;
+                    }
+                }
+                ra[p] = v;
+                q += a_step;
+                if constexpr (MASKED && MODE == kNT) mq += m_step;
+            }
+        }
+        {
+            const float *q = pb;
+            const float *mq = pm;
+#pragma unroll
+            for (int p = 0; p < kBPer; ++p) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (p * kBPass < b_rows_left && b_cols_left > 0 && (kBRows % kBPass == 0 || br + p * kBPass < kBRows)) {
+                    v = *reinterpret_cast<const float4 *>(q);
+                    if constexpr (MASKED && MODE == kTN) {
+                        const float4 m = *reinterpret_cast<const float4 *>(mq);
+                        v.x = m.x > 0.f ? v.x : 0.f;
+                        v.y = m.y > 0.f ? v.y : 0.f;
+                        v.z = m.z > 0.f ? v.z : 0.f;
+                        v.w = m.w > 0.f ? v.w : 0.f;
+                    }
+                }
+                rb[p] = v;
+                q += b_step;
+                if constexpr (MASKED && MODE == kTN) mq += m_step;
+            }
+        }
+        // advance to the next chunk
+        pa += a_adv;
+        pb += b_adv;
+        if constexpr (MASKED) pm += m_adv;
+        if constexpr (kAContrRows) a_rows_left -= kBK; else a_cols_left -= kBK;
+        if constexpr (kBContrRows) b_rows_left -= kBK; else b_cols_left -= kBK;
+    };
+    const int a_st = ar * kAStride + av, b_st = br * kBStride + bv;
+    auto stash = [&](int buf) {
+        float *as = lds + buf * kASize + a_st;
+        float *bs = lds + 2 * kASize + buf * kBSize + b_st;
+#pragma unroll
+        for (int p = 0; p < kAPer; ++p)
+            if (kARows % kAPass == 0 || ar + p * kAPass < kARows) *reinterpret_cast<float4 *>(as + p * kAPass * kAStride) = ra[p];
+#pragma unroll
+        for (int p = 0; p < kBPer; ++p)
+            if (kBRows % kBPass == 0 || br + p * kBPass < kBRows) *reinterpret_cast<float4 *>(bs + p * kBPass * kBStride) = rb[p];
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    int buf = 0;
+    if (kbeg < kend) {
+        fetch();
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t k0 = kbeg; k0 < kend; k0 += kBK) {
+        const bool more = k0 + kBK < kend;
+        if (more) fetch();
+        const float *as = lds + buf * kASize;
+        const float *bs = lds + 2 * kASize + buf * kBSize;
+#pragma unroll
+        for (int s = 0; s < kBK / 8; ++s) {
+            float a[4];
+            if constexpr (kAX) {
+                const float4 t4 = *reinterpret_cast<const float4 *>(as + (wave * 32 + li) * kXS + 8 * s + 4 * h);
+                a[0] = t4.x; a[1] = t4.y; a[2] = t4.z; a[3] = t4.w;
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) a[m] = as[(8 * s + 4 * h + m) * kAStride + wave * 32 + li];
+            }
+            float b[TN][4];
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                if constexpr (kBX) {
+                    const float4 t4 = *reinterpret_cast<const float4 *>(bs + (t * 32 + li) * kXS + 8 * s + 4 * h);
+                    b[t][0] = t4.x; b[t][1] = t4.y; b[t][2] = t4.z; b[t][3] = t4.w;
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) b[t][m] = bs[(8 * s + 4 * h + m) * kBStride + t * 32 + li];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[m], b[t][m], acc[t], 0, 0, 0);
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    float *out;
+    int64_t ldo, nrows, ncols;
+    if constexpr (MODE == kTN) {
+        if (g.ws != nullptr) {
+            out = g.ws + (int64_t)blockIdx.x * g.ws_slab;
+            ldo = g.ws_ld;
+        } else {
+            out = g.C;
+            ldo = g.ldc;
+        }
+        nrows = g.K;
+        ncols = g.N;
+    } else {
+        out = g.C;
+        ldo = g.ldc;
+        nrows = g.M;
+        ncols = g.N;
+    }
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+    const int64_t rbase = row0 + wave * 32 + 4 * h;
+    const int rows_left = (int)min(max(nrows - rbase, (int64_t)0), (int64_t)64);
+    const int cols_left = (int)min(max(ncols - col0 - li, (int64_t)0), (int64_t)BN);
+    float *prow = out + rbase * ldo + col0 + li;
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+#pragma unroll
+        for (int vv = 0; vv < 4; ++vv) {
+            if (8 * v4 + vv < rows_left) {
+                float *q = prow + (int64_t)(8 * v4 + vv) * ldo;
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    float x = acc[t][4 * v4 + vv];
+                    if (relu) x = fmaxf(x, 0.f);
+                    if (t * 32 < cols_left) q[t * 32] = x;
+                }
+            }
+        }
+    }
+}
+
 // C[e] = sum over splits of ws[s][e], s ascending within four interleaved chains that are then
 // added in chain order -- a fixed order, so the result does not depend on scheduling.
 __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ ws, int64_t ws_ld, int64_t ws_slab,
@@ -287,9 +515,27 @@ int vec_ok(const float *p, int64_t ld) { return (p == nullptr || (reinterpret_ca
 
 int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
 
+template <int MODE, bool MASKED>
+void launch_vec(const GemmArgs &g, int tn, dim3 grid, hipStream_t st)
+{
+    switch (tn) {
+        case 1: gemm_f32_vec_kernel<MODE, 1, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        case 2: gemm_f32_vec_kernel<MODE, 2, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+        default: gemm_f32_vec_kernel<MODE, 4, MASKED><<<grid, kThreads, 0, st>>>(g); break;
+    }
+}
+
 template <int MODE>
 void launch_gemm(const GemmArgs &g, int tn, dim3 grid, hipStream_t st)
 {
+    // aligned operands and extents that are multiples of 4 -> the lean kernel; anything else -> the general one
+    const bool ext4 = (MODE == kTN) ? (g.K % 4 == 0 && g.N % 4 == 0) : (MODE == kNN ? (g.K % 4 == 0 && g.N % 4 == 0) : g.K % 4 == 0);
+    const bool vec = g.a_vec && g.b_vec && (g.mask == nullptr || g.m_vec) && ext4 && PLX_GEMM_LEAN;
+    if (vec) {
+        if (g.mask != nullptr && MODE != kNN) launch_vec<MODE, true>(g, tn, grid, st);
+        else launch_vec<MODE, false>(g, tn, grid, st);
+        return;
+    }
     switch (tn) {
         case 1: gemm_f32_kernel<MODE, 1><<<grid, kThreads, 0, st>>>(g); break;
         case 2: gemm_f32_kernel<MODE, 2><<<grid, kThreads, 0, st>>>(g); break;
