@@ -137,7 +137,7 @@ int plx_cast_f32_bf16(int64_t M, int64_t N, const float *X, int64_t ldx, uint16_
                       void *stream);
 
 /* Y = max(X, 0) and dX = dY ⊙ [Y > 0] for callers that keep F.relu outside the layer
- * (examples/train.py:77-78). */
+ * (examples/train.py:77-78).  Outputs may alias inputs. */
 int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream);
 int plx_relu_bwd_f32(int64_t M, int64_t N, const float *dY, int64_t lddy, const float *Y, int64_t ldy, float *dX,
                      int64_t lddx, void *stream);

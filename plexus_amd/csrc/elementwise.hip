@@ -13,9 +13,8 @@ namespace {
 
 // grid-stride over rows x (cols / 4) float4 lanes when everything is 16-byte aligned, scalars otherwise
 template <bool BWD, bool VEC4>
-__global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const float *__restrict__ in, int64_t ldi,
-                                                   const float *__restrict__ ref, int64_t ldr, float *__restrict__ out,
-                                                   int64_t ldo)
+__global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const float *in, int64_t ldi, const float *ref,
+                                                   int64_t ldr, float *out, int64_t ldo)  // out may alias in (or ref)
 {
     const int64_t per_row = VEC4 ? N / 4 : N;
     const int64_t total = M * per_row;

@@ -57,7 +57,11 @@ class GCNConvFunction(torch.autograd.Function):
         dropout_p=0.0,
         dropout_seed=0,
         dropout_offset=0,
+        transform_first=False,
     ):
+        if transform_first:
+            return GCNConvFunction._forward_transform_first(
+                ctx, x, edge_index, edge_index_t, weight, local_features_shape, local_weight_shape, layer_num, fuse_relu)
         timers = get_timers()
         timers.start("gcn conv fwd")
         A = ops.as_csr(edge_index)
@@ -90,12 +94,85 @@ class GCNConvFunction(torch.autograd.Function):
         ctx.layer_num = layer_num
         ctx.fuse_relu = fuse_relu
         ctx.bf16 = bf16
+        ctx.transform_first = False
         ctx.grad_scale = 1.0 / (1.0 - dropout_p) if dropout_p > 0.0 else 1.0
         timers.stop("gcn conv fwd")
         return OUT
 
+    # ---- re-associated product:  A.(H.W)  instead of the reference's  (A.H).W ----
+    # The two are the same matrix; when the layer narrows (out < in) the sparse product then gathers rows
+    # of `out` instead of `in` elements, and the gather volume is what the layer costs.  Backward likewise:
+    # T = A^T.G, GRAD_W = H^T.T, GRAD_H = T.W^T.  fp32 results differ from the reference order by rounding only.
+    @staticmethod
+    def _forward_transform_first(ctx, x, edge_index, edge_index_t, weight, local_features_shape, local_weight_shape,
+                                 layer_num, fuse_relu):
+        if x.dtype != torch.float32:
+            raise ValueError("transform-first association is implemented for fp32 storage")
+        timers = get_timers()
+        timers.start("gcn conv fwd")
+        A = ops.as_csr(edge_index)
+        H = x.detach().reshape(local_features_shape)
+        W = weight.detach().reshape(local_weight_shape)
+        d_out = local_weight_shape[1]
+        d_pad = (d_out + 3) // 4 * 4  # rows of Z padded to 16 bytes so that the gather uses 128-bit loads
+        timers.start("OUT = AGG * W")
+        Z = torch.zeros((H.shape[0], d_pad), dtype=torch.float32, device=H.device) if d_pad != d_out else \
+            torch.empty((H.shape[0], d_pad), dtype=torch.float32, device=H.device)
+        ops.gemm_nn(H, W, out=Z[:, :d_out])
+        timers.stop("OUT = AGG * W")
+        timers.start("AGG = A * H")
+        OUTp = ops.spmm(A, Z)
+        timers.stop("AGG = A * H")
+        OUT = OUTp[:, :d_out]
+        if fuse_relu:
+            ops.relu(OUT, inplace=True)
+        ctx.save_for_backward(H, weight, OUT if fuse_relu else None)
+        ctx.adj_t = ops.as_csr(edge_index_t)
+        ctx.local_weight_shape = tuple(local_weight_shape)
+        ctx.x_shape = x.shape
+        ctx.layer_num = layer_num
+        ctx.fuse_relu = fuse_relu
+        ctx.bf16 = False
+        ctx.transform_first = True
+        ctx.grad_scale = 1.0
+        timers.stop("gcn conv fwd")
+        return OUT
+
+    @staticmethod
+    def _backward_transform_first(ctx, grad_output):
+        timers = get_timers()
+        timers.start("gcn conv bwd")
+        H, weight, out = ctx.saved_tensors
+        W = weight.detach().reshape(ctx.local_weight_shape)
+        d_out = ctx.local_weight_shape[1]
+        d_pad = (d_out + 3) // 4 * 4
+        m = grad_output.shape[0]
+        Gp = torch.zeros((m, d_pad), dtype=torch.float32, device=grad_output.device) if d_pad != d_out else \
+            torch.empty((m, d_pad), dtype=torch.float32, device=grad_output.device)
+        if ctx.fuse_relu:
+            ops.relu_bwd(grad_output, out, out=Gp[:, :d_out])
+        else:
+            Gp[:, :d_out].copy_(grad_output)
+        timers.start("GRAD_H = A.T * GRAD_AGG")
+        T = ops.spmm(ctx.adj_t, Gp)[:, :d_out]
+        timers.stop("GRAD_H = A.T * GRAD_AGG")
+        grad_weight = None
+        if ctx.needs_input_grad[3]:
+            timers.start("GRAD_W = AGG.T * GRAD_OUT")
+            grad_weight = ops.gemm_tn(H, T).reshape(weight.shape)
+            timers.stop("GRAD_W = AGG.T * GRAD_OUT")
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            timers.start("GRAD_AGG = GRAD_OUT * W.T")
+            grad_x = ops.gemm_nt(T, W).reshape(ctx.x_shape)
+            timers.stop("GRAD_AGG = GRAD_OUT * W.T")
+        timers.stop("gcn conv bwd")
+        return (grad_x, None, None, grad_weight) + (None,) * 13
+
     @staticmethod
     def backward(ctx, grad_output):
+        if ctx.transform_first:
+            return GCNConvFunction._backward_transform_first(ctx, grad_output)
         timers = get_timers()
         timers.start("gcn conv bwd")
         agg, weight, out = ctx.saved_tensors
@@ -128,7 +205,7 @@ class GCNConvFunction(torch.autograd.Function):
             grad_x = grad_x.reshape(ctx.x_shape)  # flat again for layer 0 (plexus/gcn_conv.py:271)
 
         timers.stop("gcn conv bwd")
-        return (grad_x, None, None, grad_weight) + (None,) * 12
+        return (grad_x, None, None, grad_weight) + (None,) * 13
 
 
 class GCNConv(torch.nn.Module):
@@ -139,14 +216,15 @@ class GCNConv(torch.nn.Module):
     ``kaiming_uniform_(a=sqrt(5))`` on an (in, out) tensor (plexus/gcn_conv.py:332-333) -- on the host
     generator, so that a seed reproduces the same weights on any device -- or taken from ``weight``.
 
-    Additions: ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (bf16 storage only) drops
+    Additions: ``association`` selects the order of the two products (see above; the default is the
+    reference's); ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (bf16 storage only) drops
     activations after the ReLU in training mode with a counter-based generator keyed by ``dropout_seed``;
     every training forward uses a fresh offset (``layer_num + 64 * call count``).  The storage type
     follows the input tensor.
     """
 
     def __init__(self, in_channels, out_channels, layer_num, weight=None, fuse_relu=False, dropout=0.0, dropout_seed=0,
-                 device=None, **kwargs):
+                 association="reference", device=None, **kwargs):
         super().__init__()
         self.layer_num = layer_num
         self.gather_features = layer_num == 0
@@ -159,6 +237,13 @@ class GCNConv(torch.nn.Module):
         self.fuse_relu = fuse_relu
         self.dropout = float(dropout)
         self.dropout_seed = int(dropout_seed)
+        # "reference": (A.H).W as plexus/gcn_conv.py:188,211 always does; "transform_first": A.(H.W);
+        # "auto": transform first when that makes the gathered rows span fewer 128-byte lines (fp32 only)
+        if association not in ("reference", "transform_first", "auto"):
+            raise ValueError("association must be 'reference', 'transform_first' or 'auto'")
+        lines = lambda d: (d * 4 + 127) // 128
+        self.transform_first = association == "transform_first" or (
+            association == "auto" and lines((out_channels + 3) // 4 * 4) < lines(in_channels))
         self.forward_calls = 0
         if device is None:
             device = "cuda" if torch.cuda.is_available() else "cpu"
@@ -196,4 +281,5 @@ class GCNConv(torch.nn.Module):
             p,
             self.dropout_seed,
             offset,
+            self.transform_first and x.dtype == torch.float32 and p == 0.0,
         )

@@ -167,15 +167,20 @@ def spmm(a, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor
     return out
 
 
-def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False) -> torch.Tensor:
-    """C = A.B, optionally max(C, 0)."""
-    _need_gpu(a, b)
+def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix."""
+    _need_gpu(a, b, out)
     a, b = _rowmajor(a), _rowmajor(b)
     m, k = a.shape
     k2, n = b.shape
     if k != k2:
         raise ValueError("gemm_nn: inner dimensions differ (%d vs %d)" % (k, k2))
-    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    if out is None:
+        c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    else:
+        c = out
+        if tuple(c.shape) != (m, n) or c.dtype != torch.float32 or (n > 1 and c.stride(1) != 1):
+            raise ValueError("gemm_nn: out must be fp32 [%d x %d] with contiguous rows" % (m, n))
     check(
         _lib.load().plx_gemm_nn_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
                                     PLX_GEMM_RELU if relu else 0, _stream()),
@@ -297,18 +302,19 @@ def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] 
     return c
 
 
-def relu(x: torch.Tensor) -> torch.Tensor:
+def relu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     _need_gpu(x)
-    x = _rowmajor(x)
-    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    if not inplace:
+        x = _rowmajor(x)
+    y = x if inplace else torch.empty(x.shape, dtype=torch.float32, device=x.device)
     check(_lib.load().plx_relu_f32(x.shape[0], x.shape[1], x.data_ptr(), _ld(x), y.data_ptr(), _ld(y), _stream()), "plx_relu_f32")
     return y
 
 
-def relu_bwd(dy: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
-    _need_gpu(dy, y)
+def relu_bwd(dy: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _need_gpu(dy, y, out)
     dy, y = _rowmajor(dy), _rowmajor(y)
-    dx = torch.empty(dy.shape, dtype=torch.float32, device=dy.device)
+    dx = out if out is not None else torch.empty(dy.shape, dtype=torch.float32, device=dy.device)
     check(
         _lib.load().plx_relu_bwd_f32(dy.shape[0], dy.shape[1], dy.data_ptr(), _ld(dy), y.data_ptr(), _ld(y),
                                      dx.data_ptr(), _ld(dx), _stream()),

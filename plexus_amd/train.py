@@ -16,7 +16,7 @@ from .utils.timers import get_timers
 
 class Net(torch.nn.Module):
     def __init__(self, num_gcn_layers, input_size, hidden_size, output_size, weights=None, fuse_relu=True, dropout=0.0,
-                 dropout_seed=0):
+                 dropout_seed=0, association="reference"):
         super().__init__()
         self.num_gcn_layers = num_gcn_layers
         self.fuse_relu = fuse_relu
@@ -26,7 +26,8 @@ class Net(torch.nn.Module):
             last = i == num_gcn_layers - 1
             self.layers.append(
                 GCNConv(dims[i], dims[i + 1], i, weight=None if weights is None else weights[i],
-                        fuse_relu=fuse_relu and not last, dropout=0.0 if last else dropout, dropout_seed=dropout_seed)
+                        fuse_relu=fuse_relu and not last, dropout=0.0 if last else dropout, dropout_seed=dropout_seed,
+                        association=association)
             )
 
     def forward(self, x, edge_index_shards):

@@ -635,3 +635,63 @@ def test_internal_timers_use_the_reference_names():
     finally:
         plexus_amd.init()
         get_timers().reset()
+
+
+@pytest.mark.parametrize("din,dout,relu", [(128, 47, False), (100, 16, True), (64, 64, True), (33, 5, False)])
+def test_transform_first_association_matches_reference_order(din, dout, relu):
+    """A.(H.W) instead of (A.H).W is the same matrix; checked against the reference-order oracle."""
+    say("transform-first layer %d->%d relu=%s" % (din, dout, relu))
+    from plexus_amd.gcn_conv import GCNConv
+
+    n = 1500
+    g = S.build_graph(n, "chunglu", 20000, seed=7, device="cpu")
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(n, din, generator=gen)
+    w = po.kaiming_uniform_weight(din, dout, gen)
+    go = torch.randn(n, dout, generator=gen)
+    outs, gxs, gws = [], [], []
+    for dt in (torch.float32, torch.float64):
+        a, at = g.torch_csr().to(dt), g.torch_csr(True).to(dt)
+        out_ref, agg_ref = po.gcn_conv_forward(x.to(dt), a, w.to(dt), (n, din), (din, dout))
+        outs.append(torch.relu(out_ref) if relu else out_ref)
+    layer = GCNConv(din, dout, 1, weight=w, fuse_relu=relu, association="transform_first")
+    assert layer.transform_first
+    xd = x.to(DEV).requires_grad_()
+    out = layer(xd, [(to_dev(g), to_dev(g, True))])
+    out.backward(go.to(DEV))
+    assert_parity(out, outs[0], outs[1], what="OUT")
+    mask = (out > 0).cpu() if relu else None  # pin the ReLU mask to the device's (sign of values within rounding of 0)
+    for dt in (torch.float32, torch.float64):
+        a, at = g.torch_csr().to(dt), g.torch_csr(True).to(dt)
+        _, agg_ref = po.gcn_conv_forward(x.to(dt), a, w.to(dt), (n, din), (din, dout))
+        gm = go.to(dt) * mask.to(dt) if relu else go.to(dt)
+        gx, gw = po.gcn_conv_backward(gm, agg_ref, w.to(dt), at, (din, dout))
+        gxs.append(gx)
+        gws.append(gw)
+    assert_parity(xd.grad, gxs[0], gxs[1], what="grad_x")
+    assert_parity(layer.weight.grad, gws[0], gws[1], what="grad_w")
+    # "auto" picks it exactly when the gathered rows get shorter in 128-byte lines
+    assert GCNConv(128, 47, 2, association="auto").transform_first
+    assert GCNConv(1433, 16, 0, association="auto").transform_first
+    assert not GCNConv(100, 128, 0, association="auto").transform_first
+    assert not GCNConv(128, 128, 1, association="auto").transform_first
+    assert not GCNConv(128, 47, 2).transform_first
+
+
+def test_config1_ten_epochs_with_auto_association():
+    say("config 1, 10 epochs, association=auto")
+    from plexus_amd.train import Net, make_optimizer, run_epochs
+
+    g, x, y, dims = S.config1(device="cpu", seed=0)
+    weights = S.glorot_weights(dims, seed=0)
+    n = g.shape[0]
+    ref64, _, _ = po.train_epochs(x.double(), [w.double() for w in weights], dims,
+                                  [(g.torch_csr().double(), g.torch_csr(True).double())], y, n, 7, epochs=10)
+    model = Net(2, dims[0], dims[1], dims[2], weights=weights, association="auto")
+    assert model.layers[0].transform_first and not model.layers[1].transform_first  # 16 -> 7 stays inside one line
+    feats = x.reshape(-1).to(DEV).requires_grad_()
+    opt = make_optimizer(model, feats)
+    shards = [(g.torch_csr().to(DEV), g.torch_csr(True).to(DEV))]
+    losses = run_epochs(model, opt, feats, shards, y.to(DEV), n, 7, 10)
+    for l, r64 in zip(losses, ref64):
+        assert abs(l - r64) <= FP32_TOL * abs(r64)
