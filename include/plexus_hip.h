@@ -85,6 +85,14 @@ size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D);
 /* fp32 values, fp32 H and Y. */
 int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
                      int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+/* Rows [row_begin, row_end) of the same product: only those rows of Y (the base of the full M x D output) are
+ * written.  The row-chunked aggregation of plexus/gcn_conv.py:67-128 (extract_csr_submatrix + SpMM per chunk +
+ * torch.cat) without building sub-matrices; a caller can hand each finished chunk on (e.g. to a collective on
+ * another stream) while the next one runs.  Chunks of one plan may run concurrently: their scratch rows in
+ * `workspace` are disjoint. */
+int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const float *H,
+                          int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                          void *stream);
 /* fp32 values, bf16 H and Y (raw uint16 bit patterns), fp32 accumulation, round-to-nearest-even store. */
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
                       uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);

@@ -15,6 +15,7 @@
 //     than that are tiled over gridDim.y.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <vector>
 
@@ -36,10 +37,13 @@ struct SpmmArgs {
     int64_t ldh;
     int64_t ldy;
     int64_t ldws;
-    int32_t M;
-    int32_t n_seg;
+    int32_t M;         // rows are [row_begin, row_end)
+    int32_t n_seg;     // segment tasks of this launch
     int32_t D;
     int32_t seg_len;
+    int32_t row_begin;
+    int32_t row_end;
+    int32_t seg_base;  // index of the first segment task in the plan's tables
 };
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
@@ -195,13 +199,13 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
     bool to_ws;
     int64_t out_row;
     if (task < p.n_seg) {
-        a = p.seg_begin[task];
-        b = p.seg_end[task];
+        a = p.seg_begin[p.seg_base + task];
+        b = p.seg_end[p.seg_base + task];
         to_ws = true;
-        out_row = task;
+        out_row = p.seg_base + task;  // partial rows are indexed by the plan-wide segment number
     } else {
-        const int64_t r = task - p.n_seg;
-        if (r >= p.M) return;
+        const int64_t r = p.row_begin + (task - p.n_seg);
+        if (r >= p.row_end) return;
         a = p.rowptr[r];
         b = p.rowptr[r + 1];
         if (b - a > p.seg_len) return;  // split row: its segments are separate tasks
@@ -308,11 +312,11 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
 template <typename TOUT>
 __global__ void __launch_bounds__(256) spmm_reduce_split_rows(const float *__restrict__ ws, int64_t ldws,
                                                               const int32_t *__restrict__ long_rows,
-                                                              const int32_t *__restrict__ seg_first, int32_t D,
-                                                              TOUT *__restrict__ Y, int64_t ldy)
+                                                              const int32_t *__restrict__ seg_first, int32_t q_base,
+                                                              int32_t D, TOUT *__restrict__ Y, int64_t ldy)
 {
     __shared__ float4 part[16][16];
-    const int q = blockIdx.x;
+    const int q = q_base + blockIdx.x;
     const int chain = threadIdx.x >> 4;
     const int l = threadIdx.x & 15;
     const int d = blockIdx.y * 64 + l * 4;
@@ -372,6 +376,7 @@ struct plx_spmm_plan {
     int64_t n_long, n_seg;
     int32_t *tables;  // device: long_rows[n_long] | seg_first[n_long+1] | seg_begin[n_seg] | seg_end[n_seg]
     const int32_t *long_rows, *seg_first, *seg_begin, *seg_end;
+    std::vector<int32_t> h_long_rows, h_seg_first;  // host copies, to cut row ranges out of the plan
 };
 
 namespace {
@@ -406,12 +411,14 @@ int launch_for_vec(const SpmmArgs &a, int lpr, int nacc, dim3 grid, hipStream_t 
 }
 
 template <typename T>
-int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t ldh, int64_t D, T *Y, int64_t ldy,
-              void *workspace, size_t workspace_bytes, void *stream)
+int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const T *H, int64_t ldh,
+              int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
 {
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
+    PLX_REQUIRE(row_begin >= 0 && row_begin <= row_end && row_end <= plan->M, "spmm: row range [%lld, %lld) outside [0, %lld)",
+                (long long)row_begin, (long long)row_end, (long long)plan->M);
     PLX_REQUIRE(D >= 0 && D < (1ll << 30), "spmm: bad feature width D=%lld", (long long)D);
-    if (plan->M == 0 || D == 0) return PLX_OK;
+    if (row_begin == row_end || D == 0) return PLX_OK;
     PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
@@ -447,13 +454,22 @@ int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t l
     a.ldh = ldh;
     a.ldy = ldy;
     a.ldws = ws_ld(D);
+    // split rows inside the range, and their segments
+    const auto lr_begin = plan->h_long_rows.begin(), lr_end = plan->h_long_rows.end();
+    const int64_t q0 = std::lower_bound(lr_begin, lr_end, (int32_t)row_begin) - lr_begin;
+    const int64_t q1 = std::lower_bound(lr_begin, lr_end, (int32_t)row_end) - lr_begin;
+    const int64_t s0 = q1 > q0 ? plan->h_seg_first[(size_t)q0] : 0;
+    const int64_t s1 = q1 > q0 ? plan->h_seg_first[(size_t)q1] : 0;
     a.M = (int32_t)plan->M;
-    a.n_seg = (int32_t)plan->n_seg;
+    a.n_seg = (int32_t)(s1 - s0);
     a.D = (int32_t)D;
     a.seg_len = plan->seg_len;
+    a.row_begin = (int32_t)row_begin;
+    a.row_end = (int32_t)row_end;
+    a.seg_base = (int32_t)s0;
 
     hipStream_t st = plx::as_stream(stream);
-    const int64_t tasks = plan->M + plan->n_seg;
+    const int64_t tasks = (row_end - row_begin) + (s1 - s0);
     dim3 grid((unsigned)plx::ceil_div(tasks, 4), (unsigned)tiles, 1);
     int rc = -1;
     switch (vec) {
@@ -468,9 +484,9 @@ int spmm_impl(const plx_spmm_plan *plan, const float *val, const T *H, int64_t l
     if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "spmm: no kernel for vec=%d lpr=%d nacc=%d", vec, lpr, nacc);
     PLX_LAUNCH_CHECK("spmm_csr_kernel");
 
-    if (plan->n_long > 0) {
-        dim3 rgrid((unsigned)plan->n_long, (unsigned)plx::ceil_div(D, 64), 1);
-        spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)D, Y, ldy);
+    if (q1 > q0) {
+        dim3 rgrid((unsigned)(q1 - q0), (unsigned)plx::ceil_div(D, 64), 1);
+        spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)D, Y, ldy);
         PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
     }
     return PLX_OK;
@@ -590,6 +606,8 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
             delete p;
             return plx::fail(PLX_ERR_HIP, "plan_create: table upload failed: %s", hipGetErrorString(e));
         }
+        p->h_long_rows.assign(lr, lr + nl);
+        p->h_seg_first.assign(sf, sf + nl + 1);
         p->long_rows = p->tables;
         p->seg_first = p->tables + nl;
         p->seg_begin = p->seg_first + nl + 1;
@@ -630,13 +648,20 @@ size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)
 int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
                      int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
 {
-    return spmm_impl<float>(plan, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+    return spmm_impl<float>(plan, 0, plan ? plan->M : 0, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const float *H,
+                          int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                          void *stream)
+{
+    return spmm_impl<float>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
 }
 
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
                       uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
 {
-    return spmm_impl<uint16_t>(plan, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+    return spmm_impl<uint16_t>(plan, 0, plan ? plan->M : 0, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -167,6 +167,39 @@ def spmm(a, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor
     return out
 
 
+def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk=None) -> torch.Tensor:
+    """Row-chunked Y = A.H with the reference's chunk boundaries (plexus/gcn_conv.py:77-91).
+
+    Each chunk is one launch writing its rows of the full output; ``on_chunk(i, (start, end), y)`` is called after
+    chunk i has been enqueued (the place where the reference starts the chunk's all-reduce, gcn_conv.py:103-110).
+    The rows are bit-identical to the un-chunked product."""
+    a = as_csr(a)
+    _need_gpu(h)
+    h = _rowmajor(h)
+    if h.dtype != torch.float32:
+        raise TypeError("chunked_spmm: fp32 only")
+    m, k = a.shape
+    if h.shape[0] != k:
+        raise ValueError("chunked_spmm: A is %dx%d but H has %d rows" % (m, k, h.shape[0]))
+    d = h.shape[1]
+    y = torch.empty((m, d), dtype=torch.float32, device=h.device)
+    ws, ws_bytes = a._workspace(d)
+    lib = _lib.load()
+    num_chunks = max(1, (m + max_rows_per_chunk - 1) // max_rows_per_chunk)
+    rows_per_chunk = m // num_chunks
+    for i in range(num_chunks):
+        start = i * rows_per_chunk
+        end = m if i == num_chunks - 1 else (i + 1) * rows_per_chunk
+        check(
+            lib.plx_spmm_csr_rows_f32(a._plan, start, end, a.val.data_ptr(), h.data_ptr(), _ld(h), d, y.data_ptr(), _ld(y),
+                                      ws.data_ptr() if ws is not None else None, ws_bytes, _stream()),
+            "plx_spmm_csr_rows_f32",
+        )
+        if on_chunk is not None:
+            on_chunk(i, (start, end), y)
+    return y
+
+
 def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix."""
     _need_gpu(a, b, out)

@@ -695,3 +695,35 @@ def test_config1_ten_epochs_with_auto_association():
     losses = run_epochs(model, opt, feats, shards, y.to(DEV), n, 7, 10)
     for l, r64 in zip(losses, ref64):
         assert abs(l - r64) <= FP32_TOL * abs(r64)
+
+
+def test_row_chunked_spmm_is_bit_identical_and_hands_chunks_on():
+    say("row-chunked SpMM (blocked aggregation)")
+    import plexus_amd
+    from plexus_amd.gcn_conv import GCNConv
+
+    g = S.build_graph(5000, "chunglu", 60000, seed=3, device="cpu", gamma=2.1)
+    a = to_dev(g, seg_len=64)
+    assert a.n_long_rows > 3
+    h = torch.randn(5000, 36, generator=torch.Generator().manual_seed(0)).to(DEV)
+    full = ops.spmm(a, h)
+    seen = []
+    y = ops.chunked_spmm(a, h, max_rows_per_chunk=700, on_chunk=lambda i, rng, out: seen.append((i, rng)))
+    assert torch.equal(y, full)
+    assert [r for _, r in seen] == po.chunk_bounds(5000, 700)  # the reference's chunk boundaries
+    assert torch.equal(ops.chunked_spmm(a, h), full)  # one chunk
+    ref = po.chunked_spmm(g.torch_csr(), h.cpu(), max_rows_per_chunk=700)
+    assert rel_err(y, ref) <= FP32_TOL
+    # through the layer: block_aggregation gives the same output and gradients
+    w = po.kaiming_uniform_weight(36, 8, torch.Generator().manual_seed(1))
+    outs = []
+    for blocked in (False, True):
+        plexus_amd.init(block_aggregation=blocked)
+        layer = GCNConv(36, 8, 1, weight=w)
+        x = h.clone().requires_grad_()
+        o = layer(x, [(a, to_dev(g, True))])
+        o.sum().backward()
+        outs.append((o.detach(), x.grad, layer.weight.grad))
+    plexus_amd.init()
+    for u, v in zip(*outs):
+        assert torch.equal(u, v)
