@@ -54,6 +54,24 @@ const char *plx_last_error(void);
 int plx_csr_narrow_i64(int64_t M, int64_t nnz, const int64_t *rowptr64, const int64_t *col64, int32_t *rowptr32,
                        int32_t *col32, void *stream);
 
+/* CSR of the transpose, built on the device: rowptr_t[K+1], col_t[nnz], val_t[nnz]; rows in order, columns
+ * ascending within a row -- entry for entry what adj_local.transpose(0, 1).to_sparse_csr() gives on the host
+ * (plexus/utils/dataloader.py:368).  Stable radix sort by column plus streaming kernels; `workspace` must be
+ * 256-byte aligned. */
+size_t plx_csr_transpose_workspace_bytes(int64_t M, int64_t K, int64_t nnz);
+int plx_csr_transpose_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, const int32_t *col, const float *val,
+                          int32_t *rowptr_t, int32_t *col_t, float *val_t, void *workspace, size_t workspace_bytes, void *stream);
+
+/* A rank's CSR block from an edge list, on the device: keep the edges with r0 <= row < r1 and c0 <= col < c1,
+ * re-base them to the block, sort by (row, col) and add the weights of duplicate edges -- the sequence
+ * mask / re-base / sparse_coo_tensor / to_sparse_csr of plexus/utils/dataloader.py:343-367 (and
+ * benchmarking/spmm.py:67-84).  rowptr has r1 - r0 + 1 entries; col_out / val_out need room for n_edges entries;
+ * the number of stored entries is returned in *nnz_host (the call synchronises `stream` twice to learn it). */
+size_t plx_coo_block_to_csr_workspace_bytes(int64_t n_edges, int64_t block_rows, int64_t block_cols);
+int plx_coo_block_to_csr_f32(int64_t n_edges, const int64_t *row, const int64_t *col, const float *weight, int64_t r0, int64_t r1,
+                             int64_t c0, int64_t c1, int32_t *rowptr, int32_t *col_out, float *val_out, int64_t *nnz_host,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* Host-only row analysis behind plx_spmm_plan_create, exported so it can be tested without a GPU.
  * Rows longer than seg_len are split into ceil(len/seg_len) near-equal segments.  Writes at most
  * `cap_long` row ids to long_rows_host, cap_long+1 entries to seg_first_host and `cap_seg` entries to

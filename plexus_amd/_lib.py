@@ -24,6 +24,10 @@ SIGNATURES = {
     "plx_error_string": (C.c_char_p, [C.c_int]),
     "plx_last_error": (C.c_char_p, []),
     "plx_csr_narrow_i64": (C.c_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "plx_csr_transpose_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_csr_transpose_f32": (C.c_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "plx_coo_block_to_csr_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_coo_block_to_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, C.POINTER(_i64), _vp, _sz, _vp]),
     "plx_spmm_segments_host": (C.c_int, [_i64, _vp, _i32, C.POINTER(_i64), C.POINTER(_i64), _vp, _vp, _i64, _vp, _vp, _i64]),
     "plx_spmm_plan_create": (C.c_int, [C.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _i32, _vp]),
     "plx_spmm_plan_destroy": (C.c_int, [_vp]),

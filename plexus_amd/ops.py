@@ -127,6 +127,64 @@ class CsrMatrix:
         )
 
 
+def _aligned_workspace(nbytes: int, device) -> torch.Tensor:
+    """uint8 scratch whose data pointer is 256-byte aligned (torch's allocator hands out 512-byte aligned blocks)."""
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+    assert ws.data_ptr() % 256 == 0
+    return ws
+
+
+def csr_transpose(a: CsrMatrix, seg_len: int = 0) -> CsrMatrix:
+    """The CSR of A^T, built on the device (what the reference's loader builds on the host, dataloader.py:368)."""
+    m, k = a.shape
+    lib = _lib.load()
+    rowptr_t = torch.empty(k + 1, dtype=torch.int32, device=a.device)
+    col_t = torch.empty(a.nnz, dtype=torch.int32, device=a.device)
+    val_t = torch.empty(a.nnz, dtype=torch.float32, device=a.device)
+    need = int(lib.plx_csr_transpose_workspace_bytes(m, k, a.nnz))
+    ws = _aligned_workspace(need, a.device)
+    check(
+        lib.plx_csr_transpose_f32(m, k, a.nnz, a.rowptr.data_ptr(), a.col.data_ptr() if a.nnz else None,
+                                  a.val.data_ptr() if a.nnz else None, rowptr_t.data_ptr(), col_t.data_ptr() if a.nnz else None,
+                                  val_t.data_ptr() if a.nnz else None, ws.data_ptr(), need, _stream()),
+        "plx_csr_transpose_f32",
+    )
+    return CsrMatrix(rowptr_t, col_t, val_t, (k, m), seg_len)
+
+
+def csr_pair_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, shape, row_range=None, col_range=None,
+                        seg_len: int = 0):
+    """(A, A^T) of a rank's block from an edge list, on the device.
+
+    Counterpart of the loader's ``__split_adj`` (plexus/utils/dataloader.py:327-375): mask the edges to
+    ``row_range x col_range``, re-base, build the CSR (duplicates summed) and the CSR of its transpose."""
+    _need_gpu(edge_index, edge_weight)
+    r0, r1 = row_range if row_range is not None else (0, int(shape[0]))
+    c0, c1 = col_range if col_range is not None else (0, int(shape[1]))
+    ei = edge_index.to(torch.int64)
+    rows, cols = ei[0].contiguous(), ei[1].contiguous()
+    w = edge_weight.to(torch.float32).contiguous()
+    n = int(rows.numel())
+    lib = _lib.load()
+    mb, kb = r1 - r0, c1 - c0
+    rowptr = torch.empty(mb + 1, dtype=torch.int32, device=w.device)
+    col_out = torch.empty(max(n, 1), dtype=torch.int32, device=w.device)
+    val_out = torch.empty(max(n, 1), dtype=torch.float32, device=w.device)
+    need = int(lib.plx_coo_block_to_csr_workspace_bytes(n, mb, kb))
+    ws = _aligned_workspace(need, w.device)
+    nnz = _lib.C.c_int64(0)
+    check(
+        lib.plx_coo_block_to_csr_f32(n, rows.data_ptr() if n else None, cols.data_ptr() if n else None, w.data_ptr() if n else None,
+                                     r0, r1, c0, c1, rowptr.data_ptr(), col_out.data_ptr(), val_out.data_ptr(), _lib.C.byref(nnz),
+                                     ws.data_ptr(), need, _stream()),
+        "plx_coo_block_to_csr_f32",
+    )
+    del ws
+    k = int(nnz.value)
+    a = CsrMatrix(rowptr, col_out[:k].clone(), val_out[:k].clone(), (mb, kb), seg_len)
+    return a, csr_transpose(a, seg_len)
+
+
 def as_csr(a, seg_len: int = 0) -> CsrMatrix:
     """CsrMatrix of ``a``; a torch CSR tensor is converted once and the result is cached on it."""
     if isinstance(a, CsrMatrix):

@@ -727,3 +727,51 @@ def test_row_chunked_spmm_is_bit_identical_and_hands_chunks_on():
     plexus_amd.init()
     for u, v in zip(*outs):
         assert torch.equal(u, v)
+
+
+def test_device_csr_transpose_matches_host_construction():
+    say("device CSR transpose")
+    cases = [S.build_graph(3000, "chunglu", 40000, seed=1, device="cpu"),
+             S.build_graph(4096, "rmat", 30000, seed=2, device="cpu", double_perm=True, block=((0, 2048), (0, 1024))),
+             S.build_graph(300, "uniform", 0, seed=3, device="cpu", exact_pairs=50)]
+    for g in cases:
+        a = to_dev(g)
+        at = ops.csr_transpose(a)
+        assert at.shape == (g.shape[1], g.shape[0])
+        assert torch.equal(at.rowptr.cpu().long(), g.rowptr_t)
+        assert torch.equal(at.col.cpu().long(), g.col_t)
+        assert torch.equal(at.val.cpu(), g.val_t)  # bit-exact: values are moved, not recomputed
+        # and it is what torch builds on the host (the reference's way)
+        ref = g.torch_csr().transpose(0, 1).to_sparse_csr()
+        assert torch.equal(at.rowptr.cpu().long(), ref.crow_indices()) and torch.equal(at.col.cpu().long(), ref.col_indices())
+        assert torch.equal(at.val.cpu(), ref.values())
+    # empty matrix
+    e = ops.CsrMatrix(torch.zeros(11, dtype=torch.int64, device=DEV), torch.zeros(0, dtype=torch.int64, device=DEV),
+                      torch.zeros(0, device=DEV), (10, 7))
+    et = ops.csr_transpose(e)
+    assert et.shape == (7, 10) and et.nnz == 0 and (et.rowptr == 0).all()
+
+
+def test_device_block_csr_from_edge_list_matches_loader_sequence():
+    say("device COO block -> CSR pair")
+    gen = torch.Generator().manual_seed(0)
+    n = 500
+    ei = torch.randint(0, n, (2, 6000), generator=gen)
+    ei = torch.cat([ei, ei[:, :500]], dim=1)  # 500 duplicated edges: the host path sums them
+    w = torch.rand(ei.shape[1], generator=gen)
+    for rr, cr in [((0, n), (0, n)), ((100, 350), (0, 250)), ((0, 10), (490, 500)), ((200, 200), (0, n))]:
+        a_ref, at_ref = po.build_csr_pair(ei, w, (n, n), rr, cr)
+        a, at = ops.csr_pair_from_edges(ei.to(DEV), w.to(DEV), (n, n), rr, cr)
+        assert a.shape == tuple(a_ref.shape) and at.shape == tuple(at_ref.shape)
+        assert torch.equal(a.rowptr.cpu().long(), a_ref.crow_indices())
+        assert torch.equal(a.col.cpu().long(), a_ref.col_indices())
+        assert rel_err(a.val.cpu(), a_ref.values()) <= FP32_TOL if a.nnz else True
+        assert torch.equal(at.rowptr.cpu().long(), at_ref.crow_indices())
+        assert torch.equal(at.col.cpu().long(), at_ref.col_indices())
+        assert rel_err(at.val.cpu(), at_ref.values()) <= FP32_TOL if a.nnz else True
+    # the pair feeds the layer directly
+    h = torch.randn(n, 16, generator=gen)
+    a, at = ops.csr_pair_from_edges(ei.to(DEV), w.to(DEV), (n, n))
+    a_ref, at_ref = po.build_csr_pair(ei, w, (n, n))
+    assert rel_err(ops.spmm(a, h.to(DEV)), po.spmm(a_ref, h)) <= FP32_TOL
+    assert rel_err(ops.spmm(at, h.to(DEV)), po.spmm(at_ref, h)) <= FP32_TOL
