@@ -16,8 +16,12 @@ def rel_err(x, ref):
     """max|x - ref| / max|ref| -- the parity measure of every fp32 / bf16 comparison in this suite."""
     import torch
 
-    x = torch.as_tensor(x).detach().double().cpu()
-    ref = torch.as_tensor(ref).detach().double().cpu()
+    x = torch.as_tensor(x).detach()
+    ref = torch.as_tensor(ref).detach()
+    # compare where the larger operand already lives (full-size tensors stay on the GPU)
+    dev = x.device if x.is_cuda else ref.device
+    x = x.to(dev).double()
+    ref = ref.to(dev).double()
     denom = ref.abs().max().item()
     if denom == 0.0:
         return (x - ref).abs().max().item()

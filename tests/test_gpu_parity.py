@@ -311,6 +311,12 @@ def test_config1_ten_epoch_loss_curve(fuse_relu):
     opt = make_optimizer(model, feats)
     shards = [(g.torch_csr().to(DEV), g.torch_csr(True).to(DEV))]
     losses = run_epochs(model, opt, feats, shards, y.to(DEV), n, 7, 10)
+    import json
+    import os
+    golden = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1_golden.json")))
+    assert g.nnz == golden["nnz"]
+    for l, want in zip(losses, golden["losses_fp64"]):  # the committed fp64 loss curve of the oracle
+        assert abs(l - want) <= FP32_TOL * abs(want)
     print("gpu   ", ["%.6f" % v for v in losses], flush=True)
     print("oracle", ["%.6f" % v for v in ref_losses], flush=True)
     for l, r, r64 in zip(losses, ref_losses, ref64):

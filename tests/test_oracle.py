@@ -298,3 +298,24 @@ def test_csr_pair_construction_and_block():
     assert torch.equal(a.to_dense(), dense[5:15, 0:10])
     assert torch.equal(a_t.to_dense(), dense[5:15, 0:10].t())
     assert po.pad_dimension(10, 4) == 12 and po.pad_dimension(12, 4) == 12 and po.pad_dimension(7, 2, 3) == 12
+
+
+def test_oracle_reproduces_committed_config1_fixture():
+    """Drift guard: the oracle (and the synthetic generator feeding it) still gives the committed result."""
+    import importlib.util
+    import json
+    import os
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_config1_golden", os.path.join(here, "make_config1_golden.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    want = json.load(open(os.path.join(here, "config1_golden.json")))
+    got = mod.compute()
+    for key in ("nnz", "col_checksum", "x_ones", "label_histogram"):
+        assert got[key] == want[key], key
+    assert abs(got["val_sum"] - want["val_sum"]) <= 1e-9 * abs(want["val_sum"])
+    assert np.allclose(got["losses_fp64"], want["losses_fp64"], rtol=1e-10, atol=0)
+    assert np.allclose(got["final_weight_abs_sum"], want["final_weight_abs_sum"], rtol=1e-9)
+    assert abs(got["logits_epoch0_abs_sum"] - want["logits_epoch0_abs_sum"]) <= 1e-9 * want["logits_epoch0_abs_sum"]
+    assert want["losses_fp64"][-1] < want["losses_fp64"][0]
