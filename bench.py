@@ -134,6 +134,24 @@ def main():
         del h, out
     dom = spmm[d_main]
 
+    # ceiling of the memory system for this access pattern: random rows of a table as large as H, nothing else
+    gather_ceiling = None
+    if not bf16:
+        import ctypes
+
+        tab = S.normal_features(n, 128, dev, seed=3)
+        sink = torch.zeros(1, device=dev)
+        done = ctypes.c_int64(0)
+        lib = _lib.load()
+        call = lambda: _lib.check(lib.plx_diag_random_gather_f32(tab.data_ptr(), n, 128, 128, nnz, ctypes.byref(done), sink.data_ptr(),
+                                                                 torch.cuda.current_stream().cuda_stream), "plx_diag_random_gather_f32")
+        ms = time_gpu(call, 2, 5)
+        gather_ceiling = {"GBps": done.value * 512 / ms / 1e6, "table_MB": n * 512 / 1e6, "row_bytes": 512,
+                          "spmm_gather_GBps": nnz * 512 / dom["ms"] / 1e6}
+        print("# random 512-byte row gathers on a %.0f MB table: %.0f GB/s; the SpMM gathers %.0f GB/s of rows of H"
+              % (gather_ceiling["table_MB"], gather_ceiling["GBps"], gather_ceiling["spmm_gather_GBps"]), file=sys.stderr, flush=True)
+        del tab
+
     # ---- the epoch ----
     epoch_ms = None
     epoch_ms_tf = None
@@ -235,6 +253,7 @@ def main():
         "spmm_pct_of_hbm_peak": 100.0 * dom["alg_GBps"] / HBM_PEAK_GBPS,
         "spmm_GFLOPs": dom["GFLOPs"],
         "spmm_gather_model_GBps": dom["gather_GBps"],
+        "random_gather_ceiling": gather_ceiling,
         "spmm_D%d" % d_side: spmm[d_side],
         "prep_ms": {"narrow_indices_and_plan": prep_plan_ms, "device_transpose_and_plan": prep_transpose_ms},
         "epoch_ms": epoch_ms,

@@ -111,6 +111,12 @@ int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H
 int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const float *H,
                           int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
                           void *stream);
+/* Diagnostic for the benchmark, not part of the path: performs about n_gathers reads of uniformly random rows
+ * (D fp32 each, D in {16, 32, 64, 128, 256}) of `table` with the SpMM's load shape and nothing else, so that
+ * timing it gives the memory system's ceiling for this access pattern on a table of this size.
+ * *gathers_done receives the exact count. */
+int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int64_t D, int64_t n_gathers, int64_t *gathers_done,
+                               float *sink, void *stream);
 /* fp32 values, bf16 H and Y (raw uint16 bit patterns), fp32 accumulation, round-to-nearest-even store. */
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
                       uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);

@@ -364,6 +364,47 @@ __global__ void narrow_i64_kernel(int64_t n, const int64_t *__restrict__ src, in
     for (; i < n; i += stride) dst[i] = (int32_t)src[i];
 }
 
+// Diagnostic: what the memory system gives to the access pattern of the SpMM when nothing else is in the
+// way -- uniformly random rows of a dense table, 128-bit loads, G rows per wavefront instruction, 8 loads in
+// flight per lane, row numbers from a hash (no index stream, no arithmetic worth mentioning).
+__device__ __forceinline__ uint32_t mix32(uint32_t x)
+{
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+
+template <int LPR>
+__global__ void __launch_bounds__(256) random_gather_kernel(const float4 *__restrict__ table, uint32_t rows, int64_t ld4, int iters,
+                                                            float *__restrict__ sink)
+{
+    constexpr int G = kWave / LPR;
+    constexpr int U = 8;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = (uint32_t)((blockIdx.x * 256 + threadIdx.x) >> 6);
+    const int g = lane / LPR, t = lane % LPR;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int it = 0; it < iters; it += U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t r = mix32((wave * 1315423911u) ^ (uint32_t)((it + u) * G + g) * 2654435761u) % rows;
+            v[u] = table[(int64_t)r * ld4 + t];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            acc.x += v[u].x;
+            acc.y += v[u].y;
+            acc.z += v[u].z;
+            acc.w += v[u].w;
+        }
+    }
+    if (acc.x + acc.y + acc.z + acc.w == 1.2345678e30f) sink[0] = 1.f;  // keeps the loads alive
+}
+
 int64_t ws_ld(int64_t D) { return (D + 3) / 4 * 4; }
 
 }  // namespace
@@ -656,6 +697,33 @@ int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t 
                           void *stream)
 {
     return spmm_impl<float>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int64_t D, int64_t n_gathers, int64_t *gathers_done,
+                               float *sink, void *stream)
+{
+    PLX_REQUIRE(table && sink && gathers_done, "random_gather: NULL argument");
+    PLX_REQUIRE(rows >= 1 && rows < (1ll << 32) && ld >= D && ld % 4 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0,
+                "random_gather: bad table shape or alignment");
+    PLX_REQUIRE(D == 16 || D == 32 || D == 64 || D == 128 || D == 256, "random_gather: D must be 16, 32, 64, 128 or 256");
+    const int lpr = (int)(D / 4);
+    const int gpi = kWave / lpr;                 // rows per wavefront instruction
+    const int64_t waves = 256ll * 32 * 4;        // 32 workgroups of 4 wavefronts per compute unit
+    int64_t iters = std::max<int64_t>(8, n_gathers / (waves * gpi) / 8 * 8);
+    PLX_REQUIRE(iters < (1ll << 30), "random_gather: too many gathers");
+    *gathers_done = waves * gpi * iters;
+    hipStream_t st = plx::as_stream(stream);
+    const unsigned blocks = (unsigned)(waves / 4);
+    const float4 *t4 = reinterpret_cast<const float4 *>(table);
+    switch (lpr) {
+        case 4: random_gather_kernel<4><<<blocks, 256, 0, st>>>(t4, (uint32_t)rows, ld / 4, (int)iters, sink); break;
+        case 8: random_gather_kernel<8><<<blocks, 256, 0, st>>>(t4, (uint32_t)rows, ld / 4, (int)iters, sink); break;
+        case 16: random_gather_kernel<16><<<blocks, 256, 0, st>>>(t4, (uint32_t)rows, ld / 4, (int)iters, sink); break;
+        case 32: random_gather_kernel<32><<<blocks, 256, 0, st>>>(t4, (uint32_t)rows, ld / 4, (int)iters, sink); break;
+        default: random_gather_kernel<64><<<blocks, 256, 0, st>>>(t4, (uint32_t)rows, ld / 4, (int)iters, sink); break;
+    }
+    PLX_LAUNCH_CHECK("random_gather_kernel");
+    return PLX_OK;
 }
 
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
