@@ -186,13 +186,20 @@ def main():
         losses.append(float(loss))
         print("# epoch: %.2f ms (wall %.2f ms), loss %.4f -> %.4f" % (epoch_ms, wall_ms, losses[0], losses[-1]),
               file=sys.stderr, flush=True)
-        if not bf16:
+        if True:
             # the same epoch with the narrowing last layer computed as A.(H.W) (an option of this build; the
             # reference always aggregates first, and the headline number above keeps the reference's order)
             del model, opt
-            x2 = S.normal_features(n, dims[0], dev, seed=1).reshape(-1).requires_grad_()
-            model2 = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True, association="auto")
-            opt2 = make_optimizer(model2, x2)
+            if bf16:
+                x2_master = S.normal_features(n, dims[0], dev, seed=1).reshape(-1)
+                x2 = x2_master.to(torch.bfloat16).requires_grad_()
+                model2 = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True, dropout=0.5,
+                             dropout_seed=0, association="auto")
+                opt2 = make_optimizer(model2, x2_master, features_bf16=x2)
+            else:
+                x2 = S.normal_features(n, dims[0], dev, seed=1).reshape(-1).requires_grad_()
+                model2 = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True, association="auto")
+                opt2 = make_optimizer(model2, x2)
             for _ in range(args.warmup):
                 train(model2, opt2, x2, shards, y, n, dims[-1])
             e0 = torch.cuda.Event(enable_timing=True)

@@ -110,19 +110,24 @@ class GCNConvFunction(torch.autograd.Function):
     @staticmethod
     def _forward_transform_first(ctx, x, edge_index, edge_index_t, weight, local_features_shape, local_weight_shape,
                                  layer_num, fuse_relu):
-        if x.dtype != torch.float32:
-            raise ValueError("transform-first association is implemented for fp32 storage")
+        bf16 = x.dtype == torch.bfloat16
+        if bf16 and fuse_relu:
+            raise ValueError("transform-first association with bf16 storage is implemented for layers without a fused ReLU")
         timers = get_timers()
         timers.start("gcn conv fwd")
         A = ops.as_csr(edge_index)
         H = x.detach().reshape(local_features_shape)
         W = weight.detach().reshape(local_weight_shape)
         d_out = local_weight_shape[1]
-        d_pad = (d_out + 3) // 4 * 4  # rows of Z padded to 16 bytes so that the gather uses 128-bit loads
+        quantum = 8 if bf16 else 4  # rows of Z padded to 16 bytes so that the gather uses 128-bit loads
+        d_pad = (d_out + quantum - 1) // quantum * quantum
         timers.start("OUT = AGG * W")
-        Z = torch.zeros((H.shape[0], d_pad), dtype=torch.float32, device=H.device) if d_pad != d_out else \
-            torch.empty((H.shape[0], d_pad), dtype=torch.float32, device=H.device)
-        ops.gemm_nn(H, W, out=Z[:, :d_out])
+        alloc = torch.zeros if d_pad != d_out else torch.empty
+        Z = alloc((H.shape[0], d_pad), dtype=x.dtype, device=H.device)
+        if bf16:
+            Z[:, :d_out].copy_(ops.gemm_nt_bf16(H, ops.cast_bf16(W, transpose=True)))
+        else:
+            ops.gemm_nn(H, W, out=Z[:, :d_out])
         timers.stop("OUT = AGG * W")
         timers.start("AGG = A * H")
         OUTp = ops.spmm(A, Z)
@@ -136,7 +141,7 @@ class GCNConvFunction(torch.autograd.Function):
         ctx.x_shape = x.shape
         ctx.layer_num = layer_num
         ctx.fuse_relu = fuse_relu
-        ctx.bf16 = False
+        ctx.bf16 = bf16
         ctx.transform_first = True
         ctx.grad_scale = 1.0
         timers.stop("gcn conv fwd")
@@ -149,10 +154,11 @@ class GCNConvFunction(torch.autograd.Function):
         H, weight, out = ctx.saved_tensors
         W = weight.detach().reshape(ctx.local_weight_shape)
         d_out = ctx.local_weight_shape[1]
-        d_pad = (d_out + 3) // 4 * 4
+        quantum = 8 if ctx.bf16 else 4
+        d_pad = (d_out + quantum - 1) // quantum * quantum
         m = grad_output.shape[0]
-        Gp = torch.zeros((m, d_pad), dtype=torch.float32, device=grad_output.device) if d_pad != d_out else \
-            torch.empty((m, d_pad), dtype=torch.float32, device=grad_output.device)
+        alloc = torch.zeros if d_pad != d_out else torch.empty
+        Gp = alloc((m, d_pad), dtype=grad_output.dtype, device=grad_output.device)
         if ctx.fuse_relu:
             ops.relu_bwd(grad_output, out, out=Gp[:, :d_out])
         else:
@@ -163,12 +169,12 @@ class GCNConvFunction(torch.autograd.Function):
         grad_weight = None
         if ctx.needs_input_grad[3]:
             timers.start("GRAD_W = AGG.T * GRAD_OUT")
-            grad_weight = ops.gemm_tn(H, T).reshape(weight.shape)
+            grad_weight = (ops.gemm_tn_bf16(H, T) if ctx.bf16 else ops.gemm_tn(H, T)).reshape(weight.shape)
             timers.stop("GRAD_W = AGG.T * GRAD_OUT")
         grad_x = None
         if ctx.needs_input_grad[0]:
             timers.start("GRAD_AGG = GRAD_OUT * W.T")
-            grad_x = ops.gemm_nt(T, W).reshape(ctx.x_shape)
+            grad_x = (ops.gemm_nt_bf16(T, ops.cast_bf16(W)) if ctx.bf16 else ops.gemm_nt(T, W)).reshape(ctx.x_shape)
             timers.stop("GRAD_AGG = GRAD_OUT * W.T")
         timers.stop("gcn conv bwd")
         return (grad_x, None, None, grad_weight) + (None,) * 13
@@ -245,6 +251,7 @@ class GCNConv(torch.nn.Module):
         # "auto": transform first when that makes the gathered rows span fewer 128-byte lines (fp32 only)
         if association not in ("reference", "transform_first", "auto"):
             raise ValueError("association must be 'reference', 'transform_first' or 'auto'")
+        # decided on fp32 row lengths; bf16 rows are half as long, which narrows the same layers
         lines = lambda d: (d * 4 + 127) // 128
         self.transform_first = association == "transform_first" or (
             association == "auto" and lines((out_channels + 3) // 4 * 4) < lines(in_channels))
@@ -285,5 +292,5 @@ class GCNConv(torch.nn.Module):
             p,
             self.dropout_seed,
             offset,
-            self.transform_first and x.dtype == torch.float32 and p == 0.0,
+            self.transform_first and p == 0.0 and (x.dtype == torch.float32 or not self.fuse_relu),
         )

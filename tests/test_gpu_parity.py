@@ -609,6 +609,17 @@ def test_bf16_three_layer_network_with_dropout():
     for layer, gw in zip(model.layers, gws_ref):
         assert layer.weight.grad.dtype == torch.float32
         assert rel_err(layer.weight.grad, gw) <= BF16_TOL
+    # the narrowing last layer computed as A.(H.W): same result within the bf16 bar
+    model_tf = Net(3, dims[0], dims[1], dims[-1], weights=ws, fuse_relu=True, dropout=0.5, dropout_seed=seed, association="auto")
+    assert model_tf.layers[2].transform_first and not model_tf.layers[0].transform_first
+    model_tf.train()
+    x_tf = bf(x).to(DEV).requires_grad_()
+    logits_tf = model_tf(x_tf, shards)
+    parallel_cross_entropy(logits_tf, y.to(DEV), 3, n, 47).backward()
+    assert rel_err(logits_tf.float(), ref_logits) <= BF16_TOL
+    assert rel_err(x_tf.grad.float(), gx_ref.reshape(n, dims[0])) <= BF16_TOL
+    for layer, gw in zip(model_tf.layers, gws_ref):
+        assert rel_err(layer.weight.grad, gw) <= BF16_TOL
     # eval mode: no dropout, deterministic
     model.eval()
     e1 = model(xd.detach(), shards)
