@@ -111,6 +111,8 @@ __global__ void __launch_bounds__(256) adamw_kernel(int64_t n, float *__restrict
 }
 
 // AdamW with a bf16 gradient; optionally refreshes a bf16 copy of the parameter in the same pass
+// (14 bytes read and 12 or 14 written per element; VEC4: four elements per lane, 128-bit fp32 and 64-bit bf16 accesses)
+template <bool VEC4>
 __global__ void __launch_bounds__(256) adamw_grad_bf16_kernel(int64_t n, float *__restrict__ p, const uint16_t *__restrict__ g,
                                                               float *__restrict__ m, float *__restrict__ v, float decay,
                                                               float one_minus_b1, float b2, float one_minus_b2,
@@ -118,16 +120,38 @@ __global__ void __launch_bounds__(256) adamw_grad_bf16_kernel(int64_t n, float *
                                                               uint16_t *__restrict__ p16)
 {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const float ge = plx::bf16_to_f32(g[i]);
-        const float me = m[i] + (ge - m[i]) * one_minus_b1;
-        const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
-        const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
-        const float pe = p[i] * decay - step_size * (me / denom);
-        p[i] = pe;
-        m[i] = me;
-        v[i] = ve;
-        if (p16 != nullptr) p16[i] = (uint16_t)plx::f32_to_bf16(pe);
+    const int64_t count = VEC4 ? n / 4 : n;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        if constexpr (VEC4) {
+            float4 pp = reinterpret_cast<float4 *>(p)[i];
+            const uint2 gw = reinterpret_cast<const uint2 *>(g)[i];
+            float4 mm = reinterpret_cast<float4 *>(m)[i];
+            float4 vv = reinterpret_cast<float4 *>(v)[i];
+            const float ge[4] = {__uint_as_float(gw.x << 16), __uint_as_float(gw.x & 0xffff0000u), __uint_as_float(gw.y << 16),
+                                 __uint_as_float(gw.y & 0xffff0000u)};
+            float *pe = &pp.x, *me = &mm.x, *ve = &vv.x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                me[e] = me[e] + (ge[e] - me[e]) * one_minus_b1;
+                ve[e] = ve[e] * b2 + (ge[e] * ge[e]) * one_minus_b2;
+                const float denom = sqrtf(ve[e]) * inv_bc2_sqrt + eps;
+                pe[e] = pe[e] * decay - step_size * (me[e] / denom);
+            }
+            reinterpret_cast<float4 *>(p)[i] = pp;
+            reinterpret_cast<float4 *>(m)[i] = mm;
+            reinterpret_cast<float4 *>(v)[i] = vv;
+            if (p16 != nullptr) reinterpret_cast<uint2 *>(p16)[i] = make_uint2(plx::pack_bf16x2(pp.x, pp.y), plx::pack_bf16x2(pp.z, pp.w));
+        } else {
+            const float ge = plx::bf16_to_f32(g[i]);
+            const float me = m[i] + (ge - m[i]) * one_minus_b1;
+            const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
+            const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
+            const float pe = p[i] * decay - step_size * (me / denom);
+            p[i] = pe;
+            m[i] = me;
+            v[i] = ve;
+            if (p16 != nullptr) p16[i] = (uint16_t)plx::f32_to_bf16(pe);
+        }
     }
 }
 
@@ -207,10 +231,18 @@ int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float
     PLX_REQUIRE(param && grad && exp_avg && exp_avg_sq, "adamw: NULL operand");
     const double bc1 = 1.0 - std::pow((double)beta1, (double)step);
     const double bc2 = 1.0 - std::pow((double)beta2, (double)step);
-    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(n, 256), 256 * 32);
-    adamw_grad_bf16_kernel<<<blocks, 256, 0, plx::as_stream(stream)>>>(n, param, grad, exp_avg, exp_avg_sq, 1.0f - lr * weight_decay,
-                                                                      1.0f - beta1, beta2, 1.0f - beta2, (float)((double)lr / bc1),
-                                                                      (float)(1.0 / std::sqrt(bc2)), eps, param_bf16);
+    const bool v4 = n % 4 == 0 && reinterpret_cast<uintptr_t>(param) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % 8 == 0 &&
+                    reinterpret_cast<uintptr_t>(exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(exp_avg_sq) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(param_bf16) % 8 == 0;
+    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(v4 ? n / 4 : n, 256), 256 * 32);
+    hipStream_t st = plx::as_stream(stream);
+    const float decay = 1.0f - lr * weight_decay, step_size = (float)((double)lr / bc1), inv_bc2_sqrt = (float)(1.0 / std::sqrt(bc2));
+    if (v4)
+        adamw_grad_bf16_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2,
+                                                             1.0f - beta2, step_size, inv_bc2_sqrt, eps, param_bf16);
+    else
+        adamw_grad_bf16_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2,
+                                                              1.0f - beta2, step_size, inv_bc2_sqrt, eps, param_bf16);
     PLX_LAUNCH_CHECK("adamw_grad_bf16_kernel");
     return PLX_OK;
 }

@@ -206,7 +206,8 @@ def test_relu_kernels():
         assert torch.equal(dx.cpu(), dy * (x > 0))
 
 
-@pytest.mark.parametrize("m,c", [(1, 1), (10, 7), (1000, 47), (333, 64), (257, 100), (50, 1000), (4100, 16)])
+@pytest.mark.parametrize("m,c", [(1, 1), (10, 7), (1000, 47), (333, 64), (257, 100), (50, 1000), (4100, 16), (1031, 41), (2055, 63),
+                                 (777, 3), (515, 33)])
 def test_softmax_xent(m, c):
     say("softmax_xent %dx%d" % (m, c))
     gen = torch.Generator().manual_seed(m + c)
@@ -224,10 +225,11 @@ def test_softmax_xent(m, c):
     assert abs(loss.item() - torch.nn.functional.cross_entropy(logits.double(), y).item()) <= FP32_TOL * abs(closs)
 
 
-def test_softmax_xent_special_cases_and_no_mutation():
-    say("softmax_xent masks, padding, gscale")
+@pytest.mark.parametrize("c", [12, 13])  # even: padded-tile kernel; odd: contiguous-copy kernel
+def test_softmax_xent_special_cases_and_no_mutation(c):
+    say("softmax_xent masks, padding, gscale, C=%d" % c)
     gen = torch.Generator().manual_seed(9)
-    m, c = 40, 12
+    m = 40
     logits = torch.randn(m, c, generator=gen)
     y = torch.randint(0, 10, (m,), generator=gen)
     y[3] = -1
@@ -247,6 +249,11 @@ def test_softmax_xent_special_cases_and_no_mutation():
     # row offset shifts the padded-row test
     loss2, _ = ops.softmax_xent(ld, yd, num_nodes, num_classes, row_offset=30)
     assert loss2.item() > loss.item()
+    # the same rows as a strided view of a wider matrix (leading dimension > C)
+    wide = torch.zeros(m, c + 5, device=DEV)
+    wide[:, :c] = ld
+    loss3, dl3 = ops.softmax_xent(wide[:, :c], yd, num_nodes, num_classes, gscale=2.5)
+    assert abs(loss3.item() - closs) <= FP32_TOL * abs(closs) and rel_err(dl3.cpu(), cgrad) <= FP32_TOL
 
 
 def test_gcn_norm_kernel():
@@ -535,7 +542,7 @@ def test_gemm_tn_bf16(m, n, k):
     assert torch.equal(c, ops.gemm_tn_bf16(a.to(DEV), g.to(DEV)).cpu())  # bit-reproducible
 
 
-@pytest.mark.parametrize("m,c", [(10, 7), (1000, 47), (257, 100), (50, 1000)])
+@pytest.mark.parametrize("m,c", [(10, 7), (1000, 47), (257, 100), (50, 1000), (1031, 41), (333, 64)])
 def test_softmax_xent_bf16(m, c):
     say("softmax_xent bf16 %dx%d" % (m, c))
     gen = torch.Generator().manual_seed(m + c)
@@ -548,12 +555,12 @@ def test_softmax_xent_bf16(m, c):
     assert rel_err(dl.float().cpu(), cgrad) <= 2.0 ** -8
 
 
-def test_adamw_bf16_gradient_and_shadow():
-    say("AdamW with bf16 gradient and bf16 shadow")
+@pytest.mark.parametrize("n", [10007, 300 * 1024])  # scalar kernel; four-element vector kernel
+def test_adamw_bf16_gradient_and_shadow(n):
+    say("AdamW with bf16 gradient and bf16 shadow, n=%d" % n)
     from plexus_amd.optim import AdamW
 
     gen = torch.Generator().manual_seed(3)
-    n = 10007
     master0 = torch.randn(n, generator=gen)
     master = master0.clone().to(DEV)
     shadow = bf(master).clone().requires_grad_()
