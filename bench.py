@@ -60,6 +60,7 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the graph (for quick checks)")
     ap.add_argument("--seg-len", type=int, default=0, help="split rows longer than this (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
+    ap.add_argument("--no-cpu-epoch", action="store_true", help="host baseline: time the SpMM only, not a whole epoch")
     ap.add_argument("--spmm-only", action="store_true", help="time only the SpMM kernels")
     ap.add_argument("--spmm-iters", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[3, 5],
@@ -236,6 +237,21 @@ def main():
                "max_rel_err_gpu_vs_cpu": err}
         print("# cpu: %.1f ms per SpMM on %d threads, gpu-vs-cpu max rel err %.2e" % (cpu_s * 1e3, cpu["cores"], err),
               file=sys.stderr, flush=True)
+        del y_cpu, y_gpu, h_cpu
+        if not (args.no_cpu_epoch or args.spmm_only):
+            # one whole epoch of the reference's operator chain on the host (fp32; the bf16 configuration runs
+            # fp32 math there too, without dropout): forward, loss, backward, AdamW over weights and features
+            at_cpu = torch.sparse_csr_tensor(g.rowptr_t.cpu(), g.col_t.cpu(), g.val_t.cpu(), size=(g.shape[1], g.shape[0]))
+            x_cpu = S.normal_features(n, dims[0], dev, seed=1).cpu()
+            y_lab = S.uniform_labels(n, dims[-1], dev, seed=2).cpu()
+            t3 = time.time()
+            cpu_losses, _, _ = po.train_epochs(x_cpu, [w.clone() for w in S.glorot_weights(dims, seed=0)], dims, [(a_cpu, at_cpu)],
+                                               y_lab, n, dims[-1], epochs=1)
+            cpu["epoch_ms"] = (time.time() - t3) * 1e3
+            cpu["epoch_sample"] = "one epoch (forward, loss, backward, AdamW) of the same workload, fp32, timed once without warm-up"
+            cpu["epoch_first_loss"] = cpu_losses[0]
+            print("# cpu: %.0f ms per epoch, first loss %.4f (gpu first loss %.4f)" % (cpu["epoch_ms"], cpu_losses[0], losses[0] if losses else float("nan")),
+                  file=sys.stderr, flush=True)
 
     line = {
         "metric": "SpMM HBM GB/s (% of peak) + GCN fwd+bwd epoch ms on 1 MI355X",
