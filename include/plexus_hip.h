@@ -72,6 +72,20 @@ int plx_coo_block_to_csr_f32(int64_t n_edges, const int64_t *row, const int64_t 
                              int64_t c0, int64_t c1, int32_t *rowptr, int32_t *col_out, float *val_out, int64_t *nnz_host,
                              void *workspace, size_t workspace_bytes, void *stream);
 
+/* Graph preprocessing on the device (plexus/utils/dataset.py:128-243).  The reference permutes the adjacency
+ * matrix with sparse products P.A.P2^T, P[i, perm[i]] = 1 (:137-190), i.e. new[i, j] = old[perm[i], perm2[j]]:
+ * an edge (r, c) moves to (inv_perm[r], inv_perm2[c]).
+ *   plx_invert_permutation_i64: inv[perm[i]] = i.
+ *   plx_relabel_edges_i64: (row_out[e], col_out[e]) = (map_row[row[e]], map_col[col[e]]); an id outside
+ *     [0, n_rows) / [0, n_cols) gives -1, which plx_coo_block_to_csr_f32 then drops.  Outputs may alias inputs.
+ *   plx_csr_to_coo_i64: the edge list (row, col) of a CSR matrix in storage order, int64 as torch edge lists
+ *     are -- the to_edge_index step of :195-199. */
+int plx_invert_permutation_i64(int64_t n, const int64_t *perm, int64_t *inv, void *stream);
+int plx_relabel_edges_i64(int64_t n_edges, const int64_t *row, const int64_t *col, const int64_t *map_row, int64_t n_rows,
+                          const int64_t *map_col, int64_t n_cols, int64_t *row_out, int64_t *col_out, void *stream);
+int plx_csr_to_coo_i64(int64_t M, int64_t nnz, const int32_t *rowptr, const int32_t *col, int64_t *row_out, int64_t *col_out,
+                       void *stream);
+
 /* Host-only row analysis behind plx_spmm_plan_create, exported so it can be tested without a GPU.
  * Rows longer than seg_len are split into ceil(len/seg_len) near-equal segments.  Writes at most
  * `cap_long` row ids to long_rows_host, cap_long+1 entries to seg_first_host and `cap_seg` entries to

@@ -117,6 +117,133 @@ def gcn_norm_csr_values(crow: torch.Tensor, col: torch.Tensor, val: torch.Tensor
 
 
 # --------------------------------------------------------------------------
+# vertex permutation and 2-D partition files (plexus/utils/dataset.py, dataloader.py)
+# --------------------------------------------------------------------------
+def permute_graph(edge_index, edge_weight, x, y, perm, perm2=None, directed=False):
+    """dataset.py:128-236 -- A = P.A.P2^T (and A2 = P2.A.P^T for the double permutation) through the same sparse
+    products with permutation matrices P[i, perm[i]] = 1, then x = x[perm2], y = y[perm], y_2 = y[perm2].
+
+    Returns a dict with the fields the reference stores on its data object.  Without ``perm2`` the single
+    permutation of :189-193 (P2 = P) is applied.
+    """
+    n = x.shape[0]
+    ar = torch.arange(n)
+    ones = torch.ones(n, dtype=torch.float32)
+
+    def pmat(p):
+        return torch.sparse_coo_tensor(torch.stack([ar, p]), ones, (n, n)).to_sparse_csr()
+
+    def to_edges(csr):  # to_edge_index: rows expanded from the row pointer, storage order
+        crow = csr.crow_indices()
+        rows = torch.repeat_interleave(torch.arange(n), crow[1:] - crow[:-1])
+        return torch.stack([rows, csr.col_indices()]), csr.values()
+
+    adj = torch.sparse_coo_tensor(edge_index, edge_weight, (n, n)).to_sparse_csr()
+    if directed:
+        adj = adj.transpose(0, 1).to_sparse_csr()
+    P = pmat(perm)
+    out = {}
+    if perm2 is not None:
+        P2 = pmat(perm2)
+        a1 = torch.sparse.mm(torch.sparse.mm(P, adj), P2.transpose(0, 1).to_sparse_csr())
+        a2 = torch.sparse.mm(torch.sparse.mm(P2, adj), P.transpose(0, 1).to_sparse_csr())
+        out["edge_index"], out["edge_weight"] = to_edges(a1)
+        out["edge_index_2"], out["edge_weight_2"] = to_edges(a2)
+        out["x"] = x[perm2, :]
+        out["y"] = y[perm]
+        out["y_2"] = y[perm2]
+    else:
+        a1 = torch.sparse.mm(torch.sparse.mm(P, adj), P.transpose(0, 1).to_sparse_csr())
+        out["edge_index"], out["edge_weight"] = to_edges(a1)
+        out["x"] = x[perm, :]
+        out["y"] = y[perm]
+    return out
+
+
+def load_partitioned(data_dir: str, num_gcn_layers: int, num_gpus=(1, 1, 1), ranks=(0, 0, 0)):
+    """dataloader.py:47-151 (index ranges), :153-325 (merging partition files), :327-452 (cutting, padding),
+    :454-540 (load) for a partitioned directory, on the host with stock torch operators.
+
+    ``num_gpus`` and ``ranks`` are in the reference's ("z", "x", "y") order (:57).  Returns
+    (adj_shards as torch CSR pairs, flat features, labels, num_nodes, num_features, num_classes).
+    Vertex ids stay int64 when files are merged (the reference concatenates onto an empty fp32 tensor, :163,205,
+    which would turn them into floats).
+    """
+    import glob
+    import os
+
+    double_perm = os.path.exists(os.path.join(data_dir, "edge_index", "1"))
+    parts = len(glob.glob(os.path.join(data_dir, "output_labels", "0", "*.pt")))
+    num_nodes, num_features, num_classes = torch.load(os.path.join(data_dir, "metadata.pt"), weights_only=True)
+
+    nodes_step = pad_dimension(num_nodes, num_gpus[1]) // num_gpus[1]
+    feats_step = pad_dimension(num_features, num_gpus[2], num_gpus[0]) // num_gpus[2]
+    nodes_start, nodes_stop = ranks[1] * nodes_step, (ranks[1] + 1) * nodes_step
+    feats_start, feats_stop = ranks[2] * feats_step, (ranks[2] + 1) * feats_step
+    depth_step = pad_dimension((nodes_stop - nodes_start) * (feats_stop - feats_start), num_gpus[0]) // num_gpus[0]
+    depth_start, depth_stop = ranks[0] * depth_step, (ranks[0] + 1) * depth_step
+    if num_gcn_layers % 3 == 1:
+        lg = 0
+    elif num_gcn_layers % 3 == 2:
+        lg = 2
+    else:
+        lg = 1
+    labels_step = pad_dimension(num_nodes, num_gpus[lg]) // num_gpus[lg]
+    labels_start, labels_stop = ranks[lg] * labels_step, (ranks[lg] + 1) * labels_step
+
+    blocks = []
+    for i in range(min(3, num_gcn_layers)):
+        d1, d2 = ((0, 1), (2, 0), (1, 2))[i]
+        s1 = pad_dimension(num_nodes, num_gpus[d1]) // num_gpus[d1]
+        s2 = pad_dimension(num_nodes, num_gpus[d2]) // num_gpus[d2]
+        blocks.append(((ranks[d1] * s1, (ranks[d1] + 1) * s1), (ranks[d2] * s2, (ranks[d2] + 1) * s2)))
+
+    psize = pad_dimension(num_nodes, parts) // parts
+    fsize = pad_dimension(num_features, parts) // parts
+
+    def covering(start, stop, size):
+        return range(min(start // size, parts), min(((stop - 1) // size) + 1, parts))
+
+    adj_shards = []
+    for layer in range(min(6 if double_perm else 3, num_gcn_layers)):
+        (r0, r1), (c0, c1) = blocks[layer % 3]
+        which = 1 if (double_perm and layer % 2 != 0) else 0
+        idx = torch.empty((2, 0), dtype=torch.int64)
+        val = torch.empty(0)
+        for i in covering(r0, r1, psize):
+            for j in covering(c0, c1, psize):
+                ei, w = torch.load(os.path.join(data_dir, "edge_index", str(which), "%d_%d.pt" % (i, j)), weights_only=True)
+                idx = torch.cat((idx, ei), dim=1)
+                val = torch.cat((val, w), dim=0)
+        adj_shards.append(build_csr_pair(idx, val, (num_nodes, num_nodes), (r0, r1), (c0, c1)))
+
+    merged = None
+    for i in covering(nodes_start, nodes_stop, psize):
+        row = None
+        for j in covering(feats_start, feats_stop, fsize):
+            t = torch.load(os.path.join(data_dir, "input_features", "%d_%d.pt" % (i, j)), weights_only=True)
+            row = t if row is None else torch.cat((row, t), dim=1)
+        merged = row if merged is None else torch.cat((merged, row), dim=0)
+    pn0 = (nodes_start // psize) * psize
+    pf0 = (feats_start // fsize) * fsize
+    if merged is None:
+        merged = torch.zeros(nodes_stop - nodes_start, feats_stop - feats_start)
+        pn0, pf0 = nodes_start, feats_start
+    local = merged[nodes_start - pn0 : nodes_stop - pn0, feats_start - pf0 : feats_stop - pf0]
+    local = F.pad(local, (0, (feats_stop - feats_start) - local.shape[1], 0, (nodes_stop - nodes_start) - local.shape[0]))
+    features = local.reshape(-1)[depth_start:depth_stop]
+
+    which = 1 if (double_perm and num_gcn_layers % 2 == 0) else 0
+    labels = torch.empty(0, dtype=torch.int64)
+    for i in covering(labels_start, labels_stop, psize):
+        labels = torch.cat((labels, torch.load(os.path.join(data_dir, "output_labels", str(which), "%d.pt" % i), weights_only=True)))
+    pl0 = (labels_start // psize) * psize
+    labels = labels[labels_start - pl0 : labels_stop - pl0]
+    labels = F.pad(labels, (0, (labels_stop - labels_start) - labels.shape[0])).to(torch.int64)
+    return adj_shards, features, labels, num_nodes, num_features, num_classes
+
+
+# --------------------------------------------------------------------------
 # plexus/gcn_conv.py
 # --------------------------------------------------------------------------
 def extract_csr_submatrix(csr: torch.Tensor, start_row: int, end_row: int) -> torch.Tensor:

@@ -158,6 +158,14 @@ def csr_pair_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, sha
 
     Counterpart of the loader's ``__split_adj`` (plexus/utils/dataloader.py:327-375): mask the edges to
     ``row_range x col_range``, re-base, build the CSR (duplicates summed) and the CSR of its transpose."""
+    a = csr_from_edges(edge_index, edge_weight, shape, row_range, col_range, seg_len)
+    return a, csr_transpose(a, seg_len)
+
+
+def csr_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, shape, row_range=None, col_range=None,
+                   seg_len: int = 0) -> "CsrMatrix":
+    """The CSR block ``row_range x col_range`` of an edge list (plexus/utils/dataloader.py:343-367): edges outside
+    the block are dropped, the rest re-based, sorted by (row, column) and duplicates summed."""
     _need_gpu(edge_index, edge_weight)
     r0, r1 = row_range if row_range is not None else (0, int(shape[0]))
     c0, c1 = col_range if col_range is not None else (0, int(shape[1]))
@@ -181,8 +189,47 @@ def csr_pair_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, sha
     )
     del ws
     k = int(nnz.value)
-    a = CsrMatrix(rowptr, col_out[:k].clone(), val_out[:k].clone(), (mb, kb), seg_len)
-    return a, csr_transpose(a, seg_len)
+    return CsrMatrix(rowptr, col_out[:k].clone(), val_out[:k].clone(), (mb, kb), seg_len)
+
+
+def invert_permutation(perm: torch.Tensor) -> torch.Tensor:
+    """inv with inv[perm[i]] = i (int64, on the device)."""
+    _need_gpu(perm)
+    perm = perm.to(torch.int64).contiguous()
+    inv = torch.empty_like(perm)
+    check(_lib.load().plx_invert_permutation_i64(perm.numel(), perm.data_ptr(), inv.data_ptr(), _stream()), "plx_invert_permutation_i64")
+    return inv
+
+
+def relabel_edges(edge_index: torch.Tensor, map_row: torch.Tensor, map_col: torch.Tensor) -> torch.Tensor:
+    """Edge list with (row, col) replaced by (map_row[row], map_col[col]) -- the vertex relabelling that the
+    reference writes as P.A.P2^T (plexus/utils/dataset.py:137-190) when the maps are the inverse permutations."""
+    _need_gpu(edge_index, map_row, map_col)
+    ei = edge_index.to(torch.int64).contiguous()
+    map_row = map_row.to(torch.int64).contiguous()
+    map_col = map_col.to(torch.int64).contiguous()
+    out = torch.empty_like(ei)
+    n = int(ei.shape[1])
+    check(
+        _lib.load().plx_relabel_edges_i64(n, ei[0].data_ptr(), ei[1].data_ptr(), map_row.data_ptr(), map_row.numel(),
+                                          map_col.data_ptr(), map_col.numel(), out[0].data_ptr(), out[1].data_ptr(), _stream()),
+        "plx_relabel_edges_i64",
+    )
+    return out
+
+
+def csr_to_edges(a: "CsrMatrix"):
+    """(edge_index int64 [2, nnz], edge_weight) of a CSR matrix in storage order (rows, then columns, ascending),
+    as to_edge_index gives them in plexus/utils/dataset.py:195-216."""
+    a = as_csr(a)
+    nnz = int(a.col.numel())
+    ei = torch.empty((2, nnz), dtype=torch.int64, device=a.col.device)
+    check(
+        _lib.load().plx_csr_to_coo_i64(a.shape[0], nnz, a.rowptr.data_ptr(), a.col.data_ptr() if nnz else None,
+                                       ei[0].data_ptr() if nnz else None, ei[1].data_ptr() if nnz else None, _stream()),
+        "plx_csr_to_coo_i64",
+    )
+    return ei, a.val
 
 
 def as_csr(a, seg_len: int = 0) -> CsrMatrix:

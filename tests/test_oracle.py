@@ -319,3 +319,97 @@ def test_oracle_reproduces_committed_config1_fixture():
     assert np.allclose(got["final_weight_abs_sum"], want["final_weight_abs_sum"], rtol=1e-9)
     assert abs(got["logits_epoch0_abs_sum"] - want["logits_epoch0_abs_sum"]) <= 1e-9 * want["logits_epoch0_abs_sum"]
     assert want["losses_fp64"][-1] < want["losses_fp64"][0]
+
+
+# ---- vertex permutation and the 2-D partition files ----
+def _raw_graph(n=83, pairs=500, seed=11):
+    g = torch.Generator().manual_seed(seed)
+    ei = torch.randint(0, n, (2, pairs), generator=g)
+    w = torch.rand(pairs, generator=g) + 0.1
+    ei_n, w_n = po.gcn_norm(ei, n, w)
+    coo = torch.sparse_coo_tensor(ei_n, w_n, (n, n)).coalesce()  # distinct entries, so dense forms are comparable
+    return coo.indices(), coo.values(), g
+
+
+def test_permutation_by_sparse_products_equals_index_maps():
+    n = 83
+    ei, w, g = _raw_graph(n)
+    x = torch.randn(n, 10, generator=g)
+    y = torch.randint(0, 5, (n,), generator=g)
+    perm, perm2 = torch.randperm(n, generator=g), torch.randperm(n, generator=g)
+    dense = torch.sparse_coo_tensor(ei, w, (n, n)).to_dense()
+    out = po.permute_graph(ei, w, x, y, perm, perm2)
+    d1 = torch.sparse_coo_tensor(out["edge_index"], out["edge_weight"], (n, n)).to_dense()
+    d2 = torch.sparse_coo_tensor(out["edge_index_2"], out["edge_weight_2"], (n, n)).to_dense()
+    assert torch.equal(d1, dense[perm][:, perm2])  # entry (i, j) of the result is entry (perm[i], perm2[j])
+    assert torch.equal(d2, dense[perm2][:, perm])
+    assert torch.equal(out["x"], x[perm2]) and torch.equal(out["y"], y[perm]) and torch.equal(out["y_2"], y[perm2])
+    rows = out["edge_index"][0]
+    assert (rows[1:] >= rows[:-1]).all()  # rows in order; the sparse product leaves the columns of a row unsorted
+    assert torch.unique(rows * n + out["edge_index"][1]).numel() == rows.numel()  # no duplicates
+    # a layer is equivariant: (P A P2^T)(P2 H) = P (A H)
+    h = torch.randn(n, 4, generator=g, dtype=torch.float64)
+    assert torch.allclose(d1.double() @ h[perm2], (dense.double() @ h)[perm], atol=1e-12)
+    # single permutation and the directed case (the transpose is what gets permuted)
+    single = po.permute_graph(ei, w, x, y, perm)
+    ds = torch.sparse_coo_tensor(single["edge_index"], single["edge_weight"], (n, n)).to_dense()
+    assert torch.equal(ds, dense[perm][:, perm]) and torch.equal(single["x"], x[perm])
+    dd = po.permute_graph(ei, w, x, y, perm, perm2, directed=True)
+    assert torch.equal(torch.sparse_coo_tensor(dd["edge_index"], dd["edge_weight"], (n, n)).to_dense(), dense.t()[perm][:, perm2])
+
+
+@pytest.mark.parametrize("parts", [1, 2, 3, 5])
+@pytest.mark.parametrize("layers,num_gpus,ranks", [(3, (1, 1, 1), (0, 0, 0)), (3, (2, 2, 2), (1, 0, 1)), (4, (2, 3, 1), (1, 2, 0)),
+                                                   (2, (1, 2, 4), (0, 1, 3)), (6, (3, 2, 2), (2, 1, 1))])
+def test_partition_files_and_loader_restatement_vs_dense_slicing(tmp_path, parts, layers, num_gpus, ranks):
+    """Files written by the product's partition writer (host code), read back by the oracle's restatement of the
+    loader; both pinned by slicing zero-padded dense matrices."""
+    from plexus_amd.utils import dataset as D
+
+    n, f, classes = 83, 10, 5
+    ei, w, g = _raw_graph(n)
+    x = torch.randn(n, f, generator=g)
+    y = torch.randint(0, classes, (n,), generator=g)
+    perm, perm2 = torch.randperm(n, generator=g), torch.randperm(n, generator=g)
+    pg = po.permute_graph(ei, w, x, y, perm, perm2)
+    graph = D.ProcessedGraph(pg["edge_index"], pg["edge_weight"], pg["x"], pg["y"], classes, pg["edge_index_2"], pg["edge_weight_2"], pg["y_2"])
+    D.partition_graph_2d(graph, parts, str(tmp_path))
+    # layout: exactly the files the reference's loader opens
+    import os
+    assert sorted(os.listdir(tmp_path)) == ["edge_index", "input_features", "metadata.pt", "output_labels"]
+    assert sorted(os.listdir(tmp_path / "edge_index" / "1")) == sorted("%d_%d.pt" % (i, j) for i in range(parts) for j in range(parts))
+    assert torch.load(tmp_path / "metadata.pt", weights_only=True) == (n, f, classes)
+    e00, w00 = torch.load(tmp_path / "edge_index" / "0" / "0_0.pt", weights_only=True)
+    assert e00.dtype == torch.int64 and e00.shape[0] == 2 and w00.dtype == torch.float32
+    total = sum(torch.load(tmp_path / "edge_index" / "0" / ("%d_%d.pt" % (i, j)), weights_only=True)[1].numel()
+                for i in range(parts) for j in range(parts))
+    assert total == graph.edge_weight.numel()  # every edge lands in exactly one file
+
+    shards, feats, labels, nn, nf, nc = po.load_partitioned(str(tmp_path), layers, num_gpus, ranks)
+    assert (nn, nf, nc) == (n, f, classes)
+    big = 2 * n + 16
+    dense = [torch.zeros(big, big), torch.zeros(big, big)]
+    dense[0][:n, :n] = torch.sparse_coo_tensor(pg["edge_index"], pg["edge_weight"], (n, n)).to_dense()
+    dense[1][:n, :n] = torch.sparse_coo_tensor(pg["edge_index_2"], pg["edge_weight_2"], (n, n)).to_dense()
+    groups = [(0, 1), (2, 0), (1, 2)]
+    assert len(shards) == min(6, layers)
+    for layer, (a, at) in enumerate(shards):
+        g1, g2 = groups[layer % 3]
+        s1 = po.pad_dimension(n, num_gpus[g1]) // num_gpus[g1]
+        s2 = po.pad_dimension(n, num_gpus[g2]) // num_gpus[g2]
+        want = dense[layer % 2][ranks[g1] * s1:(ranks[g1] + 1) * s1, ranks[g2] * s2:(ranks[g2] + 1) * s2]
+        assert tuple(a.shape) == (s1, s2) and torch.equal(a.to_dense(), want) and torch.equal(at.to_dense(), want.t())
+    # features: rows of the x group, columns of the y group (padded to y * z), flattened and cut by the depth group
+    ns = po.pad_dimension(n, num_gpus[1]) // num_gpus[1]
+    fs = po.pad_dimension(f, num_gpus[2], num_gpus[0]) // num_gpus[2]
+    xp = torch.zeros(big, big)
+    xp[:n, :f] = pg["x"]
+    slab = xp[ranks[1] * ns:(ranks[1] + 1) * ns, ranks[2] * fs:(ranks[2] + 1) * fs].reshape(-1)
+    ds = slab.numel() // num_gpus[0]
+    assert slab.numel() % num_gpus[0] == 0 and torch.equal(feats, slab[ranks[0] * ds:(ranks[0] + 1) * ds])
+    # labels: the group that splits the rows of the last layer's output; second labels for an even layer count
+    lg = {1: 0, 2: 2, 0: 1}[layers % 3]
+    ls = po.pad_dimension(n, num_gpus[lg]) // num_gpus[lg]
+    yp = torch.zeros(big, dtype=torch.int64)
+    yp[:n] = pg["y_2"] if layers % 2 == 0 else pg["y"]
+    assert torch.equal(labels, yp[ranks[lg] * ls:(ranks[lg] + 1) * ls])
