@@ -41,6 +41,9 @@ SIGNATURES = {
     "plx_diag_random_gather_f32": (C.c_int, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_i64), _vp, _vp]),
     "plx_spmm_csr_bf16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_gemm_nn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp]),
+    "plx_gemm_f32_split_workspace_bytes": (_sz, [_i64, _i64]),
+    "plx_gemm_nn_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp, _sz, _vp]),
+    "plx_gemm_nt_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
@@ -61,6 +64,8 @@ SIGNATURES = {
 
 PLX_GEMM_RELU = 1
 PLX_GEMM_DROPOUT = 2
+# plx_status of include/plexus_hip.h
+PLX_OK, PLX_ERR_INVALID, PLX_ERR_HIP, PLX_ERR_WORKSPACE, PLX_ERR_UNSUPPORTED, PLX_ERR_NOMEM = 0, -1, -2, -3, -4, -5
 
 _lib = None
 

@@ -1,0 +1,345 @@
+// fp32 dense products of the GCN layer on the bf16 matrix cores: every fp32 operand is split exactly into three
+// bf16 pieces, x = x0 + x1 + x2 (8 + 8 + 8 mantissa bits, each piece the round-to-nearest bf16 of what the
+// previous ones left), and the product is accumulated in fp32 from the six piece products
+//     a0.b0 + a0.b1 + a1.b0 + a1.b1 + a0.b2 + a2.b0
+// -- the terms left out (a1.b2, a2.b1, a2.b2) are below 2^-24 of the result, the rounding level of an fp32
+// product.  v_mfma_f32_32x32x16_bf16 runs at 16 times the rate of the fp32 MFMA, so six of them still cost
+// 2.7 times less matrix-core time, which moves these tall-skinny products from the MFMA bound to the HBM bound.
+//
+//   NT form   C[M x N] = epilogue((A*mask)[M x K] . Bp[N x K]^T)     A, mask, C fp32 in memory;
+//             Bp = the three bf16 planes of the small operand, made once per call by split_planes_kernel:
+//               forward   OUT      = AGG . W         Bp = planes of W^T   (+ ReLU)
+//               backward  GRAD_AGG = GRAD_OUT . W^T  Bp = planes of W     (+ ReLU mask on GRAD_OUT)
+//   TN form   C[K x N] = A[M x K]^T . (B*mask)[M x N]                GRAD_W = AGG^T . GRAD_OUT, both operands
+//             split on the fly, tiles transposed on their way into LDS, M split over workgroups with a
+//             fixed-order reduction of the partial tiles.
+//
+// The large operand is read as fp32 with 128-bit loads, split in registers and stored to LDS as three bf16
+// planes; an MFMA lane then reads its 8 consecutive contraction elements of a plane with one 128-bit LDS load.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "bf16.h"
+#include "common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // plain vector type: register arrays of it stay in registers
+
+constexpr int kBM = 128;     // rows of the large operand per workgroup tile
+constexpr int kBK = 32;      // contraction chunk
+constexpr int kS = kBK + 8;  // LDS row stride of a plane in bf16 elements (80 bytes: 128-bit reads conflict-free)
+constexpr int kThreads = 256;
+
+struct SplitArgs {
+    const float *A;
+    const float *mask;
+    const uint16_t *Bp;  // [3][Np][Kp] bf16 planes, zero padded
+    float *C;
+    int64_t lda, ldmask, ldc;
+    int64_t M, N, K;
+    int64_t Np, Kp;
+    unsigned flags;
+    // TN form
+    const float *B;
+    int64_t ldb;
+    int64_t rows_per_split;
+    float *ws;
+    int64_t ws_ld, ws_slab;
+};
+
+// x = p0 + p1 + p2 exactly (bf16 pieces, round to nearest even each); pieces of 2 values packed per word
+__device__ __forceinline__ void split2(float x, float y, uint32_t &p0, uint32_t &p1, uint32_t &p2)
+{
+    p0 = plx::pack_bf16x2(x, y);
+    const float rx = x - __uint_as_float(p0 << 16), ry = y - __uint_as_float(p0 & 0xffff0000u);
+    p1 = plx::pack_bf16x2(rx, ry);
+    const float sx = rx - __uint_as_float(p1 << 16), sy = ry - __uint_as_float(p1 & 0xffff0000u);
+    p2 = plx::pack_bf16x2(sx, sy);
+}
+
+// the three bf16 planes of a small fp32 matrix, optionally transposed: P[p][n][k] = piece p of X(n, k) with
+// X(n, k) = B[k][n] (transpose) or B[n][k]; zero outside N x K
+__global__ void __launch_bounds__(256) split_planes_kernel(const float *__restrict__ B, int64_t ldb, int transpose, int64_t N,
+                                                           int64_t K, int64_t Np, int64_t Kp, uint16_t *__restrict__ P)
+{
+    const int64_t total = Np * Kp;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t n = i / Kp, k = i % Kp;
+        float x = 0.f;
+        if (n < N && k < K) x = transpose ? B[k * ldb + n] : B[n * ldb + k];
+        uint32_t p0, p1, p2;
+        split2(x, 0.f, p0, p1, p2);
+        P[i] = (uint16_t)p0;
+        P[total + i] = (uint16_t)p1;
+        P[2 * total + i] = (uint16_t)p2;
+    }
+}
+
+// six piece products of one 32 x 32 x 16 block, smallest terms first
+__device__ __forceinline__ floatx16 mfma6(bf16x8 a0, bf16x8 a1, bf16x8 a2, bf16x8 b0, bf16x8 b1, bf16x8 b2, floatx16 acc)
+{
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, b0, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc, 0, 0, 0);
+    return acc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// NT form.  Workgroups are persistent: workgroup b takes the row panels b, b + gridDim.x, ... and, per panel,
+// every column tile; the steps (panel, column tile, chunk) form one software pipeline in which the global
+// loads of step q + 1 are in flight while the MFMAs of step q run.  Requires A (and mask) 16-byte aligned
+// with leading dimensions that are multiples of 4, and K % 4 == 0.
+// ------------------------------------------------------------------------------------------------
+template <int TN, bool MASKED>
+__global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitArgs g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr int kAVec = kBM * kBK / 4 / kThreads;  // float4 per thread and chunk of A: 4
+    constexpr int kBItems = 3 * BN * (kBK / 8);      // 16-byte vectors of the three B planes per chunk
+    constexpr int kBVec = (kBItems + kThreads - 1) / kThreads;
+    constexpr int kAPlane = kBM * kS, kBPlane = BN * kS;
+
+    __shared__ __attribute__((aligned(16))) uint16_t lds[3 * kAPlane + 3 * kBPlane];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    const int rt = threadIdx.x >> 3;  // thread (rt, kq) owns float4 kq of rows rt, rt + 32, rt + 64, rt + 96 of a chunk
+    const int kq = threadIdx.x & 7;
+
+    const int64_t n_rp = (g.M + kBM - 1) / kBM;
+    const int n_ct = (int)((g.N + BN - 1) / BN);
+    const int n_kc = (int)((g.K + kBK - 1) / kBK);
+    const int K = (int)g.K;
+    const int64_t my_panels = n_rp > (int64_t)blockIdx.x ? (n_rp - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const int64_t steps = my_panels * n_ct * n_kc;
+    if (steps == 0) return;
+
+    // Step q of the pipeline is (row panel, column tile, chunk), chunk fastest.  A is fetched two steps ahead
+    // (HBM latency), the B planes one step ahead (L2).  Both fetch cursors advance without divisions, and
+    // everything that does not depend on the step (offsets inside a chunk, LDS addresses) is computed once.
+    int64_t a_rp = blockIdx.x;
+    int a_ct = 0, a_kc = 0;
+    int b_ct = 0, b_kc = 0;
+    const int64_t lda32 = 32 * g.lda, ldm32 = 32 * g.ldmask;
+
+    auto fetch_a = [&](float4(&dst)[kAVec]) __attribute__((always_inline)) {
+        const int64_t row = a_rp * kBM + rt;
+        const int k = a_kc * kBK + kq * 4;
+        const int rows_left = (int)min(g.M - row, (int64_t)kBM);  // rows row + 32 p with 32 p < rows_left exist
+        const float *pa = g.A + row * g.lda + k;
+        const float *pm = MASKED ? g.mask + row * g.ldmask + k : nullptr;
+#pragma unroll
+        for (int p = 0; p < kAVec; ++p) {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (32 * p < rows_left && k < K) {
+                v = *reinterpret_cast<const float4 *>(pa);
+                if constexpr (MASKED) {
+                    const float4 m = *reinterpret_cast<const float4 *>(pm);
+                    v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
+                }
+            }
+            dst[p] = v;
+            pa += lda32;
+            if constexpr (MASKED) pm += ldm32;
+        }
+        if (++a_kc == n_kc) {
+            a_kc = 0;
+            if (++a_ct == n_ct) {
+                a_ct = 0;
+                a_rp += gridDim.x;
+            }
+        }
+    };
+
+    // B items of this thread: (plane, row, 16-byte vector) -> offset inside a chunk of the planes / inside LDS
+    int b_goff[kBVec], b_loff[kBVec];
+#pragma unroll
+    for (int j = 0; j < kBVec; ++j) {
+        const int id = min((int)threadIdx.x + j * kThreads, kBItems - 1);  // surplus threads repeat the last item
+        const int plane = id / (BN * 4), rem = id % (BN * 4);
+        b_goff[j] = (int)(plane * g.Np * g.Kp + (int64_t)(rem >> 2) * g.Kp + (rem & 3) * 8);  // planes hold < 2^31 elements
+        b_loff[j] = 3 * kAPlane + plane * kBPlane + (rem >> 2) * kS + (rem & 3) * 8;
+    }
+    u32x4 rb[kBVec];
+    auto fetch_b = [&]() __attribute__((always_inline)) {
+        // planes are zero padded to Np x Kp, so no guards
+        const uint16_t *pb = g.Bp + ((int64_t)b_ct * BN) * g.Kp + b_kc * kBK;
+#pragma unroll
+        for (int j = 0; j < kBVec; ++j) rb[j] = *reinterpret_cast<const u32x4 *>(pb + b_goff[j]);
+        if (++b_kc == n_kc) {
+            b_kc = 0;
+            if (++b_ct == n_ct) b_ct = 0;
+        }
+    };
+    uint16_t *const a_dst = lds + rt * kS + kq * 4;
+    auto stash = [&](const float4(&a)[kAVec]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < kAVec; ++p) {
+            uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
+            split2(a[p].x, a[p].y, lo0, lo1, lo2);
+            split2(a[p].z, a[p].w, hi0, hi1, hi2);
+            uint16_t *dst = a_dst + 32 * p * kS;
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(lo0, hi0);
+            *reinterpret_cast<uint2 *>(dst + kAPlane) = make_uint2(lo1, hi1);
+            *reinterpret_cast<uint2 *>(dst + 2 * kAPlane) = make_uint2(lo2, hi2);
+        }
+#pragma unroll
+        for (int j = 0; j < kBVec; ++j)
+            if ((int)threadIdx.x + j * kThreads < kBItems) *reinterpret_cast<u32x4 *>(lds + b_loff[j]) = rb[j];
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    const uint16_t *const as = lds + (wave * 32 + li) * kS + 8 * h;
+    const uint16_t *const bs = lds + 3 * kAPlane + li * kS + 8 * h;
+    int64_t rp = blockIdx.x;  // the step being computed
+    int ct = 0, kc = 0;
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+
+    auto step = [&](int64_t q, float4(&cur)[kAVec]) __attribute__((always_inline)) {
+        stash(cur);
+        __syncthreads();
+        if (q + 2 < steps) fetch_a(cur);
+        if (q + 1 < steps) fetch_b();
+#pragma unroll
+        for (int s = 0; s < kBK / 16; ++s) {
+            const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(as + 16 * s);
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(as + kAPlane + 16 * s);
+            const bf16x8 a2 = *reinterpret_cast<const bf16x8 *>(as + 2 * kAPlane + 16 * s);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const uint16_t *bt = bs + t * 32 * kS + 16 * s;
+                const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(bt);
+                const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(bt + kBPlane);
+                const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bt + 2 * kBPlane);
+                acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
+            }
+        }
+        if (++kc == n_kc) {
+            // the tile is complete: register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
+            const int64_t r0 = rp * kBM + wave * 32 + 4 * h;
+            const int c0 = ct * BN + li;
+            float *pc = g.C + r0 * g.ldc + c0;
+            const int rows_left = (int)min(g.M - r0, (int64_t)32);  // row r0 + d exists iff d < rows_left
+            const int N = (int)g.N;
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const bool col_ok = c0 + t * 32 < N;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int d = 8 * (v / 4) + (v % 4);
+                    float x = acc[t][v];
+                    if (relu) x = fmaxf(x, 0.f);
+                    if (col_ok && d < rows_left) pc[(int64_t)d * g.ldc + t * 32] = x;
+                    acc[t][v] = 0.f;
+                }
+            }
+            kc = 0;
+            if (++ct == n_ct) {
+                ct = 0;
+                rp += gridDim.x;
+            }
+        }
+        __syncthreads();
+    };
+
+    float4 ra0[kAVec], ra1[kAVec];
+    fetch_a(ra0);
+    fetch_b();
+    if (steps > 1) fetch_a(ra1);
+    for (int64_t q = 0; q < steps; q += 2) {
+        step(q, ra0);
+        if (q + 1 < steps) step(q + 1, ra1);
+    }
+}
+
+int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
+
+template <bool MASKED>
+void launch_nt(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
+{
+    switch (tn) {
+        case 1: gemm_split_nt_kernel<1, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
+        case 2: gemm_split_nt_kernel<2, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
+        default: gemm_split_nt_kernel<4, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
+    }
+}
+
+bool aligned16(const void *p, int64_t ld) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0); }
+
+int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
+
+// C = epilogue((A*mask) . X^T) with X (N x K) = B^T (transpose_b) or B
+int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+            int transpose_b, float *C, int64_t ldc, const float *mask, int64_t ldmask, unsigned flags, void *workspace,
+            size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K > 0 && N < (1ll << 30) && K < (1ll << 30), "%s: bad dimension", who);
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(C != nullptr && A != nullptr && B != nullptr, "%s: NULL operand", who);
+    PLX_REQUIRE(lda >= K && ldc >= N && (mask == nullptr || ldmask >= K), "%s: leading dimension too small", who);
+    PLX_REQUIRE(aligned16(A, lda) && aligned16(mask, ldmask) && K % 4 == 0,
+                "%s: A and mask must be 16-byte aligned with leading dimensions and K multiples of 4", who);
+    const int tn = pick_tn(N);
+    const int64_t Np = round_up(N, 32 * tn), Kp = round_up(std::max<int64_t>(K, 1), kBK);
+    const size_t need = (size_t)3 * Np * Kp * sizeof(uint16_t);
+    if (workspace == nullptr || workspace_bytes < need)
+        return plx::fail(PLX_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+    PLX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "%s: workspace must be 16-byte aligned", who);
+    hipStream_t st = plx::as_stream(stream);
+    uint16_t *planes = static_cast<uint16_t *>(workspace);
+    split_planes_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(Np * Kp, 256), 4096), 256, 0, st>>>(B, ldb, transpose_b, N, K, Np,
+                                                                                                    Kp, planes);
+    PLX_LAUNCH_CHECK("split_planes_kernel");
+    SplitArgs g{};
+    g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
+    g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags;
+    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, kBM), 2 * 256);
+    if (mask != nullptr)
+        launch_nt<true>(g, tn, blocks, st);
+    else
+        launch_nt<false>(g, tn, blocks, st);
+    PLX_LAUNCH_CHECK("gemm_split_nt_kernel");
+    return PLX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t plx_gemm_f32_split_workspace_bytes(int64_t N, int64_t K)
+{
+    if (N <= 0 || K < 0) return 0;
+    const int64_t Np = round_up(N, 32 * pick_tn(N)), Kp = round_up(std::max<int64_t>(K, 1), kBK);
+    return (size_t)3 * Np * Kp * sizeof(uint16_t);
+}
+
+int plx_gemm_nn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                          int64_t ldc, unsigned flags, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(ldb >= N, "gemm_nn_split: leading dimension too small");
+    return nt_form("gemm_nn_split", M, N, K, A, lda, B, ldb, 1, C, ldc, nullptr, 0, flags, workspace, workspace_bytes, stream);
+}
+
+int plx_gemm_nt_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                          int64_t ldc, const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(ldb >= K, "gemm_nt_split: leading dimension too small");
+    return nt_form("gemm_nt_split", M, N, K, A, lda, B, ldb, 0, C, ldc, mask, ldmask, 0u, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

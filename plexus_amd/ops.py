@@ -5,6 +5,7 @@ libplexus_hip.so on the current HIP stream.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -305,6 +306,22 @@ def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk
     return y
 
 
+# fp32 products run on the bf16 matrix cores from exact three-way splits of the operands (fp32-level accuracy)
+# when the operands are aligned for it; PLEXUS_FP32_GEMM=mfma32 keeps every product on the fp32 MFMA kernels.
+SPLIT_GEMM = os.environ.get("PLEXUS_FP32_GEMM", "split") != "mfma32"
+
+
+def _split_ok(k: int, *mats) -> bool:
+    if not SPLIT_GEMM or k <= 0 or k % 4:
+        return False
+    return all(t is None or (t.data_ptr() % 16 == 0 and _ld(t) % 4 == 0) for t in mats)
+
+
+def _split_ws(n: int, k: int, device):
+    need = int(_lib.load().plx_gemm_f32_split_workspace_bytes(n, k))
+    return _aligned_workspace(need, device), need
+
+
 def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix."""
     _need_gpu(a, b, out)
@@ -319,6 +336,14 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
         c = out
         if tuple(c.shape) != (m, n) or c.dtype != torch.float32 or (n > 1 and c.stride(1) != 1):
             raise ValueError("gemm_nn: out must be fp32 [%d x %d] with contiguous rows" % (m, n))
+    if _split_ok(k, a):
+        ws, need = _split_ws(n, k, a.device)
+        check(
+            _lib.load().plx_gemm_nn_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                              PLX_GEMM_RELU if relu else 0, ws.data_ptr(), need, _stream()),
+            "plx_gemm_nn_f32_split",
+        )
+        return c
     check(
         _lib.load().plx_gemm_nn_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
                                     PLX_GEMM_RELU if relu else 0, _stream()),
@@ -340,6 +365,15 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
         if mask.shape != a.shape:
             raise ValueError("gemm_nt: mask shape differs from A")
     c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    if _split_ok(k, a, mask):
+        ws, need = _split_ws(n, k, a.device)
+        check(
+            _lib.load().plx_gemm_nt_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                              mask.data_ptr() if mask is not None else None,
+                                              _ld(mask) if mask is not None else 0, ws.data_ptr(), need, _stream()),
+            "plx_gemm_nt_f32_split",
+        )
+        return c
     check(
         _lib.load().plx_gemm_nt_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
                                     mask.data_ptr() if mask is not None else None,

@@ -131,9 +131,19 @@ GEMM_SHAPES = [(1, 1, 1), (5, 3, 2), (127, 16, 33), (128, 32, 32), (300, 47, 128
                (260, 7, 16), (200, 16, 1433), (150, 256, 256), (64, 130, 70)]
 
 
-@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
-def test_gemm_nn(m, n, k):
-    say("gemm_nn %dx%dx%d" % (m, n, k))
+@pytest.fixture(params=["split", "mfma32"])
+def fp32_gemm_path(request):
+    """Both implementations of the fp32 products: exact three-way bf16 splits on the bf16 matrix cores (taken when
+    the operands are aligned for it) and the fp32 MFMA kernels."""
+    keep = ops.SPLIT_GEMM
+    ops.SPLIT_GEMM = request.param == "split"
+    yield request.param
+    ops.SPLIT_GEMM = keep
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(3000, 128, 96), (777, 48, 128), (2049, 200, 40)])
+def test_gemm_nn(m, n, k, fp32_gemm_path):
+    say("gemm_nn %dx%dx%d %s" % (m, n, k, fp32_gemm_path))
     gen = torch.Generator().manual_seed(m + n + k)
     a = torch.randn(m, k, generator=gen)
     b = torch.randn(k, n, generator=gen)
@@ -145,9 +155,45 @@ def test_gemm_nn(m, n, k):
     assert rel_err(cr, np.maximum(ref, 0)) <= FP32_TOL and (cr >= 0).all()
 
 
-@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
-def test_gemm_nt_and_mask(m, n, k):
-    say("gemm_nt %dx%dx%d" % (m, n, k))
+def test_split_gemm_is_taken_and_keeps_fp32_accuracy_on_hard_inputs():
+    """The split path must not lose what an fp32 product keeps: operands spanning many binades, exact small
+    integers, a column slice as output, and the workspace / alignment contract."""
+    say("split gemm: wide dynamic range, exact integers, contract")
+    from plexus_amd import _lib
+
+    gen = torch.Generator().manual_seed(7)
+    m, k, n = 2000, 128, 64
+    a = torch.randn(m, k, generator=gen) * torch.exp2(torch.randint(-20, 20, (m, 1), generator=gen).float())
+    b = torch.randn(k, n, generator=gen) * torch.exp2(torch.randint(-20, 20, (1, n), generator=gen).float())
+    ref = a.double() @ b.double()
+    got = ops.gemm_nn(a.to(DEV), b.to(DEV)).cpu().double()
+    # row- and column-scaled data: compare element-wise against the scale of each dot product
+    scale = (a.double().abs() @ b.double().abs())
+    err_split = ((got - ref).abs() / scale).max().item()
+    keep, ops.SPLIT_GEMM = ops.SPLIT_GEMM, False
+    err_mfma32 = ((ops.gemm_nn(a.to(DEV), b.to(DEV)).cpu().double() - ref).abs() / scale).max().item()
+    ops.SPLIT_GEMM = keep
+    assert err_split <= 16 * 2.0 ** -24 and err_split <= 2 * err_mfma32  # the level of an fp32 accumulation over K = 128
+    ai = torch.randint(-50, 50, (m, k), generator=gen).float()
+    bi = torch.randint(-50, 50, (k, n), generator=gen).float()
+    assert torch.equal(ops.gemm_nn(ai.to(DEV), bi.to(DEV)).cpu(), ai @ bi)  # integer products below 2^24 are exact
+    wide = torch.zeros(m, n + 8, device=DEV)
+    ops.gemm_nn(ai.to(DEV), bi.to(DEV), out=wide[:, 3:3 + n])
+    assert torch.equal(wide[:, 3:3 + n].cpu(), ai @ bi) and (wide[:, :3] == 0).all() and (wide[:, 3 + n:] == 0).all()
+    lib = _lib.load()
+    need = int(lib.plx_gemm_f32_split_workspace_bytes(n, k))
+    assert need == 3 * 64 * 128 * 2
+    ad, bd, cd = ai.to(DEV), bi.to(DEV), torch.empty(m, n, device=DEV)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.plx_gemm_nn_f32_split(m, n, k, ad.data_ptr(), k, bd.data_ptr(), n, cd.data_ptr(), n, 0, ws.data_ptr(), need - 1, stream) == _lib.PLX_ERR_WORKSPACE
+    assert lib.plx_gemm_nn_f32_split(m, n, k, ad.data_ptr() + 4, k, bd.data_ptr(), n, cd.data_ptr(), n, 0, ws.data_ptr(), need, stream) == _lib.PLX_ERR_INVALID
+    assert lib.plx_gemm_nn_f32_split(m, n, k - 2, ad.data_ptr(), k, bd.data_ptr(), n, cd.data_ptr(), n, 0, ws.data_ptr(), need, stream) == _lib.PLX_ERR_INVALID
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(3000, 128, 96), (777, 48, 128), (2049, 200, 40)])
+def test_gemm_nt_and_mask(m, n, k, fp32_gemm_path):
+    say("gemm_nt %dx%dx%d %s" % (m, n, k, fp32_gemm_path))
     gen = torch.Generator().manual_seed(m * 3 + n + k)
     g = torch.randn(m, k, generator=gen)
     w = torch.randn(n, k, generator=gen)
