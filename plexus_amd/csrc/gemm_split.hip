@@ -267,6 +267,180 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// NT form for a small operand of at most 128 x 128 (the layer widths of the benchmark network): the three
+// planes of B stay in LDS for the life of the workgroup, and every wavefront streams its own 32-row panels
+// of A through a private LDS tile.  There is no workgroup barrier after the planes are loaded, so the eight
+// wavefronts of a workgroup drift apart and the matrix cores of a SIMD run one wavefront's MFMAs while the
+// other wavefront splits and stages its next chunk.  A chunk is 32 rows x 16 contraction elements (two float4
+// per lane); chunks are requested kRing steps before they are used.
+// ------------------------------------------------------------------------------------------------
+constexpr int kRWaves = 8;            // wavefronts per workgroup
+constexpr int kRCK = 16;              // contraction elements per chunk
+constexpr int kRAS = kRCK + 8;        // stride of the private A tile (48 bytes: 128-bit reads conflict-free)
+constexpr int kRMaxK = 128, kRMaxN = 128;
+constexpr int kRBS = kRMaxK + 8;      // stride of the resident B planes (272 bytes)
+constexpr int kRAPlane = 32 * kRAS;   // bf16 elements of one private plane
+constexpr size_t kRLdsBytes = ((size_t)3 * kRMaxN * kRBS + (size_t)kRWaves * 3 * kRAPlane) * sizeof(uint16_t);
+
+template <int TN, bool MASKED>
+__global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel(const SplitArgs g)
+{
+    constexpr int kSteps = kRMaxK / kRCK;   // chunk positions of a panel (positions past K are skipped)
+    constexpr int kRing = MASKED ? 4 : 8;   // register slots = how many positions ahead a chunk is requested
+    extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
+    uint16_t *const bres = rlds;                               // [3][kRMaxN][kRBS]
+    constexpr int kBPlane = kRMaxN * kRBS;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    uint16_t *const apriv = rlds + 3 * kBPlane + wave * 3 * kRAPlane;  // [3][32][kRAS], this wavefront's
+
+    // the planes of B: [3][Np][Kp] in memory -> LDS, 16-byte vectors; rows and columns past Np / Kp stay unread
+    {
+        const int vec_per_row = (int)g.Kp / 8;
+        const int items = 3 * (int)g.Np * vec_per_row;
+        for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
+            const int plane = id / ((int)g.Np * vec_per_row), rem = id % ((int)g.Np * vec_per_row);
+            const int row = rem / vec_per_row, q = rem % vec_per_row;
+            *reinterpret_cast<u32x4 *>(bres + plane * kBPlane + row * kRBS + q * 8) =
+                *reinterpret_cast<const u32x4 *>(g.Bp + ((int64_t)plane * g.Np + row) * g.Kp + q * 8);
+        }
+    }
+    __syncthreads();
+
+    const int K = (int)g.K;
+    const int n_kc = (K + kRCK - 1) / kRCK;
+    const int64_t n_panels = (g.M + 31) / 32;
+    const int64_t first = (int64_t)blockIdx.x * kRWaves + wave, stride = (int64_t)gridDim.x * kRWaves;
+    if (first >= n_panels) return;
+
+    // lane (r, kq) owns float4 kq of rows r and r + 16 of a chunk.  The fetch cursor walks the positions
+    // (panel, 0 .. kSteps - 1) in order and loads the ones that hold data.
+    const int r = lane >> 2, kq = lane & 3;
+    int64_t f_panel = first;
+    int f_kc = 0;
+    const int64_t lda16 = 16 * g.lda, ldm16 = 16 * g.ldmask;
+    float4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
+    auto fetch = [&](float4(&dst)[2], float4(&mdst)[2]) __attribute__((always_inline)) {
+        if (f_kc < n_kc && f_panel < n_panels) {
+            const int64_t row = f_panel * 32 + r;
+            const int k = f_kc * kRCK + kq * 4;
+            const int rows_left = (int)min(g.M - row, (int64_t)32);  // rows row + 16 p with 16 p < rows_left exist
+            const float *pa = g.A + row * g.lda + k;
+            const float *pm = MASKED ? g.mask + row * g.ldmask + k : nullptr;
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f), m = make_float4(1.f, 1.f, 1.f, 1.f);
+                if (16 * p < rows_left && k < K) {
+                    v = *reinterpret_cast<const float4 *>(pa);
+                    if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
+                }
+                dst[p] = v;
+                if constexpr (MASKED) mdst[p] = m;
+                pa += lda16;
+                if constexpr (MASKED) pm += ldm16;
+            }
+        }
+        if (++f_kc == kSteps) {
+            f_kc = 0;
+            f_panel += stride;
+        }
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    uint16_t *const a_dst = apriv + r * kRAS + kq * 4;
+    const uint16_t *const a_src = apriv + li * kRAS + 8 * h;
+    const uint16_t *const b_src = bres + li * kRBS + 8 * h;
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+    const int N = (int)g.N;
+
+    // one position: split the chunk into the private tile, hand its registers to the position kRing ahead, multiply
+    auto step = [&](int kc, float4(&cur)[2], float4(&mcur)[2]) __attribute__((always_inline)) {
+        const bool live = kc < n_kc;
+        if (live) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                float4 v = cur[p];
+                if constexpr (MASKED) {
+                    const float4 m = mcur[p];
+                    v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
+                }
+                uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
+                split2(v.x, v.y, lo0, lo1, lo2);
+                split2(v.z, v.w, hi0, hi1, hi2);
+                uint16_t *dst = a_dst + 16 * p * kRAS;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(lo0, hi0);
+                *reinterpret_cast<uint2 *>(dst + kRAPlane) = make_uint2(lo1, hi1);
+                *reinterpret_cast<uint2 *>(dst + 2 * kRAPlane) = make_uint2(lo2, hi2);
+            }
+        }
+        fetch(cur, mcur);
+        if (live) {
+            const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(a_src);
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(a_src + kRAPlane);
+            const bf16x8 a2 = *reinterpret_cast<const bf16x8 *>(a_src + 2 * kRAPlane);
+            const uint16_t *bk = b_src + kc * kRCK;
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(bk + t * 32 * kRBS);
+                const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(bk + t * 32 * kRBS + kBPlane);
+                const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bk + t * 32 * kRBS + 2 * kBPlane);
+                acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
+            }
+        }
+    };
+
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0]);
+    for (int64_t panel = first; panel < n_panels; panel += stride) {
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+        // the panel is complete: register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
+        const int64_t r0 = panel * 32 + 4 * h;
+        float *pc = g.C + r0 * g.ldc + li;
+        const int rows_left = (int)min(g.M - r0, (int64_t)32);
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+            const bool col_ok = li + t * 32 < N;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int d = 8 * (v / 4) + (v % 4);
+                float x = acc[t][v];
+                if (relu) x = fmaxf(x, 0.f);
+                if (col_ok && d < rows_left) pc[(int64_t)d * g.ldc + t * 32] = x;
+                acc[t][v] = 0.f;
+            }
+        }
+    }
+}
+
+template <int TN, bool MASKED>
+int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
+{
+    // more than 64 KB of dynamic LDS has to be allowed per kernel and device (a host-side setting, cheap to repeat)
+    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASKED>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRLdsBytes));
+    gemm_split_nt_resident_kernel<TN, MASKED><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    return PLX_OK;
+}
+
+template <bool MASKED>
+int launch_resident_tn(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
+{
+    switch (tn) {
+        case 1: return launch_resident<1, MASKED>(g, blocks, st);
+        case 2: return launch_resident<2, MASKED>(g, blocks, st);
+        default: return launch_resident<4, MASKED>(g, blocks, st);
+    }
+}
+
 int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
 
 template <bool MASKED>
@@ -308,6 +482,13 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags;
+    if (Np <= kRMaxN && Kp <= kRMaxK) {
+        const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
+        const int rc = mask != nullptr ? launch_resident_tn<true>(g, tn, blocks, st) : launch_resident_tn<false>(g, tn, blocks, st);
+        if (rc != PLX_OK) return rc;
+        PLX_LAUNCH_CHECK("gemm_split_nt_resident_kernel");
+        return PLX_OK;
+    }
     const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, kBM), 2 * 256);
     if (mask != nullptr)
         launch_nt<true>(g, tn, blocks, st);
