@@ -11,34 +11,47 @@
 
 namespace {
 
-// grid-stride over rows x (cols / 4) float4 lanes when everything is 16-byte aligned, scalars otherwise
-template <bool BWD, bool VEC4>
+// These passes are bound by HBM.  What reaches the highest rates here: one 128-bit item per thread with a grid
+// that covers the tensor (no grid-stride loop), and non-temporal accesses, since nothing is read twice.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_nt(const float *q)
+{
+    const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(q));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void store_nt(float *q, float4 x)
+{
+    const f32x4 t = {x.x, x.y, x.z, x.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4 *>(q));
+}
+
+// one item (float4 when everything is 16-byte aligned, else one element) per thread; FLAT: rows are contiguous
+// in all operands, so the matrix is addressed as one long row without a division
+template <bool BWD, bool VEC4, bool FLAT>
 __global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const float *in, int64_t ldi, const float *ref,
                                                    int64_t ldr, float *out, int64_t ldo)  // out may alias in (or ref)
 {
     const int64_t per_row = VEC4 ? N / 4 : N;
-    const int64_t total = M * per_row;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t r = i / per_row;
-        const int64_t c = (i % per_row) * (VEC4 ? 4 : 1);
-        if constexpr (VEC4) {
-            const float4 x = *reinterpret_cast<const float4 *>(in + r * ldi + c);
-            float4 y;
-            if constexpr (BWD) {
-                const float4 m = *reinterpret_cast<const float4 *>(ref + r * ldr + c);
-                y = make_float4(m.x > 0.f ? x.x : 0.f, m.y > 0.f ? x.y : 0.f, m.z > 0.f ? x.z : 0.f, m.w > 0.f ? x.w : 0.f);
-            } else {
-                y = make_float4(fmaxf(x.x, 0.f), fmaxf(x.y, 0.f), fmaxf(x.z, 0.f), fmaxf(x.w, 0.f));
-            }
-            *reinterpret_cast<float4 *>(out + r * ldo + c) = y;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M * per_row) return;
+    const int64_t r = FLAT ? 0 : i / per_row;
+    const int64_t c = (FLAT ? i : i % per_row) * (VEC4 ? 4 : 1);
+    if constexpr (VEC4) {
+        const float4 x = load_nt(in + r * ldi + c);
+        float4 y;
+        if constexpr (BWD) {
+            const float4 m = load_nt(ref + r * ldr + c);
+            y = make_float4(m.x > 0.f ? x.x : 0.f, m.y > 0.f ? x.y : 0.f, m.z > 0.f ? x.z : 0.f, m.w > 0.f ? x.w : 0.f);
         } else {
-            const float x = in[r * ldi + c];
-            if constexpr (BWD)
-                out[r * ldo + c] = ref[r * ldr + c] > 0.f ? x : 0.f;
-            else
-                out[r * ldo + c] = fmaxf(x, 0.f);
+            y = make_float4(fmaxf(x.x, 0.f), fmaxf(x.y, 0.f), fmaxf(x.z, 0.f), fmaxf(x.w, 0.f));
         }
+        store_nt(out + r * ldo + c, y);
+    } else {
+        const float x = in[r * ldi + c];
+        if constexpr (BWD)
+            out[r * ldo + c] = ref[r * ldr + c] > 0.f ? x : 0.f;
+        else
+            out[r * ldo + c] = fmaxf(x, 0.f);
     }
 }
 
@@ -71,47 +84,45 @@ __global__ void __launch_bounds__(256) gcn_scale_kernel(int64_t M, const int32_t
     for (int j = a + lane; j < b; j += 64) out[j] = (dr * val[j]) * dinv[col[j]];
 }
 
-// one pass over (p, g, m, v): 16 bytes read and 12 written per element
+// one pass over (p, g, m, v): 16 bytes read and 12 written per element; one item per thread
 template <bool VEC4>
 __global__ void __launch_bounds__(256) adamw_kernel(int64_t n, float *__restrict__ p, const float *__restrict__ g,
                                                     float *__restrict__ m, float *__restrict__ v, float decay,
                                                     float one_minus_b1, float b2, float one_minus_b2, float step_size,
                                                     float inv_bc2_sqrt, float eps)
 {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t count = VEC4 ? n / 4 : n;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
-        if constexpr (VEC4) {
-            float4 pp = reinterpret_cast<float4 *>(p)[i];
-            const float4 gg = reinterpret_cast<const float4 *>(g)[i];
-            float4 mm = reinterpret_cast<float4 *>(m)[i];
-            float4 vv = reinterpret_cast<float4 *>(v)[i];
-            float *pe = &pp.x, *me = &mm.x, *ve = &vv.x;
-            const float *ge = &gg.x;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (VEC4 ? n / 4 : n)) return;
+    if constexpr (VEC4) {
+        float4 pp = load_nt(p + 4 * i);
+        const float4 gg = load_nt(g + 4 * i);
+        float4 mm = load_nt(m + 4 * i);
+        float4 vv = load_nt(v + 4 * i);
+        float *pe = &pp.x, *me = &mm.x, *ve = &vv.x;
+        const float *ge = &gg.x;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                me[e] = me[e] + (ge[e] - me[e]) * one_minus_b1;
-                ve[e] = ve[e] * b2 + (ge[e] * ge[e]) * one_minus_b2;
-                const float denom = sqrtf(ve[e]) * inv_bc2_sqrt + eps;
-                pe[e] = pe[e] * decay - step_size * (me[e] / denom);
-            }
-            reinterpret_cast<float4 *>(p)[i] = pp;
-            reinterpret_cast<float4 *>(m)[i] = mm;
-            reinterpret_cast<float4 *>(v)[i] = vv;
-        } else {
-            const float ge = g[i];
-            const float me = m[i] + (ge - m[i]) * one_minus_b1;
-            const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
-            const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
-            p[i] = p[i] * decay - step_size * (me / denom);
-            m[i] = me;
-            v[i] = ve;
+        for (int e = 0; e < 4; ++e) {
+            me[e] = me[e] + (ge[e] - me[e]) * one_minus_b1;
+            ve[e] = ve[e] * b2 + (ge[e] * ge[e]) * one_minus_b2;
+            const float denom = sqrtf(ve[e]) * inv_bc2_sqrt + eps;
+            pe[e] = pe[e] * decay - step_size * (me[e] / denom);
         }
+        store_nt(p + 4 * i, pp);
+        store_nt(m + 4 * i, mm);
+        store_nt(v + 4 * i, vv);
+    } else {
+        const float ge = g[i];
+        const float me = m[i] + (ge - m[i]) * one_minus_b1;
+        const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
+        const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
+        p[i] = p[i] * decay - step_size * (me / denom);
+        m[i] = me;
+        v[i] = ve;
     }
 }
 
 // AdamW with a bf16 gradient; optionally refreshes a bf16 copy of the parameter in the same pass
-// (14 bytes read and 12 or 14 written per element; VEC4: four elements per lane, 128-bit fp32 and 64-bit bf16 accesses)
+// (14 bytes read and 12 or 14 written per element; VEC4: four elements per thread, 128-bit fp32 and 64-bit bf16 accesses)
 template <bool VEC4>
 __global__ void __launch_bounds__(256) adamw_grad_bf16_kernel(int64_t n, float *__restrict__ p, const uint16_t *__restrict__ g,
                                                               float *__restrict__ m, float *__restrict__ v, float decay,
@@ -119,39 +130,37 @@ __global__ void __launch_bounds__(256) adamw_grad_bf16_kernel(int64_t n, float *
                                                               float step_size, float inv_bc2_sqrt, float eps,
                                                               uint16_t *__restrict__ p16)
 {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    const int64_t count = VEC4 ? n / 4 : n;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
-        if constexpr (VEC4) {
-            float4 pp = reinterpret_cast<float4 *>(p)[i];
-            const uint2 gw = reinterpret_cast<const uint2 *>(g)[i];
-            float4 mm = reinterpret_cast<float4 *>(m)[i];
-            float4 vv = reinterpret_cast<float4 *>(v)[i];
-            const float ge[4] = {__uint_as_float(gw.x << 16), __uint_as_float(gw.x & 0xffff0000u), __uint_as_float(gw.y << 16),
-                                 __uint_as_float(gw.y & 0xffff0000u)};
-            float *pe = &pp.x, *me = &mm.x, *ve = &vv.x;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (VEC4 ? n / 4 : n)) return;
+    if constexpr (VEC4) {
+        float4 pp = load_nt(p + 4 * i);
+        const uint2 gw = reinterpret_cast<const uint2 *>(g)[i];
+        float4 mm = load_nt(m + 4 * i);
+        float4 vv = load_nt(v + 4 * i);
+        const float ge[4] = {__uint_as_float(gw.x << 16), __uint_as_float(gw.x & 0xffff0000u), __uint_as_float(gw.y << 16),
+                             __uint_as_float(gw.y & 0xffff0000u)};
+        float *pe = &pp.x, *me = &mm.x, *ve = &vv.x;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                me[e] = me[e] + (ge[e] - me[e]) * one_minus_b1;
-                ve[e] = ve[e] * b2 + (ge[e] * ge[e]) * one_minus_b2;
-                const float denom = sqrtf(ve[e]) * inv_bc2_sqrt + eps;
-                pe[e] = pe[e] * decay - step_size * (me[e] / denom);
-            }
-            reinterpret_cast<float4 *>(p)[i] = pp;
-            reinterpret_cast<float4 *>(m)[i] = mm;
-            reinterpret_cast<float4 *>(v)[i] = vv;
-            if (p16 != nullptr) reinterpret_cast<uint2 *>(p16)[i] = make_uint2(plx::pack_bf16x2(pp.x, pp.y), plx::pack_bf16x2(pp.z, pp.w));
-        } else {
-            const float ge = plx::bf16_to_f32(g[i]);
-            const float me = m[i] + (ge - m[i]) * one_minus_b1;
-            const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
-            const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
-            const float pe = p[i] * decay - step_size * (me / denom);
-            p[i] = pe;
-            m[i] = me;
-            v[i] = ve;
-            if (p16 != nullptr) p16[i] = (uint16_t)plx::f32_to_bf16(pe);
+        for (int e = 0; e < 4; ++e) {
+            me[e] = me[e] + (ge[e] - me[e]) * one_minus_b1;
+            ve[e] = ve[e] * b2 + (ge[e] * ge[e]) * one_minus_b2;
+            const float denom = sqrtf(ve[e]) * inv_bc2_sqrt + eps;
+            pe[e] = pe[e] * decay - step_size * (me[e] / denom);
         }
+        store_nt(p + 4 * i, pp);
+        store_nt(m + 4 * i, mm);
+        store_nt(v + 4 * i, vv);
+        if (p16 != nullptr) reinterpret_cast<uint2 *>(p16)[i] = make_uint2(plx::pack_bf16x2(pp.x, pp.y), plx::pack_bf16x2(pp.z, pp.w));
+    } else {
+        const float ge = plx::bf16_to_f32(g[i]);
+        const float me = m[i] + (ge - m[i]) * one_minus_b1;
+        const float ve = v[i] * b2 + (ge * ge) * one_minus_b2;
+        const float denom = sqrtf(ve) * inv_bc2_sqrt + eps;
+        const float pe = p[i] * decay - step_size * (me / denom);
+        p[i] = pe;
+        m[i] = me;
+        v[i] = ve;
+        if (p16 != nullptr) p16[i] = (uint16_t)plx::f32_to_bf16(pe);
     }
 }
 
@@ -162,21 +171,33 @@ int relu_common(bool bwd, int64_t M, int64_t N, const float *in, int64_t ldi, co
     if (M == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(in && out && (!bwd || ref), "relu: NULL operand");
     PLX_REQUIRE(ldi >= N && ldo >= N && (!bwd || ldr >= N), "relu: leading dimension smaller than N");
+    const bool flat = ldi == N && ldo == N && (!bwd || ldr == N);  // contiguous rows everywhere: one long row
+    if (flat) {
+        N *= M;
+        M = 1;
+        ldi = ldo = ldr = N;
+    }
     const bool v4 = N % 4 == 0 && aligned4(in, ldi) && aligned4(out, ldo) && (!bwd || aligned4(ref, ldr));
     const int64_t total = M * (v4 ? N / 4 : N);
-    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(total, 256), 256 * 32);
+    const int64_t nblocks = plx::ceil_div(total, 256);
+    PLX_REQUIRE(nblocks < (1ll << 31), "relu: tensor too large for one launch");
+    const unsigned blocks = (unsigned)nblocks;
     hipStream_t st = plx::as_stream(stream);
+#define PLX_RELU_LAUNCH(B, V, F) relu_kernel<B, V, F><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo)
     if (bwd) {
-        if (v4)
-            relu_kernel<true, true><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
-        else
-            relu_kernel<true, false><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+        if (v4) {
+            if (flat) PLX_RELU_LAUNCH(true, true, true); else PLX_RELU_LAUNCH(true, true, false);
+        } else {
+            if (flat) PLX_RELU_LAUNCH(true, false, true); else PLX_RELU_LAUNCH(true, false, false);
+        }
     } else {
-        if (v4)
-            relu_kernel<false, true><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
-        else
-            relu_kernel<false, false><<<blocks, 256, 0, st>>>(M, N, in, ldi, ref, ldr, out, ldo);
+        if (v4) {
+            if (flat) PLX_RELU_LAUNCH(false, true, true); else PLX_RELU_LAUNCH(false, true, false);
+        } else {
+            if (flat) PLX_RELU_LAUNCH(false, false, true); else PLX_RELU_LAUNCH(false, false, false);
+        }
     }
+#undef PLX_RELU_LAUNCH
     PLX_LAUNCH_CHECK("relu_kernel");
     return PLX_OK;
 }
@@ -210,7 +231,8 @@ int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, fl
     const bool v4 = n % 4 == 0 && reinterpret_cast<uintptr_t>(param) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(exp_avg_sq) % 16 == 0;
     const int64_t count = v4 ? n / 4 : n;
-    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(count, 256), 256 * 32);
+    PLX_REQUIRE(plx::ceil_div(count, 256) < (1ll << 31), "adamw: tensor too large for one launch");
+    const unsigned blocks = (unsigned)plx::ceil_div(count, 256);
     hipStream_t st = plx::as_stream(stream);
     if (v4)
         adamw_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2, 1.0f - beta2,
@@ -234,7 +256,8 @@ int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float
     const bool v4 = n % 4 == 0 && reinterpret_cast<uintptr_t>(param) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % 8 == 0 &&
                     reinterpret_cast<uintptr_t>(exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(exp_avg_sq) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(param_bf16) % 8 == 0;
-    const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(v4 ? n / 4 : n, 256), 256 * 32);
+    PLX_REQUIRE(plx::ceil_div(v4 ? n / 4 : n, 256) < (1ll << 31), "adamw: tensor too large for one launch");
+    const unsigned blocks = (unsigned)plx::ceil_div(v4 ? n / 4 : n, 256);
     hipStream_t st = plx::as_stream(stream);
     const float decay = 1.0f - lr * weight_decay, step_size = (float)((double)lr / bc1), inv_bc2_sqrt = (float)(1.0 / std::sqrt(bc2));
     if (v4)
