@@ -52,6 +52,97 @@ def time_gpu(fn, warmup, iters):
     return start.elapsed_time(stop) / iters
 
 
+def bench_side_config(args, dev):
+    """Configurations 2 and 4 (parity-test cases; timed here so that the figures quoted for them can be re-measured).
+
+    Config 2: SpMM only on the R-MAT graph (232,965 nodes, about 114.6 M entries), H 232,965 x 602 and x 128;
+    a step is one SpMM at D = 602.  Config 4: one rank's block of a 2 x 2 x 2 grid (rows and columns [0, N/2) of a
+    doubly permuted R-MAT graph with N = 8,388,608), local widths 64 -> 64 -> 64 -> 24; a step is forward, loss and
+    backward of the three layers on that block (no optimizer: the rank's share of an epoch without collectives)."""
+    import torch
+
+    from plexus_amd import ops
+    from plexus_amd.cross_entropy import parallel_cross_entropy
+    from plexus_amd.train import Net
+    from plexus_amd.utils import synthetic as S
+
+    t0 = time.time()
+    g = S.config2_graph(dev, seed=0, scale=args.scale) if args.config == 2 else S.config4_block(dev, seed=0, scale=args.scale)
+    m, k = g.shape
+    nnz = g.nnz
+    stats = g.degree_stats()
+    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape, args.seg_len)
+    torch.cuda.synchronize()
+    print("# graph: %s, long rows %d, segments %d, generated and prepared in %.1f s" % (stats, a.n_long_rows, a.n_segments, time.time() - t0),
+          file=sys.stderr, flush=True)
+    widths = (602, 128) if args.config == 2 else (64,)
+    spmm = {}
+    for d in widths:
+        h = S.normal_features(k, d, dev, seed=d)
+        out = torch.empty(m, d, device=dev)
+        ms = time_gpu(lambda: ops.spmm(a, h, out=out), 5, args.spmm_iters)
+        b = spmm_bytes(m, k, nnz, d)
+        spmm[d] = {"ms": ms, "alg_bytes": b, "alg_GBps": b / ms / 1e6, "GFLOPs": 2.0 * nnz * d / ms / 1e6,
+                   "gather_GBps": (nnz * 8 + (m + 1) * 4 + nnz * d * 4 + m * d * 4) / ms / 1e6}
+        print("# spmm D=%d fp32: %.3f ms, %.1f GB/s algorithmic, %.1f GFLOP/s, gather model %.0f GB/s"
+              % (d, ms, spmm[d]["alg_GBps"], spmm[d]["GFLOPs"], spmm[d]["gather_GBps"]), file=sys.stderr, flush=True)
+        if d == widths[0]:
+            h0, out0 = h, out  # kept for the comparison with the host operator
+        del h, out
+    dom = spmm[widths[0]]
+    step_ms = dom["ms"]
+    extra = {}
+    if args.config == 4 and not args.spmm_only:
+        at = ops.csr_transpose(a, args.seg_len)
+        dims = [64, 64, 64, 24]
+        x = S.normal_features(k, dims[0], dev, seed=1).reshape(-1).requires_grad_()
+        y = S.uniform_labels(m, dims[-1], dev, seed=2)
+        model = Net(3, dims[0], dims[1], dims[-1], weights=S.glorot_weights(dims, seed=0), fuse_relu=True)
+
+        def one_step():
+            x.grad = None
+            for layer in model.layers:
+                layer.weight.grad = None
+            loss = parallel_cross_entropy(model(x, [(a, at)]), y, 3, m, dims[-1])
+            loss.backward()
+            return loss
+
+        step_ms = time_gpu(one_step, args.warmup, args.steps)
+        extra["block_fwd_bwd_ms"] = step_ms
+        print("# block forward + loss + backward (64-64-64-24): %.2f ms" % step_ms, file=sys.stderr, flush=True)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import plexus_oracle as po
+
+        a_cpu = torch.sparse_csr_tensor(g.rowptr.cpu(), g.col.cpu(), g.val.cpu(), size=g.shape)
+        h_cpu = h0.cpu()
+        po.spmm(a_cpu, h_cpu)
+        t2 = time.time()
+        y_cpu = po.spmm(a_cpu, h_cpu)
+        cpu_s = time.time() - t2
+        err = ((ops.spmm(a, h0).cpu().double() - y_cpu.double()).abs().max() / y_cpu.double().abs().max()).item()
+        cpu = {"value": dom["alg_bytes"] / cpu_s / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "the whole SpMM of the workload at D=%d (torch.sparse.mm, fp32, 1 timed run after 1 warm-up)" % widths[0],
+               "ms": cpu_s * 1e3, "GFLOPs": 2.0 * nnz * widths[0] / cpu_s / 1e9, "max_rel_err_gpu_vs_cpu": err}
+        print("# cpu: %.0f ms per SpMM on %d threads, gpu-vs-cpu max rel err %.2e" % (cpu_s * 1e3, cpu["cores"], err), file=sys.stderr, flush=True)
+    what = ("config 2: SpMM only, R-MAT graph, N=%d, nnz=%d (value and step = A.H at D=602)" % (m, nnz) if args.config == 2 else
+            "config 4: one rank's %d x %d block of a 2x2x2 grid, nnz=%d (value = A.H at D=64; step = 3-layer forward + loss + "
+            "backward on the block, widths 64-64-64-24, no collectives)" % (m, k, nnz))
+    line = {"metric": "SpMM HBM GB/s (% of peak) + GCN fwd+bwd epoch ms on 1 MI355X", "value": dom["alg_GBps"], "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_ms, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": what, "rows": m, "cols": k, "nnz": nnz, "max_row_nnz": stats["max_row_nnz"], "scale": args.scale,
+                       "split_rows": a.n_long_rows, "segments": a.n_segments},
+            "spmm": {str(d): v for d, v in spmm.items()},
+            "roofline": {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": dom["alg_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                         "kernel": "spmm_csr_kernel (A.H, D=%d, fp32)" % widths[0], "alg_bytes_per_launch": dom["alg_bytes"],
+                         "avg_launch_ms": dom["ms"]},
+            "cpu_baseline": cpu}
+    line.update(extra)
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -63,8 +154,9 @@ def main():
     ap.add_argument("--no-cpu-epoch", action="store_true", help="host baseline: time the SpMM only, not a whole epoch")
     ap.add_argument("--spmm-only", action="store_true", help="time only the SpMM kernels")
     ap.add_argument("--spmm-iters", type=int, default=20)
-    ap.add_argument("--config", type=int, default=3, choices=[3, 5],
-                    help="3: fp32, 100-128-128-47 (default, the headline workload); 5: bf16 storage, 256-256-256-47, dropout 0.5")
+    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5],
+                    help="3: fp32, 100-128-128-47 (default, the headline workload); 5: bf16 storage, 256-256-256-47, dropout 0.5; "
+                         "2: SpMM only on the R-MAT graph; 4: one rank's block of a 2x2x2 grid")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy (known size) to calibrate profiler byte counters")
     args = ap.parse_args()
@@ -85,6 +177,8 @@ def main():
         sys.exit(2)
     dev = "cuda"
     torch.cuda.set_device(0)
+    if args.config in (2, 4):
+        return bench_side_config(args, dev)
 
     t0 = time.time()
     g = S.config3_graph(dev, seed=0, scale=args.scale)

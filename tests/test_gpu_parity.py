@@ -380,44 +380,66 @@ def test_config1_ten_epoch_loss_curve(fuse_relu):
         assert rel_err(layer.weight, w) <= 1e-4
 
 
-@pytest.mark.parametrize("scale", [0.1, 1.0])
-def test_config3_properties_and_sampled_rows(scale):
-    """The 2.45 M-node power-law configuration (full size and a tenth of it): size-independent
-    properties of the SpMM and a comparison of sampled rows against the fp64-accumulating oracle."""
-    say("config 3 at scale %g: properties" % scale)
-    g = S.config3_graph(DEV, seed=0, scale=scale)
-    n = g.shape[0]
+def spmm_properties_and_sampled_rows(g, d):
+    """Size-independent properties of Y = A.H on a graph held on the device, and sampled rows (the longest, the
+    shortest and random ones) against the fp64-accumulating oracle; only the sampled rows leave the device."""
+    m, k = g.shape
     a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
-    at = ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (n, n))
+    at = ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (k, m))
     print(g.degree_stats(), "long rows", a.n_long_rows, "segments", a.n_segments, flush=True)
-    h = S.normal_features(n, 128, DEV, seed=1)
-    gm = S.normal_features(n, 128, DEV, seed=2)
+    h = S.normal_features(k, d, DEV, seed=1)
+    gm = S.normal_features(m, d, DEV, seed=2)
     y = ops.spmm(a, h)
     # A.1 = row sums
-    ones = torch.ones(n, 4, device=DEV)
-    rows = torch.repeat_interleave(torch.arange(n, device=DEV), g.rowptr[1:] - g.rowptr[:-1])
-    rowsum = torch.zeros(n, dtype=torch.float64, device=DEV).index_add_(0, rows, g.val.double())
+    ones = torch.ones(k, 4, device=DEV)
+    csum = torch.cat([torch.zeros(1, dtype=torch.float64, device=DEV), torch.cumsum(g.val.double(), 0)])  # fp64 prefix sums
+    rowsum = csum[g.rowptr[1:]] - csum[g.rowptr[:-1]]
     assert rel_err(ops.spmm(a, ones)[:, 0], rowsum) <= FP32_TOL
+    del csum, ones
     # adjoint identity <A.H, G> = <H, A^T.G>
     lhs = (y.double() * gm.double()).sum().item()
     rhs = (h.double() * ops.spmm(at, gm).double()).sum().item()
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), (y.double().norm() * gm.double().norm()).item() * 1e-3)
     # linearity
-    y2 = ops.spmm(a, 2.0 * h + gm)
-    assert rel_err(y2, 2.0 * y.double() + ops.spmm(a, gm).double()) <= FP32_TOL
+    y2 = ops.spmm(a, 2.0 * h + gm[:k] if m >= k else 2.0 * h)
+    if m >= k:
+        assert rel_err(y2, 2.0 * y.double() + ops.spmm(a, gm[:k].contiguous()).double()) <= FP32_TOL
+    else:
+        assert rel_err(y2, 2.0 * y.double()) <= FP32_TOL
+    del y2
     # bit reproducibility
     assert torch.equal(y, ops.spmm(a, h))
-    # sampled rows (the longest, the shortest and random ones) against the oracle
     deg = (g.rowptr[1:] - g.rowptr[:-1]).cpu()
     pick = torch.cat([torch.topk(deg, 8).indices, torch.topk(-deg, 8).indices,
-                      torch.randint(0, n, (200,), generator=torch.Generator().manual_seed(0))])
+                      torch.randint(0, m, (200,), generator=torch.Generator().manual_seed(0))])
     sub_counts = deg[pick]
     sub_rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(sub_counts, 0)])
     starts = g.rowptr[pick.to(DEV)]
     idx = torch.repeat_interleave(starts - sub_rowptr[:-1].to(DEV), sub_counts.to(DEV)) + torch.arange(int(sub_rowptr[-1]), device=DEV)
-    ci, va = g.col[idx].cpu(), g.val[idx].cpu()  # only the sampled rows leave the device
+    ci, va = g.col[idx].cpu(), g.val[idx].cpu()
     ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci.numpy(), va.numpy(), h.cpu().numpy())
     assert rel_err(y[pick.to(DEV)].cpu(), ref) <= FP32_TOL
+
+
+@pytest.mark.parametrize("scale", [0.1, 1.0])
+def test_config3_properties_and_sampled_rows(scale):
+    """The 2.45 M-node power-law configuration (full size and a tenth of it): size-independent
+    properties of the SpMM and a comparison of sampled rows against the fp64-accumulating oracle."""
+    say("config 3 at scale %g: properties" % scale)
+    spmm_properties_and_sampled_rows(S.config3_graph(DEV, seed=0, scale=scale), 128)
+
+
+@pytest.mark.parametrize("d", [602, 128])
+def test_config2_full_size_properties_and_sampled_rows(d):
+    """The SpMM-only configuration at full size: R-MAT graph with 232,965 nodes and about 114.6 M entries."""
+    say("config 2 at full size, D=%d: properties" % d)
+    spmm_properties_and_sampled_rows(S.config2_graph(DEV, seed=0), d)
+
+
+def test_config4_full_size_block_properties_and_sampled_rows():
+    """One rank's block of the 2 x 2 x 2 grid at its real shape: 4,194,304 x 4,194,304, about 64 M entries, D = 64."""
+    say("config 4 block at full size, D=64: properties")
+    spmm_properties_and_sampled_rows(S.config4_block(DEV, seed=0), 64)
 
 
 @pytest.mark.parametrize("n", [1, 7, 4096, 100003])
