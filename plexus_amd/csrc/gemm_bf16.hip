@@ -124,23 +124,26 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
     // A is bound by HBM latency, not by the matrix cores (one chunk is 16 MFMAs): all loads of up to
     // kAhead chunks are issued back to back before the first one is consumed.  B (the weight) comes from
     // L2 and keeps the usual one-chunk-ahead prefetch.
-    uint4 ra[kAhead][kAVec], rb[kBVec];
-    auto fetch_a = [&](int k0, uint4(&dst)[kAVec]) {
+    // the mask is kept beside its chunk and applied when the chunk is stored to LDS: applying it at the load
+    // would make every fetch wait for its own data and undo the prefetch
+    uint4 ra[kAhead][kAVec], rm[MASKED ? kAhead : 1][kAVec], rb[kBVec];
+    auto fetch_a = [&](int k0, uint4(&dst)[kAVec], uint4(&mdst)[kAVec]) {
         const int k = k0 + kq * 8;
 #pragma unroll
         for (int p = 0; p < kAVec; ++p) {
-            uint4 v = zero4();
+            uint4 v = zero4(), m = zero4();
             if (32 * p < a_rows && k < K) {
                 if constexpr (VEC) {
                     v = *reinterpret_cast<const uint4 *>(pa + (int64_t)(32 * p) * g.lda + k0);
-                    if constexpr (MASKED) v = mask8(v, *reinterpret_cast<const uint4 *>(pm + (int64_t)(32 * p) * g.ldmask + k0));
+                    if constexpr (MASKED) m = *reinterpret_cast<const uint4 *>(pm + (int64_t)(32 * p) * g.ldmask + k0);
                 } else {
                     const int valid = min(8, K - k);
                     v = load8(pa + (int64_t)(32 * p) * g.lda + k0, valid, g.a_vec);
-                    if constexpr (MASKED) v = mask8(v, load8(pm + (int64_t)(32 * p) * g.ldmask + k0, valid, g.m_vec));
+                    if constexpr (MASKED) m = load8(pm + (int64_t)(32 * p) * g.ldmask + k0, valid, g.m_vec);
                 }
             }
             dst[p] = v;
+            if constexpr (MASKED) mdst[p] = m;
         }
     };
     auto fetch_b = [&](int k0) {
@@ -158,11 +161,11 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
         }
     };
     const int st_off = rt * kS + kq * 8;
-    auto stash = [&](int buf, const uint4(&a)[kAVec]) {
+    auto stash = [&](int buf, const uint4(&a)[kAVec], const uint4(&m)[kAVec]) {
         uint16_t *as = lds + buf * kTile + st_off;
         uint16_t *bs = as + kBM * kS;
 #pragma unroll
-        for (int p = 0; p < kAVec; ++p) *reinterpret_cast<uint4 *>(as + 32 * p * kS) = a[p];
+        for (int p = 0; p < kAVec; ++p) *reinterpret_cast<uint4 *>(as + 32 * p * kS) = MASKED ? mask8(a[p], m[p]) : a[p];
 #pragma unroll
         for (int p = 0; p < kBVec; ++p)
             if (32 * p < BN) *reinterpret_cast<uint4 *>(bs + 32 * p * kS) = rb[p];
@@ -177,9 +180,9 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
     int buf = 0;
     for (int kk = 0; kk < K; kk += kAhead * kBK) {
 #pragma unroll
-        for (int c = 0; c < kAhead; ++c) fetch_a(kk + c * kBK, ra[c]);  // chunks past K come back as zeros
+        for (int c = 0; c < kAhead; ++c) fetch_a(kk + c * kBK, ra[c], rm[MASKED ? c : 0]);  // chunks past K come back as zeros
         fetch_b(kk);
-        stash(buf, ra[0]);
+        stash(buf, ra[0], rm[0]);
         __syncthreads();
 #pragma unroll
         for (int c = 0; c < kAhead; ++c) {
@@ -198,7 +201,7 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
                 }
             }
-            if (more) stash(buf ^ 1, ra[(c + 1) % kAhead]);
+            if (more) stash(buf ^ 1, ra[(c + 1) % kAhead], rm[MASKED ? (c + 1) % kAhead : 0]);
             __syncthreads();
             buf ^= 1;
         }
@@ -292,7 +295,7 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
     const int a_cols = (int)min(max(g.K - row0 - cq0 * 8, (int64_t)0), (int64_t)kBM);  // columns 64 p + e with 64 p + e < a_cols exist
     const int b_cols = (int)min(max(g.N - col0 - cq0 * 8, (int64_t)0), (int64_t)BN);
 
-    uint4 ra[kAItems][2], rb[kBItems][2];
+    uint4 ra[kAItems][2], rb[kBItems][2], rmk[MASKED ? kBItems : 1][2];  // mask applied at the stash, not at the load
     auto fetch = [&](int64_t m0) {
         const int rows_left = (int)min(mend - m0 - 2 * mp, (int64_t)2);  // 2: both rows of the pair exist
 #pragma unroll
@@ -313,18 +316,19 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
         for (int p = 0; p < kBItems; ++p) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint4 v = zero4();
+                uint4 v = zero4(), mk = zero4();
                 if (j < rows_left && 64 * p < b_cols && 64 * p + cq0 * 8 < BN) {
                     if constexpr (VEC) {
                         v = *reinterpret_cast<const uint4 *>(pb + j * g.ldb + 64 * p);
-                        if constexpr (MASKED) v = mask8(v, *reinterpret_cast<const uint4 *>(pm + j * g.ldmask + 64 * p));
+                        if constexpr (MASKED) mk = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask + 64 * p);
                     } else {
                         const int valid = min(8, b_cols - 64 * p);
                         v = load8(pb + j * g.ldb + 64 * p, valid, g.b_vec);
-                        if constexpr (MASKED) v = mask8(v, load8(pm + j * g.ldmask + 64 * p, valid, g.m_vec));
+                        if constexpr (MASKED) mk = load8(pm + j * g.ldmask + 64 * p, valid, g.m_vec);
                     }
                 }
                 rb[p][j] = v;
+                if constexpr (MASKED) rmk[p][j] = mk;
             }
         }
         pa += (int64_t)kBK * g.lda;
@@ -349,7 +353,12 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
         for (int p = 0; p < kAItems; ++p) stash_pair(at, mp, cq0 + 8 * p, ra[p][0], ra[p][1]);
 #pragma unroll
         for (int p = 0; p < kBItems; ++p)
-            if (cq0 + 8 * p < BN / 8) stash_pair(bt, mp, cq0 + 8 * p, rb[p][0], rb[p][1]);
+            if (cq0 + 8 * p < BN / 8) {
+                if constexpr (MASKED)
+                    stash_pair(bt, mp, cq0 + 8 * p, mask8(rb[p][0], rmk[p][0]), mask8(rb[p][1], rmk[p][1]));
+                else
+                    stash_pair(bt, mp, cq0 + 8 * p, rb[p][0], rb[p][1]);
+            }
     };
 
     floatx16 acc[TN];
