@@ -335,7 +335,12 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
     constexpr bool kAContrRows = (MODE == kTN);            // A tile rows are contraction indices (k-major)
     constexpr bool kBContrRows = (MODE != kNT);            // B tile rows are contraction indices
 
-    float4 ra[kAPer], rb[kBPer];
+    // a mask travels beside its chunk and is applied when the chunk is stored to LDS, so that a fetch only issues loads
+    constexpr int kMPer = !MASKED ? 1 : (MODE == kNT ? kAPer : kBPer);
+    float4 ra[kAPer], rb[kBPer], rmask[kMPer];
+    auto masked = [](float4 v, float4 m) {
+        return make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
+    };
     auto fetch = [&]() {
         {
             const float *q = pa;
@@ -345,13 +350,9 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (p * kAPass < a_rows_left && a_cols_left > 0 && (kARows % kAPass == 0 || ar + p * kAPass < kARows)) {
                     v = *reinterpret_cast<const float4 *>(q);
-                    if constexpr (MASKED && MODE == kNT) {
-                        const float4 m = *reinterpret_cast<const float4 *>(mq);
-                        v.x = m.x > 0.f ? v.x : 0.f;
-                        v.y = m.y > 0.f ? v.y : 0.f;
-                        v.z = m.z > 0.f ? v.z : 0.f;
-                        v.w = m.w > 0.f ? v.w : 0.f;
-                    }
+                    if constexpr (MASKED && MODE == kNT) rmask[p] = *reinterpret_cast<const float4 *>(mq);
+                } else if constexpr (MASKED && MODE == kNT) {
+                    rmask[p] = v;
                 }
                 ra[p] = v;
                 q += a_step;
@@ -366,13 +367,9 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (p * kBPass < b_rows_left && b_cols_left > 0 && (kBRows % kBPass == 0 || br + p * kBPass < kBRows)) {
                     v = *reinterpret_cast<const float4 *>(q);
-                    if constexpr (MASKED && MODE == kTN) {
-                        const float4 m = *reinterpret_cast<const float4 *>(mq);
-                        v.x = m.x > 0.f ? v.x : 0.f;
-                        v.y = m.y > 0.f ? v.y : 0.f;
-                        v.z = m.z > 0.f ? v.z : 0.f;
-                        v.w = m.w > 0.f ? v.w : 0.f;
-                    }
+                    if constexpr (MASKED && MODE == kTN) rmask[p] = *reinterpret_cast<const float4 *>(mq);
+                } else if constexpr (MASKED && MODE == kTN) {
+                    rmask[p] = v;
                 }
                 rb[p] = v;
                 q += b_step;
@@ -392,10 +389,12 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
         float *bs = lds + 2 * kASize + buf * kBSize + b_st;
 #pragma unroll
         for (int p = 0; p < kAPer; ++p)
-            if (kARows % kAPass == 0 || ar + p * kAPass < kARows) *reinterpret_cast<float4 *>(as + p * kAPass * kAStride) = ra[p];
+            if (kARows % kAPass == 0 || ar + p * kAPass < kARows)
+                *reinterpret_cast<float4 *>(as + p * kAPass * kAStride) = (MASKED && MODE == kNT) ? masked(ra[p], rmask[MASKED && MODE == kNT ? p : 0]) : ra[p];
 #pragma unroll
         for (int p = 0; p < kBPer; ++p)
-            if (kBRows % kBPass == 0 || br + p * kBPass < kBRows) *reinterpret_cast<float4 *>(bs + p * kBPass * kBStride) = rb[p];
+            if (kBRows % kBPass == 0 || br + p * kBPass < kBRows)
+                *reinterpret_cast<float4 *>(bs + p * kBPass * kBStride) = (MASKED && MODE == kTN) ? masked(rb[p], rmask[MASKED && MODE == kTN ? p : 0]) : rb[p];
     };
 
     floatx16 acc[TN];

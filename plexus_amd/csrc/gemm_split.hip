@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
     int b_ct = 0, b_kc = 0;
     const int64_t lda32 = 32 * g.lda, ldm32 = 32 * g.ldmask;
 
-    auto fetch_a = [&](float4(&dst)[kAVec]) __attribute__((always_inline)) {
+    // the mask travels beside its chunk and is applied when the chunk is split, so that a fetch only issues loads
+    auto fetch_a = [&](float4(&dst)[kAVec], float4(&mdst)[kAVec]) __attribute__((always_inline)) {
         const int64_t row = a_rp * kBM + rt;
         const int k = a_kc * kBK + kq * 4;
         const int rows_left = (int)min(g.M - row, (int64_t)kBM);  // rows row + 32 p with 32 p < rows_left exist
@@ -140,15 +141,13 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
         const float *pm = MASKED ? g.mask + row * g.ldmask + k : nullptr;
 #pragma unroll
         for (int p = 0; p < kAVec; ++p) {
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f), m = v;
             if (32 * p < rows_left && k < K) {
                 v = *reinterpret_cast<const float4 *>(pa);
-                if constexpr (MASKED) {
-                    const float4 m = *reinterpret_cast<const float4 *>(pm);
-                    v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
-                }
+                if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
             }
             dst[p] = v;
+            if constexpr (MASKED) mdst[p] = m;
             pa += lda32;
             if constexpr (MASKED) pm += ldm32;
         }
@@ -182,12 +181,17 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
         }
     };
     uint16_t *const a_dst = lds + rt * kS + kq * 4;
-    auto stash = [&](const float4(&a)[kAVec]) __attribute__((always_inline)) {
+    auto stash = [&](const float4(&a)[kAVec], const float4(&am)[kAVec]) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < kAVec; ++p) {
+            float4 v = a[p];
+            if constexpr (MASKED) {
+                const float4 m = am[p];
+                v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
+            }
             uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
-            split2(a[p].x, a[p].y, lo0, lo1, lo2);
-            split2(a[p].z, a[p].w, hi0, hi1, hi2);
+            split2(v.x, v.y, lo0, lo1, lo2);
+            split2(v.z, v.w, hi0, hi1, hi2);
             uint16_t *dst = a_dst + 32 * p * kS;
             *reinterpret_cast<uint2 *>(dst) = make_uint2(lo0, hi0);
             *reinterpret_cast<uint2 *>(dst + kAPlane) = make_uint2(lo1, hi1);
@@ -210,10 +214,10 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
     int ct = 0, kc = 0;
     const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
 
-    auto step = [&](int64_t q, float4(&cur)[kAVec]) __attribute__((always_inline)) {
-        stash(cur);
+    auto step = [&](int64_t q, float4(&cur)[kAVec], float4(&mcur)[kAVec]) __attribute__((always_inline)) {
+        stash(cur, mcur);
         __syncthreads();
-        if (q + 2 < steps) fetch_a(cur);
+        if (q + 2 < steps) fetch_a(cur, mcur);
         if (q + 1 < steps) fetch_b();
 #pragma unroll
         for (int s = 0; s < kBK / 16; ++s) {
@@ -257,13 +261,13 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
         __syncthreads();
     };
 
-    float4 ra0[kAVec], ra1[kAVec];
-    fetch_a(ra0);
+    float4 ra0[kAVec], ra1[kAVec], m0[kAVec], m1[kAVec];  // m0 / m1 are dead registers without a mask
+    fetch_a(ra0, m0);
     fetch_b();
-    if (steps > 1) fetch_a(ra1);
+    if (steps > 1) fetch_a(ra1, m1);
     for (int64_t q = 0; q < steps; q += 2) {
-        step(q, ra0);
-        if (q + 1 < steps) step(q + 1, ra1);
+        step(q, ra0, m0);
+        if (q + 1 < steps) step(q + 1, ra1, m1);
     }
 }
 
