@@ -44,6 +44,7 @@ struct SplitArgs {
     int64_t M, N, K;
     int64_t Np, Kp;
     unsigned flags;
+    int a_vec;  // A (and mask) 16-byte aligned, leading dimensions and K multiples of 4: 128-bit loads
     // TN form
     const float *B;
     int64_t ldb;
@@ -338,8 +339,21 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             for (int p = 0; p < 2; ++p) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f), m = make_float4(1.f, 1.f, 1.f, 1.f);
                 if (16 * p < rows_left && k < K) {
-                    v = *reinterpret_cast<const float4 *>(pa);
-                    if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
+                    if (g.a_vec) {
+                        v = *reinterpret_cast<const float4 *>(pa);
+                        if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
+                    } else {  // any alignment, any K: element loads
+                        v.x = pa[0];
+                        if (k + 1 < K) v.y = pa[1];
+                        if (k + 2 < K) v.z = pa[2];
+                        if (k + 3 < K) v.w = pa[3];
+                        if constexpr (MASKED) {
+                            m.x = pm[0];
+                            if (k + 1 < K) m.y = pm[1];
+                            if (k + 2 < K) m.z = pm[2];
+                            if (k + 3 < K) m.w = pm[3];
+                        }
+                    }
                 }
                 dst[p] = v;
                 if constexpr (MASKED) mdst[p] = m;
@@ -470,10 +484,12 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     if (M == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(C != nullptr && A != nullptr && B != nullptr, "%s: NULL operand", who);
     PLX_REQUIRE(lda >= K && ldc >= N && (mask == nullptr || ldmask >= K), "%s: leading dimension too small", who);
-    PLX_REQUIRE(aligned16(A, lda) && aligned16(mask, ldmask) && K % 4 == 0,
-                "%s: A and mask must be 16-byte aligned with leading dimensions and K multiples of 4", who);
     const int tn = pick_tn(N);
     const int64_t Np = round_up(N, 32 * tn), Kp = round_up(std::max<int64_t>(K, 1), kBK);
+    const bool vec = aligned16(A, lda) && aligned16(mask, ldmask) && K % 4 == 0;
+    const bool resident = Np <= kRMaxN && Kp <= kRMaxK;  // this kernel also reads A element by element
+    PLX_REQUIRE(vec || resident,
+                "%s: for weights beyond 128 x 128, A and mask must be 16-byte aligned with leading dimensions and K multiples of 4", who);
     const size_t need = (size_t)3 * Np * Kp * sizeof(uint16_t);
     if (workspace == nullptr || workspace_bytes < need)
         return plx::fail(PLX_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -485,8 +501,8 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     PLX_LAUNCH_CHECK("split_planes_kernel");
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
-    g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags;
-    if (Np <= kRMaxN && Kp <= kRMaxK) {
+    g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags; g.a_vec = vec;
+    if (resident) {
         const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
         const int rc = mask != nullptr ? launch_resident_tn<true>(g, tn, blocks, st) : launch_resident_tn<false>(g, tn, blocks, st);
         if (rc != PLX_OK) return rc;

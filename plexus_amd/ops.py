@@ -311,10 +311,12 @@ def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk
 SPLIT_GEMM = os.environ.get("PLEXUS_FP32_GEMM", "split") != "mfma32"
 
 
-def _split_ok(k: int, *mats) -> bool:
-    if not SPLIT_GEMM or k <= 0 or k % 4:
+def _split_ok(n: int, k: int, *mats) -> bool:
+    if not SPLIT_GEMM or k <= 0:
         return False
-    return all(t is None or (t.data_ptr() % 16 == 0 and _ld(t) % 4 == 0) for t in mats)
+    if n <= 128 and k <= 128:  # the kernel for small weights takes any alignment
+        return True
+    return k % 4 == 0 and all(t is None or (t.data_ptr() % 16 == 0 and _ld(t) % 4 == 0) for t in mats)
 
 
 def _split_ws(n: int, k: int, device):
@@ -336,7 +338,7 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
         c = out
         if tuple(c.shape) != (m, n) or c.dtype != torch.float32 or (n > 1 and c.stride(1) != 1):
             raise ValueError("gemm_nn: out must be fp32 [%d x %d] with contiguous rows" % (m, n))
-    if _split_ok(k, a):
+    if _split_ok(n, k, a):
         ws, need = _split_ws(n, k, a.device)
         check(
             _lib.load().plx_gemm_nn_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
@@ -365,7 +367,7 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
         if mask.shape != a.shape:
             raise ValueError("gemm_nt: mask shape differs from A")
     c = torch.empty((m, n), dtype=torch.float32, device=a.device)
-    if _split_ok(k, a, mask):
+    if _split_ok(n, k, a, mask):
         ws, need = _split_ws(n, k, a.device)
         check(
             _lib.load().plx_gemm_nt_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
