@@ -492,22 +492,39 @@ __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ 
                                                       int splits, int64_t rows, int64_t cols, float *__restrict__ C,
                                                       int64_t ldc)
 {
-    __shared__ float part[4][64];
-    const int e_local = threadIdx.x & 63;
-    const int chain = threadIdx.x >> 6;
-    const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
+    // 16 output elements per workgroup, 16 interleaved chains per element (chain j adds the partial tiles
+    // j, j + 16, ... in order); the chains are then added in chain order: the same sum whatever the timing
+    __shared__ float part[16][17];
+    const int e_local = threadIdx.x & 15;
+    const int chain = threadIdx.x >> 4;
+    const int64_t e = (int64_t)blockIdx.x * 16 + e_local;
     const int64_t total = rows * cols;
     float s = 0.f;
     int64_t r = 0, c = 0;
     if (e < total) {
         r = e / cols;
         c = e % cols;
-        const float *p = ws + r * ws_ld + c;
-        for (int i = chain; i < splits; i += 4) s += p[(int64_t)i * ws_slab];
+        const float *p = ws + r * ws_ld + c + (int64_t)chain * ws_slab;
+        const int64_t step = 16 * ws_slab;
+        int i = chain;
+        for (; i + 48 < splits; i += 64) {  // four loads in flight per chain
+            const float v0 = p[0], v1 = p[step], v2 = p[2 * step], v3 = p[3 * step];
+            s = (((s + v0) + v1) + v2) + v3;
+            p += 4 * step;
+        }
+        for (; i < splits; i += 16) {
+            s += p[0];
+            p += step;
+        }
     }
     part[chain][e_local] = s;
     __syncthreads();
-    if (chain == 0 && e < total) C[r * ldc + c] = ((part[0][e_local] + part[1][e_local]) + part[2][e_local]) + part[3][e_local];
+    if (chain == 0 && e < total) {
+        float t = part[0][e_local];
+#pragma unroll
+        for (int j = 1; j < 16; ++j) t += part[j][e_local];
+        C[r * ldc + c] = t;
+    }
 }
 
 int vec_ok(const float *p, int64_t ld) { return (p == nullptr || (reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0)) ? 1 : 0; }
@@ -556,7 +573,7 @@ int check_common(const char *who, int64_t M, int64_t N, int64_t K, const void *A
 int64_t tn_splits(int64_t M, int64_t N, int64_t K)
 {
     const int64_t tiles = plx::ceil_div(K, kBM) * plx::ceil_div(N, 32 * pick_tn(N));
-    int64_t want = std::max<int64_t>(1, 1024 / tiles);
+    int64_t want = std::max<int64_t>(1, 512 / tiles);
     int64_t by_rows = std::max<int64_t>(1, M / 256);
     return std::max<int64_t>(1, std::min(want, by_rows));
 }
@@ -643,7 +660,7 @@ int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
     PLX_LAUNCH_CHECK("gemm_f32_kernel<TN>");
     if (splits > 1) {
         const int64_t total = K * N;
-        gemm_tn_reduce<<<(unsigned)plx::ceil_div(total, 64), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc);
+        gemm_tn_reduce<<<(unsigned)plx::ceil_div(total, 16), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc);
         PLX_LAUNCH_CHECK("gemm_tn_reduce");
     }
     return PLX_OK;
