@@ -143,6 +143,80 @@ def bench_side_config(args, dev):
     print(json.dumps(line), flush=True)
 
 
+def bench_dense_kernels(args, dev):
+    """The dense products, the loss and the optimizer of config 3 (or 5) one by one, at the workload's shapes, with
+    their algorithmic bytes and flops: the kernels that a counter run of this mode profiles."""
+    import torch
+
+    from plexus_amd import ops
+    from plexus_amd.optim import AdamW
+    from plexus_amd.utils import synthetic as S
+
+    m = max(64, int(2449029 * args.scale))
+    bf16 = args.config == 5
+    dims = [256, 256, 256, 47] if bf16 else [100, 128, 128, 47]
+    e = 2 if bf16 else 4
+    rows = []
+
+    def rec(name, fn, bytes_, flops):
+        ms = time_gpu(fn, 3, args.spmm_iters)
+        rows.append({"kernel": name, "ms": ms, "GBps": bytes_ / ms / 1e6, "TFLOPs": flops / ms / 1e9,
+                     "frac_hbm_peak": bytes_ / ms / 1e6 / HBM_PEAK_GBPS})
+        print("# %-44s %7.3f ms  %7.0f GB/s (%4.1f %% of HBM peak)  %6.1f TFLOP/s" % (name, ms, rows[-1]["GBps"], 100 * rows[-1]["frac_hbm_peak"],
+                                                                                 rows[-1]["TFLOPs"]), file=sys.stderr, flush=True)
+
+    for li in range(3):
+        k, n = dims[li], dims[li + 1]
+        last = li == 2
+        if bf16:
+            a = S.normal_features(m, k, dev, seed=li, dtype=torch.bfloat16)
+            g = S.normal_features(m, n, dev, seed=10 + li, dtype=torch.bfloat16)
+            w = torch.randn(k, n, device=dev) * 0.1
+            wt16, w16 = ops.cast_bf16(w, transpose=True), ops.cast_bf16(w)
+            act = torch.relu(S.normal_features(m, n, dev, seed=20 + li)).to(torch.bfloat16)
+            rec("OUT = AGG.W %dx%d bf16%s" % (k, n, "" if last else " +ReLU +dropout"),
+                (lambda: ops.gemm_nt_bf16(a, wt16)) if last else (lambda: ops.gemm_nt_bf16(a, wt16, relu=True, dropout_p=0.5, seed=1, offset=li)),
+                e * m * (k + n), 2.0 * m * k * n)
+            rec("GRAD_AGG = (G*mask).W^T %dx%d bf16" % (n, k), (lambda: ops.gemm_nt_bf16(g, w16)) if last else (lambda: ops.gemm_nt_bf16(g, w16, mask=act, alpha=2.0)),
+                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            rec("GRAD_W = AGG^T.(G*mask) %dx%d bf16" % (k, n), (lambda: ops.gemm_tn_bf16(a, g)) if last else (lambda: ops.gemm_tn_bf16(a, g, mask=act, alpha=2.0)),
+                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+        else:
+            a = S.normal_features(m, k, dev, seed=li)
+            g = S.normal_features(m, n, dev, seed=10 + li)
+            w = torch.randn(k, n, device=dev) * 0.1
+            wt = w.t().contiguous()
+            act = torch.relu(S.normal_features(m, n, dev, seed=20 + li))
+            rec("OUT = AGG.W %dx%d%s" % (k, n, "" if last else " +ReLU"), lambda: ops.gemm_nn(a, w, relu=not last), e * m * (k + n), 2.0 * m * k * n)
+            rec("GRAD_AGG = (G*mask).W^T %dx%d" % (n, k), lambda: ops.gemm_nt(g, w, mask=None if last else act),
+                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            rec("GRAD_W = AGG^T.(G*mask) %dx%d" % (k, n), lambda: ops.gemm_tn(a, g, mask=None if last else act),
+                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            del wt
+        del a, g, act
+    logits = S.normal_features(m, dims[-1], dev, seed=3, dtype=torch.bfloat16 if bf16 else torch.float32)
+    labels = S.uniform_labels(m, dims[-1], dev, seed=2)
+    rec("cross-entropy loss + gradient, %d classes" % dims[-1], lambda: ops.softmax_xent(logits, labels, m, dims[-1]), 2 * e * m * dims[-1] + 8 * m, 0.0)
+    del logits
+    n_feat = m * dims[0]
+    p = torch.randn(n_feat, device=dev).requires_grad_()
+    if bf16:
+        shadow = p.detach().to(torch.bfloat16).requires_grad_()
+        shadow.grad = torch.randn(n_feat, device=dev).to(torch.bfloat16)
+        opt = AdamW([p], lr=3e-3, weight_decay=0.0, shadows=[(p, shadow)])
+        rec("AdamW over the features (fp32 master, bf16 gradient and copy)", opt.step, 30 * n_feat, 0.0)
+    else:
+        p.grad = torch.randn(n_feat, device=dev)
+        opt = AdamW([p], lr=3e-3, weight_decay=0.0)
+        rec("AdamW over the features", opt.step, 28 * n_feat, 0.0)
+    line = {"metric": "dense products, loss and optimizer of the workload, one by one", "value": sum(r["ms"] for r in rows), "unit": "ms",
+            "n_gpus": 1, "steps": args.spmm_iters, "warmup": 3, "ms_per_step": sum(r["ms"] for r in rows), "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+            "config": {"workload": "config %d dense kernels at M=%d, widths %s" % (args.config, m, "-".join(map(str, dims)))},
+            "kernels": rows}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,6 +227,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline")
     ap.add_argument("--no-cpu-epoch", action="store_true", help="host baseline: time the SpMM only, not a whole epoch")
     ap.add_argument("--spmm-only", action="store_true", help="time only the SpMM kernels")
+    ap.add_argument("--dense-only", action="store_true",
+                    help="time the dense products, the loss and the optimizer of the workload one by one (no graph)")
     ap.add_argument("--spmm-iters", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5],
                     help="3: fp32, 100-128-128-47 (default, the headline workload); 5: bf16 storage, 256-256-256-47, dropout 0.5; "
@@ -179,6 +255,8 @@ def main():
     torch.cuda.set_device(0)
     if args.config in (2, 4):
         return bench_side_config(args, dev)
+    if args.dense_only:
+        return bench_dense_kernels(args, dev)
 
     t0 = time.time()
     g = S.config3_graph(dev, seed=0, scale=args.scale)
