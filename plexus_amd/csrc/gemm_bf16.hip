@@ -264,6 +264,170 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
 }
 
 // ------------------------------------------------------------------------------------------------
+// NT for a weight of at most 256 x 256 with aligned operands: B stays in LDS for the life of a 512-thread
+// workgroup and every wavefront streams its own 32-row panels of A through a private LDS tile, so the main
+// loop has no workgroup barrier (the wavefronts of a SIMD overlap one's MFMAs with the other's staging).  A chunk
+// is 32 rows x 32 contraction elements, two 16-byte vectors per lane, requested kRing positions ahead.  The output
+// tile goes through the private tile 16 rows x 32 columns at a time, so that a lane holds 8 consecutive columns of
+// a row for the dropout generator and stores 16 bytes.
+// ------------------------------------------------------------------------------------------------
+constexpr int kRWaves = 8;
+constexpr int kRCK = 32;                 // contraction elements per chunk
+constexpr int kRAS = kRCK + 8;           // stride of the private tile in bf16 elements (80 bytes)
+constexpr int kRMax = 256;               // largest N and K
+constexpr int kRBS = kRMax + 8;          // stride of the resident B (528 bytes)
+constexpr int kRPrivate = 32 * kRAS;     // bf16 elements of a private tile (2,560 bytes; also 16 x 36 floats of staging)
+constexpr int kRCS = 36;                 // fp32 stride of the staged half tile
+constexpr size_t kRLdsBytes = ((size_t)kRMax * kRBS + (size_t)kRWaves * kRPrivate) * sizeof(uint16_t);
+static_assert(16 * kRCS * 4 <= kRPrivate * 2, "staged half tile must fit the private tile");
+
+template <int TN, bool MASKED>
+__global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(const Bf16Args g)
+{
+    constexpr int kSteps = kRMax / kRCK;   // chunk positions of a panel (positions past K are skipped)
+    constexpr int kRing = MASKED ? 4 : 8;  // register slots = positions ahead that a chunk is requested
+    extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
+    uint16_t *const bres = rlds;  // [kRMax][kRBS]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    uint16_t *const apriv = rlds + kRMax * kRBS + wave * kRPrivate;
+    const int K = (int)g.K, N = (int)g.N;
+
+    // B[N x K] -> LDS, zero beyond N and K up to the tile edges that the MFMAs read
+    {
+        const int kp = (K + kRCK - 1) / kRCK * kRCK, vec_per_row = kp / 8;
+        const int items = 32 * TN * vec_per_row;
+        for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
+            const int row = id / vec_per_row, q = id % vec_per_row;
+            uint4 v = zero4();
+            if (row < N && q * 8 < K) v = *reinterpret_cast<const uint4 *>(g.B + (int64_t)row * g.ldb + q * 8);
+            *reinterpret_cast<uint4 *>(bres + row * kRBS + q * 8) = v;
+        }
+    }
+    __syncthreads();
+
+    const int n_kc = (K + kRCK - 1) / kRCK;
+    const int64_t n_panels = (g.M + 31) / 32;
+    const int64_t first = (int64_t)blockIdx.x * kRWaves + wave, stride = (int64_t)gridDim.x * kRWaves;
+    if (first >= n_panels) return;
+
+    // lane (r, half) owns elements 16 half .. 16 half + 15 of row r of a chunk
+    const int r = lane >> 1, half = lane & 1;
+    int64_t f_panel = first;
+    int f_kc = 0;
+    uint4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
+    auto fetch = [&](uint4(&dst)[2], uint4(&mdst)[2]) __attribute__((always_inline)) {
+        if (f_kc < n_kc && f_panel < n_panels) {
+            const int64_t row = f_panel * 32 + r;
+            const int k = f_kc * kRCK + half * 16;
+            const uint16_t *pa = g.A + row * g.lda + k;
+            const uint16_t *pm = MASKED ? g.mask + row * g.ldmask + k : nullptr;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 v = zero4(), m = zero4();
+                if (row < g.M && k + 8 * j < K) {
+                    v = *reinterpret_cast<const uint4 *>(pa + 8 * j);
+                    if constexpr (MASKED) m = *reinterpret_cast<const uint4 *>(pm + 8 * j);
+                }
+                dst[j] = v;
+                if constexpr (MASKED) mdst[j] = m;
+            }
+        }
+        if (++f_kc == kSteps) {
+            f_kc = 0;
+            f_panel += stride;
+        }
+    };
+
+    floatx16 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+    uint16_t *const a_dst = apriv + r * kRAS + half * 16;
+    const uint16_t *const a_src = apriv + li * kRAS + 8 * h;
+    const uint16_t *const b_src = bres + li * kRBS + 8 * h;
+
+    auto step = [&](int kc, uint4(&cur)[2], uint4(&mcur)[2]) __attribute__((always_inline)) {
+        const bool live = kc < n_kc;
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                *reinterpret_cast<uint4 *>(a_dst + 8 * j) = MASKED ? mask8(cur[j], mcur[MASKED ? j : 0]) : cur[j];
+        }
+        fetch(cur, mcur);
+        if (live) {
+#pragma unroll
+            for (int s = 0; s < kRCK / 16; ++s) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8 *>(a_src + 16 * s);
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    const bf16x8 b = *reinterpret_cast<const bf16x8 *>(b_src + t * 32 * kRBS + kc * kRCK + 16 * s);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
+    const bool drop = (g.flags & PLX_GEMM_DROPOUT) != 0;
+    uint16_t *const C = static_cast<uint16_t *>(g.C);
+    float *const cs = reinterpret_cast<float *>(apriv);
+    const int srow = lane >> 2, scq = lane & 3;  // staged half tile: this lane reads 8 columns of row srow
+
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0]);
+    for (int64_t panel = first; panel < n_panels; panel += stride) {
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+        // register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) cs[(8 * (v / 4) + 4 * h + (v % 4)) * kRCS + li] = acc[t][8 * pass + v];
+                const float4 lo = *reinterpret_cast<const float4 *>(cs + srow * kRCS + scq * 8);
+                const float4 hi = *reinterpret_cast<const float4 *>(cs + srow * kRCS + scq * 8 + 4);
+                const int64_t row = panel * 32 + 16 * pass + srow;
+                const int col = t * 32 + scq * 8;
+                if (row < g.M && col < N) {
+                    float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        x[e] *= g.alpha;
+                        if (relu) x[e] = fmaxf(x[e], 0.f);
+                    }
+                    if (drop) {
+                        const uint64_t q = ((uint64_t)row * (uint64_t)N + (uint64_t)col) >> 3;  // N % 8 == 0: 8 aligned elements
+                        const plx::Philox4 rnd = plx::philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), g.off_lo, g.off_hi, g.seed_lo, g.seed_hi);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) x[e] = plx::dropout_lane16(rnd, e) >= g.thresh16 ? x[e] * g.keep_scale : 0.f;
+                    }
+                    *reinterpret_cast<uint4 *>(C + row * g.ldc + col) = make_uint4(plx::pack_bf16x2(x[0], x[1]), plx::pack_bf16x2(x[2], x[3]),
+                                                                                   plx::pack_bf16x2(x[4], x[5]), plx::pack_bf16x2(x[6], x[7]));
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+        }
+    }
+}
+
+template <int TN, bool MASKED>
+int launch_nt_resident(const Bf16Args &g, unsigned blocks, hipStream_t st)
+{
+    // more than 64 KB of dynamic LDS has to be allowed per kernel and device (a host-side setting, cheap to repeat)
+    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRLdsBytes));
+    gemm_bf16_nt_resident_kernel<TN, MASKED><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    return PLX_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
 // TN: C[K x N] (fp32) = alpha * A[M x K]^T . (B*mask)[M x N]; contraction over the rows of both
 // ------------------------------------------------------------------------------------------------
 template <int TN, bool MASKED, bool VEC>
@@ -529,6 +693,23 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     dim3 grid((unsigned)blocks, 1, 1);
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0;
     hipStream_t st = plx::as_stream(stream);
+    if (vec && g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0) {
+        const unsigned rblocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
+        const int rtn = (int)plx::ceil_div(N, 32);
+        int rc = PLX_OK;
+#define PLX_RES(T_) (mask != nullptr ? launch_nt_resident<T_, true>(g, rblocks, st) : launch_nt_resident<T_, false>(g, rblocks, st))
+        switch (rtn) {
+            case 1: rc = PLX_RES(1); break;
+            case 2: rc = PLX_RES(2); break;
+            case 3: case 4: rc = PLX_RES(4); break;
+            case 5: case 6: rc = PLX_RES(6); break;
+            default: rc = PLX_RES(8); break;
+        }
+#undef PLX_RES
+        if (rc != PLX_OK) return rc;
+        PLX_LAUNCH_CHECK("gemm_bf16_nt_resident_kernel");
+        return PLX_OK;
+    }
     if (mask != nullptr) {
         if (vec) launch_nt<true, true>(g, tn, grid, st);
         else launch_nt<true, false>(g, tn, grid, st);
