@@ -264,7 +264,7 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_nt_kernel(const Bf16Args g
 }
 
 // ------------------------------------------------------------------------------------------------
-// NT for a weight of at most 256 x 256 with aligned operands: B stays in LDS for the life of a 512-thread
+// NT for a weight of at most 256 x 256 and an output that allows 16-byte stores: B stays in LDS for the life of a 512-thread
 // workgroup and every wavefront streams its own 32-row panels of A through a private LDS tile, so the main
 // loop has no workgroup barrier (the wavefronts of a SIMD overlap one's MFMAs with the other's staging).  A chunk
 // is 32 rows x 32 contraction elements, two 16-byte vectors per lane, requested kRing positions ahead.  The output
@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
         for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
             const int row = id / vec_per_row, q = id % vec_per_row;
             uint4 v = zero4();
-            if (row < N && q * 8 < K) v = *reinterpret_cast<const uint4 *>(g.B + (int64_t)row * g.ldb + q * 8);
+            if (row < N && q * 8 < K) v = load8(g.B + (int64_t)row * g.ldb + q * 8, min(8, K - q * 8), g.b_vec);
             *reinterpret_cast<uint4 *>(bres + row * kRBS + q * 8) = v;
         }
     }
@@ -327,9 +327,10 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 uint4 v = zero4(), m = zero4();
-                if (row < g.M && k + 8 * j < K) {
-                    v = *reinterpret_cast<const uint4 *>(pa + 8 * j);
-                    if constexpr (MASKED) m = *reinterpret_cast<const uint4 *>(pm + 8 * j);
+                if (row < g.M && k + 8 * j < K) {  // element loads when an operand does not allow 16-byte ones
+                    const int valid = min(8, K - k - 8 * j);
+                    v = load8(pa + 8 * j, valid, g.a_vec);
+                    if constexpr (MASKED) m = load8(pm + 8 * j, valid, g.m_vec);
                 }
                 dst[j] = v;
                 if constexpr (MASKED) mdst[j] = m;
@@ -693,7 +694,7 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     dim3 grid((unsigned)blocks, 1, 1);
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0;
     hipStream_t st = plx::as_stream(stream);
-    if (vec && g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0) {
+    if (g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0) {
         const unsigned rblocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
         const int rtn = (int)plx::ceil_div(N, 32);
         int rc = PLX_OK;
