@@ -57,31 +57,75 @@ __global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const f
 
 bool aligned4(const void *p, int64_t ld) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0; }
 
-// one wavefront per row: dinv[r] = 1 / sqrt(sum of row r), 0 for an empty or zero row
+// d^-1/2 of the row sums.  A wavefront sums one row; rows longer than kLongRow entries (the hubs of a power-law
+// graph: one row of the benchmark graph holds 1.1 M entries) are left to the whole workgroup afterwards, with four
+// loads in flight per thread.  Both orders of summation are fixed.
+constexpr int kLongRow = 4096;
+
 __global__ void __launch_bounds__(256) row_dinv_kernel(int64_t M, const int32_t *__restrict__ rowptr,
                                                        const float *__restrict__ val, float *__restrict__ dinv)
 {
+    __shared__ float part[4];
     const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= M) return;
-    const int a = rowptr[r], b = rowptr[r + 1];
-    float s = 0.f;
-    for (int j = a + lane; j < b; j += 64) s += val[j];
+    const int wave = threadIdx.x >> 6;
+    const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+    if (r < M) {
+        const int a = rowptr[r], b = rowptr[r + 1];
+        if (b - a <= kLongRow) {
+            float s = 0.f;
+            for (int j = a + lane; j < b; j += 64) s += val[j];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-    if (lane == 0) dinv[r] = s > 0.f ? 1.f / sqrtf(s) : 0.f;
+            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            if (lane == 0) dinv[r] = s > 0.f ? 1.f / sqrtf(s) : 0.f;
+        }
+    }
+    for (int q = 0; q < 4; ++q) {  // the long rows among this workgroup's four, one after the other
+        const int64_t rq = (int64_t)blockIdx.x * 4 + q;
+        if (rq >= M) break;
+        const int a = rowptr[rq], b = rowptr[rq + 1];
+        if (b - a <= kLongRow) continue;  // uniform over the workgroup
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        int j = a + threadIdx.x;
+        for (; j + 768 < b; j += 1024) {
+            s0 += val[j];
+            s1 += val[j + 256];
+            s2 += val[j + 512];
+            s3 += val[j + 768];
+        }
+        for (; j < b; j += 256) s0 += val[j];
+        float s = (s0 + s1) + (s2 + s3);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        __syncthreads();
+        if (lane == 0) part[wave] = s;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const float t = (part[0] + part[1]) + (part[2] + part[3]);
+            dinv[rq] = t > 0.f ? 1.f / sqrtf(t) : 0.f;
+        }
+    }
 }
 
+// out[j] = dinv[row(j)] val[j] dinv[col[j]], entry by entry; the row of an entry is found by binary search in the row
+// pointer (small against the entries, so it stays in cache), which costs a hub row no more than any other.  The number
+// of entries is read from the row pointer on the device, so the host does not have to know it.
 __global__ void __launch_bounds__(256) gcn_scale_kernel(int64_t M, const int32_t *__restrict__ rowptr,
                                                         const int32_t *__restrict__ col, const float *__restrict__ val,
                                                         const float *__restrict__ dinv, float *__restrict__ out)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= M) return;
-    const int a = rowptr[r], b = rowptr[r + 1];
-    const float dr = dinv[r];
-    for (int j = a + lane; j < b; j += 64) out[j] = (dr * val[j]) * dinv[col[j]];
+    const int64_t nnz = rowptr[M];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < nnz; j += stride) {
+        int64_t lo = 0, hi = M;  // rowptr[lo] <= j < rowptr[hi]
+        while (hi - lo > 1) {
+            const int64_t mid = (lo + hi) >> 1;
+            if ((int64_t)rowptr[mid] <= j)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        out[j] = (dinv[lo] * val[j]) * dinv[col[j]];
+    }
 }
 
 // one pass over (p, g, m, v): 16 bytes read and 12 written per element; one item per thread
@@ -280,7 +324,7 @@ int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, c
     const unsigned blocks = (unsigned)plx::ceil_div(M, 4);
     row_dinv_kernel<<<blocks, 256, 0, st>>>(M, rowptr, val_in, dinv);
     PLX_LAUNCH_CHECK("row_dinv_kernel");
-    gcn_scale_kernel<<<blocks, 256, 0, st>>>(M, rowptr, col, val_in, dinv, val_out);
+    gcn_scale_kernel<<<256 * 32, 256, 0, st>>>(M, rowptr, col, val_in, dinv, val_out);
     PLX_LAUNCH_CHECK("gcn_scale_kernel");
     return PLX_OK;
 }
