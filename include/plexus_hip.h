@@ -105,7 +105,7 @@ typedef struct plx_spmm_plan plx_spmm_plan;
 
 /* Reads rowptr (M+1 int32 on the device; synchronises `stream` once), bins the rows and keeps the
  * segment tables on the device.  rowptr/col are BORROWED: they must outlive the plan.
- * seg_len <= 0 selects the default. */
+ * seg_len <= 0 selects the default (1024, or 4096 when rows hold 128 entries or more on average). */
 int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr,
                          const int32_t *col, int32_t seg_len, void *stream);
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
