@@ -13,7 +13,7 @@
  *   - the return value is 0 on success or a negative plx_status; nothing throws;
  *     plx_last_error() gives a thread-local message for the last failure;
  *   - apart from plx_spmm_plan_create (which owns a few small device tables until
- *     plx_spmm_plan_destroy) no call allocates: scratch comes from the caller, sized by the
+ *     plx_spmm_plan_destroy, and a 4-byte counter during the call) no call allocates: scratch comes from the caller, sized by the
  *     matching *_workspace_bytes query;
  *   - results are deterministic: no atomics, fixed summation order for given inputs and plan.
  */
@@ -103,8 +103,10 @@ int plx_spmm_segments_host(int64_t M, const int32_t *rowptr_host, int32_t seg_le
  * ---------------------------------------------------------------------------------------- */
 typedef struct plx_spmm_plan plx_spmm_plan;
 
-/* Reads rowptr (M+1 int32 on the device; synchronises `stream` once), bins the rows and keeps the
- * segment tables on the device.  rowptr/col are BORROWED: they must outlive the plan.
+/* Reads rowptr (M+1 int32 on the device; synchronises `stream`), bins the rows and keeps the
+ * segment tables on the device.  Checks once that rowptr runs from 0 to nnz without decreasing and that
+ * every column index lies in [0, K) (PLX_ERR_INVALID otherwise): the SpMM itself trusts them.
+ * rowptr/col are BORROWED: they must outlive the plan and keep their contents.
  * seg_len <= 0 selects the default (1024, or 4096 when rows hold 128 entries or more on average). */
 int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr,
                          const int32_t *col, int32_t seg_len, void *stream);

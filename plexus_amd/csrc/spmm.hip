@@ -364,6 +364,17 @@ __global__ void narrow_i64_kernel(int64_t n, const int64_t *__restrict__ src, in
     for (; i < n; i += stride) dst[i] = (int32_t)src[i];
 }
 
+// Counts the column indices outside [0, K): the gather of the SpMM trusts them.
+__global__ void __launch_bounds__(256) count_bad_columns_kernel(int64_t nnz, const int32_t *__restrict__ col, int32_t K,
+                                                                unsigned int *__restrict__ n_bad)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    unsigned int bad = 0;
+    for (; i < nnz; i += stride) bad += (unsigned int)col[i] >= (unsigned int)K ? 1u : 0u;
+    if (bad) atomicAdd(n_bad, bad);
+}
+
 // Diagnostic: what the memory system gives to the access pattern of the SpMM when nothing else is in the
 // way -- uniformly random rows of a dense table, 128-bit loads, G rows per wavefront instruction, 8 loads in
 // flight per lane, row numbers from a hash (no index stream, no arithmetic worth mentioning).
@@ -458,7 +469,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
     PLX_REQUIRE(row_begin >= 0 && row_begin <= row_end && row_end <= plan->M, "spmm: row range [%lld, %lld) outside [0, %lld)",
                 (long long)row_begin, (long long)row_end, (long long)plan->M);
-    PLX_REQUIRE(D >= 0 && D < (1ll << 30), "spmm: bad feature width D=%lld", (long long)D);
+    PLX_REQUIRE(D >= 0 && D <= (1ll << 21), "spmm: bad feature width D=%lld (at most 2,097,152)", (long long)D);
     if (row_begin == row_end || D == 0) return PLX_OK;
     PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
@@ -598,7 +609,8 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
     PLX_REQUIRE(out != nullptr, "plan_create: NULL output");
     *out = nullptr;
     PLX_REQUIRE(M >= 0 && K >= 0 && nnz >= 0, "plan_create: negative size");
-    PLX_REQUIRE(M < (1ll << 31) - 1 && K < (1ll << 31) && nnz < (1ll << 31), "plan_create: sizes exceed int32 indexing");
+    // the kernels step through the entries 64 at a time with 32-bit positions
+    PLX_REQUIRE(M < (1ll << 31) - 1 && K < (1ll << 31) && nnz < (1ll << 31) - 64, "plan_create: sizes exceed int32 indexing");
     PLX_REQUIRE(rowptr != nullptr, "plan_create: NULL rowptr");
     PLX_REQUIRE(nnz == 0 || col != nullptr, "plan_create: NULL col");
     // default split length, from measurements: 1,024 entries on graphs with short rows (the 2.45 M-node power-law graph:
@@ -616,6 +628,22 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
     int64_t nl = 0, ns = 0;
     int rc = plx_spmm_segments_host(M, rp.data(), seg_len, &nl, &ns, nullptr, nullptr, 0, nullptr, nullptr, 0);
     if (rc != PLX_OK) return rc;
+
+    if (nnz > 0) {  // every column index must name a row of H: one streaming pass, once per matrix
+        unsigned int *d_bad = nullptr, h_bad = 0;
+        PLX_HIP_CHECK(hipMalloc(reinterpret_cast<void **>(&d_bad), sizeof(unsigned int)));
+        hipError_t e = hipMemsetAsync(d_bad, 0, sizeof(unsigned int), st);
+        if (e == hipSuccess) {
+            const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(nnz, 256 * 8), 8192);
+            count_bad_columns_kernel<<<blocks, 256, 0, st>>>(nnz, col, (int32_t)K, d_bad);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(&h_bad, d_bad, sizeof(unsigned int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        (void)hipFree(d_bad);
+        if (e != hipSuccess) return plx::fail(PLX_ERR_HIP, "plan_create: column check failed: %s", hipGetErrorString(e));
+        PLX_REQUIRE(h_bad == 0, "plan_create: %u column indices lie outside [0, %lld)", h_bad, (long long)K);
+    }
 
     plx_spmm_plan *p = new (std::nothrow) plx_spmm_plan();
     if (!p) return plx::fail(PLX_ERR_NOMEM, "plan_create: host allocation failed");

@@ -100,6 +100,24 @@ def test_spmm_edge_cases():
     assert ops.spmm(a0, h.to(DEV)).shape == (0, 36)
 
 
+def test_spmm_plan_rejects_malformed_matrices():
+    say("spmm plan: column out of range, decreasing rowptr, wrong nnz")
+    from plexus_amd._lib import PlexusHipError
+
+    rowptr = torch.tensor([0, 2, 3, 5], dtype=torch.int64)
+    val = torch.ones(5)
+    for bad_col in ([0, 1, 4, 2, 3], [0, -1, 2, 2, 3]):  # K = 4: columns 0..3 are valid
+        with pytest.raises(PlexusHipError, match="column indices lie outside"):
+            ops.CsrMatrix(rowptr.to(DEV), torch.tensor(bad_col).to(DEV), val.to(DEV), (3, 4))
+    good_col = torch.tensor([0, 1, 3, 2, 3])
+    with pytest.raises(PlexusHipError, match="rowptr decreases"):
+        ops.CsrMatrix(torch.tensor([0, 3, 2, 5]).to(DEV), good_col.to(DEV), val.to(DEV), (3, 4))
+    with pytest.raises(PlexusHipError, match="rowptr"):
+        ops.CsrMatrix(torch.tensor([0, 2, 3, 4]).to(DEV), good_col.to(DEV), val.to(DEV), (3, 4))
+    a = ops.CsrMatrix(rowptr.to(DEV), good_col.to(DEV), val.to(DEV), (3, 4))  # the well-formed one is accepted
+    assert ops.spmm(a, torch.eye(4, device=DEV)).sum().item() == 5.0
+
+
 def test_spmm_int64_torch_csr_and_chunked_equivalence():
     say("spmm from torch CSR tensor; chunked == unchunked")
     g = graph_small(n=900, pairs=9000, seed=3)
