@@ -33,6 +33,13 @@ __global__ void iota_kernel(int64_t n, int32_t *__restrict__ out)
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (int32_t)i;
 }
 
+// a fill kernel rather than a memset node: these calls are stream-ordered and may be recorded into a graph
+__global__ void zero_i32_kernel(int64_t n, int32_t *__restrict__ out)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = 0;
+}
+
 // rowptr[c] = first position i with sorted[i] >= c, for c in [0, n_rows]; positions are sorted ascending
 template <typename KeyT, typename RowOf>
 __global__ void rowptr_from_sorted_kernel(int64_t n, const KeyT *__restrict__ sorted, int64_t n_rows, int32_t *__restrict__ rowptr,
@@ -170,7 +177,8 @@ int plx_csr_transpose_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *rowp
     PLX_REQUIRE(rowptr_t != nullptr, "csr_transpose: NULL rowptr_t");
     hipStream_t st = plx::as_stream(stream);
     if (nnz == 0) {
-        PLX_HIP_CHECK(hipMemsetAsync(rowptr_t, 0, sizeof(int32_t) * (size_t)(K + 1), st));
+        zero_i32_kernel<<<blocks_for(K + 1), 256, 0, st>>>(K + 1, rowptr_t);
+        PLX_LAUNCH_CHECK("zero_i32_kernel");
         return PLX_OK;
     }
     PLX_REQUIRE(rowptr && col && val && col_t && val_t, "csr_transpose: NULL operand");
@@ -216,7 +224,8 @@ int plx_coo_block_to_csr_f32(int64_t n_edges, const int64_t *row, const int64_t 
     hipStream_t st = plx::as_stream(stream);
     *nnz_host = 0;
     if (n_edges == 0 || Mb == 0 || Kb == 0) {
-        PLX_HIP_CHECK(hipMemsetAsync(rowptr, 0, sizeof(int32_t) * (size_t)(Mb + 1), st));
+        zero_i32_kernel<<<blocks_for(Mb + 1), 256, 0, st>>>(Mb + 1, rowptr);
+        PLX_LAUNCH_CHECK("zero_i32_kernel");
         return PLX_OK;
     }
     PLX_REQUIRE(row && col && weight && col_out && val_out, "coo_to_csr: NULL operand");
@@ -248,7 +257,8 @@ int plx_coo_block_to_csr_f32(int64_t n_edges, const int64_t *row, const int64_t 
     PLX_HIP_CHECK(hipMemcpyAsync(&kept, count, sizeof(int64_t), hipMemcpyDeviceToHost, st));
     PLX_HIP_CHECK(hipStreamSynchronize(st));
     if (kept == 0) {
-        PLX_HIP_CHECK(hipMemsetAsync(rowptr, 0, sizeof(int32_t) * (size_t)(Mb + 1), st));
+        zero_i32_kernel<<<blocks_for(Mb + 1), 256, 0, st>>>(Mb + 1, rowptr);
+        PLX_LAUNCH_CHECK("zero_i32_kernel");
         return PLX_OK;
     }
     // 2. sort by (row, col); the sort is stable, so duplicates of an edge are added in their input order
