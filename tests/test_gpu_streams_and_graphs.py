@@ -1,4 +1,5 @@
-"""The hot-path entry points are stream-ordered and allocate nothing, so a caller may record them into a HIP graph.
+"""The hot-path entry points are stream-ordered, allocate nothing and share no state: a caller may record them into
+a HIP graph, and host threads may drive different streams at once.
 
 Forward, loss and backward of a two-layer network are captured once and replayed several times with new inputs
 written into the captured buffers; eager work and synchronisations sit between the replays, and every replay is
@@ -26,6 +27,7 @@ def to_dev(g, transpose=False, seg_len=0):
     return ops.CsrMatrix(g.rowptr.to(DEV), g.col.to(DEV), g.val.to(DEV), g.shape, seg_len)
 
 
+@pytest.mark.filterwarnings("ignore:The AccumulateGrad node")  # the warm-up runs on a side stream on purpose
 @pytest.mark.parametrize("association", ["reference", "auto"])
 def test_forward_loss_backward_replay_from_a_hip_graph(association):
     say("HIP graph capture of forward + loss + backward, association=%s" % association)
@@ -79,3 +81,52 @@ def test_forward_loss_backward_replay_from_a_hip_graph(association):
         for a, b in zip(got, want):
             assert a.shape == b.shape and torch.equal(a, b), "replay %d differs from the eager step" % replay
         assert torch.isfinite(got[0]).all() and got[-1].abs().max() > 0
+
+
+def test_threads_on_their_own_streams_give_the_serial_result():
+    """The library keeps no global state: host threads driving different streams at once, each with its own matrices
+    and scratch, get what a single thread gets (ctypes releases the interpreter lock during a call)."""
+    import threading
+
+    say("four host threads, four streams")
+    n, d_in, d_out = 4000, 96, 40
+    jobs = []
+    for i in range(4):
+        g = S.build_graph(n, "chunglu", 50000, seed=20 + i, device="cpu", gamma=2.2)
+        gen = torch.Generator().manual_seed(i)
+        jobs.append(dict(a=to_dev(g, seg_len=128), at=to_dev(g, True, seg_len=128),
+                         h=torch.randn(n, d_in, generator=gen).to(DEV), w=torch.randn(d_in, d_out, generator=gen).to(DEV),
+                         y=torch.randint(0, d_out, (n,), generator=gen).to(DEV)))
+
+    def layer(j):
+        agg = ops.spmm(j["a"], j["h"])
+        out = ops.gemm_nn(agg, j["w"], relu=True)
+        loss, gout = ops.softmax_xent(out, j["y"], n, d_out)
+        gw = ops.gemm_tn(agg, gout, mask=out)
+        gh = ops.spmm(j["at"], ops.gemm_nt(gout, j["w"], mask=out))
+        return [loss, gw, gh]
+
+    serial = [[t.clone() for t in layer(j)] for j in jobs]
+    torch.cuda.synchronize()
+    results, errors = [None] * len(jobs), []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    results[i] = layer(jobs[i])
+            stream.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(100)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for want, got in zip(serial, results):
+        for a, b in zip(want, got):
+            assert torch.equal(a, b)
