@@ -417,6 +417,21 @@ def test_config1_ten_epoch_loss_curve(fuse_relu):
         assert close(layer.weight, w_64)
 
 
+def oracle_rows_of_spmm(g, h):
+    """(row ids, rows of A.H by the fp64-accumulating oracle) for the 8 longest, the 8 shortest and 200 random rows of a
+    graph held on the device; only the entries of those rows leave the device."""
+    m = g.shape[0]
+    deg = (g.rowptr[1:] - g.rowptr[:-1]).cpu()
+    pick = torch.cat([torch.topk(deg, 8).indices, torch.topk(-deg, 8).indices,
+                      torch.randint(0, m, (200,), generator=torch.Generator().manual_seed(0))])
+    sub_counts = deg[pick]
+    sub_rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(sub_counts, 0)])
+    starts = g.rowptr[pick.to(DEV)]
+    idx = torch.repeat_interleave(starts - sub_rowptr[:-1].to(DEV), sub_counts.to(DEV)) + torch.arange(int(sub_rowptr[-1]), device=DEV)
+    ci, va = g.col[idx].cpu(), g.val[idx].cpu()
+    return pick, oracle_c.csr_spmm(sub_rowptr.numpy(), ci.numpy(), va.numpy(), h.float().cpu().numpy())
+
+
 def spmm_properties_and_sampled_rows(g, d):
     """Size-independent properties of Y = A.H on a graph held on the device, and sampled rows (the longest, the
     shortest and random ones) against the fp64-accumulating oracle; only the sampled rows leave the device."""
@@ -446,15 +461,7 @@ def spmm_properties_and_sampled_rows(g, d):
     del y2
     # bit reproducibility
     assert torch.equal(y, ops.spmm(a, h))
-    deg = (g.rowptr[1:] - g.rowptr[:-1]).cpu()
-    pick = torch.cat([torch.topk(deg, 8).indices, torch.topk(-deg, 8).indices,
-                      torch.randint(0, m, (200,), generator=torch.Generator().manual_seed(0))])
-    sub_counts = deg[pick]
-    sub_rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(sub_counts, 0)])
-    starts = g.rowptr[pick.to(DEV)]
-    idx = torch.repeat_interleave(starts - sub_rowptr[:-1].to(DEV), sub_counts.to(DEV)) + torch.arange(int(sub_rowptr[-1]), device=DEV)
-    ci, va = g.col[idx].cpu(), g.val[idx].cpu()
-    ref = oracle_c.csr_spmm(sub_rowptr.numpy(), ci.numpy(), va.numpy(), h.cpu().numpy())
+    pick, ref = oracle_rows_of_spmm(g, h)
     assert rel_err(y[pick.to(DEV)].cpu(), ref) <= FP32_TOL
 
 
@@ -464,6 +471,28 @@ def test_config3_properties_and_sampled_rows(scale):
     properties of the SpMM and a comparison of sampled rows against the fp64-accumulating oracle."""
     say("config 3 at scale %g: properties" % scale)
     spmm_properties_and_sampled_rows(S.config3_graph(DEV, seed=0, scale=scale), 128)
+
+
+def test_config5_full_size_bf16_spmm_properties_and_sampled_rows():
+    """The bf16-storage configuration at full size: the 2.45 M-node graph, 256 features held as bf16, fp32 accumulation."""
+    say("config 5 at full size: bf16 SpMM, D=256")
+    g = S.config3_graph(DEV, seed=0, scale=1.0)
+    m, k = g.shape
+    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape)
+    h = S.normal_features(k, 256, DEV, seed=1).to(torch.bfloat16)
+    y = ops.spmm(a, h)
+    assert y.dtype == torch.bfloat16 and torch.equal(y, ops.spmm(a, h))
+    # sampled rows: fp32 arithmetic on the bf16-rounded inputs, one rounding of the result (2^-9 relative per element)
+    pick, ref = oracle_rows_of_spmm(g, h)
+    got = y[pick.to(DEV)].float().cpu()
+    assert rel_err(got, ref) <= 2.0 ** -8
+    # A.1 = row sums (ones are exact in bf16; the sums are rounded once)
+    csum = torch.cat([torch.zeros(1, dtype=torch.float64, device=DEV), torch.cumsum(g.val.double(), 0)])
+    rowsum = csum[g.rowptr[1:]] - csum[g.rowptr[:-1]]
+    ones = torch.ones(k, 8, device=DEV, dtype=torch.bfloat16)
+    assert rel_err(ops.spmm(a, ones)[:, 0].float(), rowsum) <= 2.0 ** -8
+    # scaling by a power of two is exact in every step: Y(4 H) == 4 Y(H) bit for bit
+    assert torch.equal(ops.spmm(a, 4.0 * h), 4.0 * y)
 
 
 @pytest.mark.parametrize("d", [602, 128])
