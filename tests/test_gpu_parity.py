@@ -118,6 +118,46 @@ def test_spmm_plan_rejects_malformed_matrices():
     assert ops.spmm(a, torch.eye(4, device=DEV)).sum().item() == 5.0
 
 
+def test_spmm_and_transpose_just_below_the_int32_limit():
+    """Maximum size: 2,145,386,496 stored entries (the entry points take fewer than 2^31 - 64), every row split into two
+    segments.  The product is checked against fp64 arithmetic by torch in row blocks, the transpose by the adjoint
+    identity and by transposing twice."""
+    say("spmm + transpose with 2.1e9 entries")
+    m, per_row, band = 2 ** 21, 1023, 1024
+    k, nnz, d = per_row * band, m * per_row, 4
+    assert 2 ** 31 - 2 ** 21 <= nnz < 2 ** 31 - 64
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    # entry j of a row lies in band j of the columns: ascending within the row, as a transpose produces them
+    col = torch.randint(0, band, (m, per_row), dtype=torch.int32, device=DEV, generator=gen)
+    col += (torch.arange(per_row, dtype=torch.int32, device=DEV) * band)[None, :]
+    col = col.reshape(-1)
+    val = torch.rand(nnz, device=DEV, generator=gen)
+    rowptr = (torch.arange(m + 1, dtype=torch.int64, device=DEV) * per_row).to(torch.int32)
+    assert int(rowptr[-1]) == nnz
+    a = ops.CsrMatrix(rowptr, col, val, (m, k), seg_len=512)
+    assert a.n_long_rows == m and a.n_segments == 2 * m
+    h = torch.randn(k, d, device=DEV, generator=gen)
+    y = ops.spmm(a, h)
+    block = 2 ** 16
+    worst, largest = 0.0, 0.0
+    for r0 in range(0, m, block):
+        c = col[r0 * per_row:(r0 + block) * per_row].long()
+        ref = (h[c].double().view(block, per_row, d) * val[r0 * per_row:(r0 + block) * per_row].double().view(block, per_row, 1)).sum(1)
+        worst = max(worst, (y[r0:r0 + block].double() - ref).abs().max().item())
+        largest = max(largest, ref.abs().max().item())
+        del c, ref
+    print("max error %.3e of %.3e" % (worst, largest), flush=True)
+    assert worst <= FP32_TOL * largest
+    at = ops.csr_transpose(a, seg_len=4096)
+    assert at.shape == (k, m) and at.nnz == nnz
+    gm = torch.randn(m, d, device=DEV, generator=gen)
+    lhs = (y.double() * gm.double()).sum().item()
+    rhs = (h.double() * ops.spmm(at, gm).double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-5 * (y.double().norm() * gm.double().norm()).item()
+    att = ops.csr_transpose(at)
+    assert torch.equal(att.rowptr, a.rowptr) and torch.equal(att.col, a.col) and torch.equal(att.val, a.val)
+
+
 def test_spmm_int64_torch_csr_and_chunked_equivalence():
     say("spmm from torch CSR tensor; chunked == unchunked")
     g = graph_small(n=900, pairs=9000, seed=3)
