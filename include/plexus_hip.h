@@ -240,14 +240,16 @@ int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, c
  *   no amsgrad):
  *     p *= 1 - lr * weight_decay;  m += (g - m) (1 - beta1);  v = beta2 v + (1 - beta2) g^2;
  *     p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
- *   `step` is the 1-based count of this update.
+ *   `step` is the 1-based count of this update.  The hyperparameters are doubles, as the Python optimizer holds
+ *   them; each is rounded to fp32 where torch rounds it (1 - beta is formed in double first), so the moments and
+ *   the parameters follow torch.optim.AdamW to within a few roundings of fp32.
  * ---------------------------------------------------------------------------------------- */
-int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, float lr, float beta1,
-                  float beta2, float eps, float weight_decay, int64_t step, void *stream);
+int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, double lr, double beta1,
+                  double beta2, double eps, double weight_decay, int64_t step, void *stream);
 /* same update with a bf16 gradient (fp32 parameter and moments); optionally also writes bf16(param) to
  * param_bf16 (may be NULL) so that the next forward needs no separate cast pass */
-int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, float lr,
-                            float beta1, float beta2, float eps, float weight_decay, int64_t step, uint16_t *param_bf16,
+int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, double lr,
+                            double beta1, double beta2, double eps, double weight_decay, int64_t step, uint16_t *param_bf16,
                             void *stream);
 
 #ifdef __cplusplus

@@ -16,6 +16,7 @@ _i64 = C.c_int64
 _i32 = C.c_int32
 _sz = C.c_size_t
 _f32 = C.c_float
+_f64 = C.c_double
 _u32 = C.c_uint
 
 # name -> (restype, argtypes); mirrors include/plexus_hip.h one to one
@@ -52,8 +53,8 @@ SIGNATURES = {
     "plx_softmax_xent_workspace_bytes": (_sz, [_i64, _i64]),
     "plx_softmax_xent_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
     "plx_gcn_norm_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "plx_adamw_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32, _f32, _i64, _vp]),
-    "plx_adamw_f32_grad_bf16": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f32, _f32, _f32, _f32, _f32, _i64, _vp, _vp]),
+    "plx_adamw_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64, _i64, _vp]),
+    "plx_adamw_f32_grad_bf16": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64, _i64, _vp, _vp]),
     "plx_gemm_nt_bf16": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _u32, _f32,
                                    C.c_uint64, C.c_uint64, _vp]),
     "plx_gemm_tn_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),

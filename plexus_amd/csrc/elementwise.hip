@@ -261,17 +261,35 @@ int plx_relu_bwd_f32(int64_t M, int64_t N, const float *dY, int64_t lddy, const 
     return relu_common(true, M, N, dY, lddy, Y, ldy, dX, lddx, stream);
 }
 
-int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, float lr, float beta1,
-                  float beta2, float eps, float weight_decay, int64_t step, void *stream)
+// The hyperparameters arrive as doubles, as Python holds them, and are rounded to fp32 only where torch's optimizer
+// rounds them (1 - beta as a double first), so that the moments match torch.optim.AdamW to fp32 rounding.
+struct AdamScalars {
+    float decay, one_minus_b1, b2, one_minus_b2, step_size, inv_bc2_sqrt, eps;
+};
+
+static AdamScalars adam_scalars(double lr, double beta1, double beta2, double eps, double weight_decay, int64_t step)
+{
+    const double bc1 = 1.0 - std::pow(beta1, (double)step);
+    const double bc2 = 1.0 - std::pow(beta2, (double)step);
+    AdamScalars a;
+    a.decay = (float)(1.0 - lr * weight_decay);
+    a.one_minus_b1 = (float)(1.0 - beta1);
+    a.b2 = (float)beta2;
+    a.one_minus_b2 = (float)(1.0 - beta2);
+    a.step_size = (float)(lr / bc1);
+    a.inv_bc2_sqrt = (float)(1.0 / std::sqrt(bc2));
+    a.eps = (float)eps;
+    return a;
+}
+
+int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, float *exp_avg_sq, double lr, double beta1,
+                  double beta2, double eps, double weight_decay, int64_t step, void *stream)
 {
     PLX_REQUIRE(n >= 0 && step >= 1, "adamw: bad size or step (n=%lld step=%lld)", (long long)n, (long long)step);
     if (n == 0) return PLX_OK;
     PLX_REQUIRE(param && grad && exp_avg && exp_avg_sq, "adamw: NULL operand");
-    const double bc1 = 1.0 - std::pow((double)beta1, (double)step);
-    const double bc2 = 1.0 - std::pow((double)beta2, (double)step);
-    const float step_size = (float)((double)lr / bc1);
-    const float inv_bc2_sqrt = (float)(1.0 / std::sqrt(bc2));
-    const float decay = 1.0f - lr * weight_decay;
+    PLX_REQUIRE(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0, "adamw: betas must lie in [0, 1)");
+    const AdamScalars a = adam_scalars(lr, beta1, beta2, eps, weight_decay, step);
     const bool v4 = n % 4 == 0 && reinterpret_cast<uintptr_t>(param) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(exp_avg_sq) % 16 == 0;
     const int64_t count = v4 ? n / 4 : n;
@@ -279,37 +297,36 @@ int plx_adamw_f32(int64_t n, float *param, const float *grad, float *exp_avg, fl
     const unsigned blocks = (unsigned)plx::ceil_div(count, 256);
     hipStream_t st = plx::as_stream(stream);
     if (v4)
-        adamw_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2, 1.0f - beta2,
-                                                   step_size, inv_bc2_sqrt, eps);
+        adamw_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, a.decay, a.one_minus_b1, a.b2, a.one_minus_b2,
+                                                   a.step_size, a.inv_bc2_sqrt, a.eps);
     else
-        adamw_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2, 1.0f - beta2,
-                                                    step_size, inv_bc2_sqrt, eps);
+        adamw_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, a.decay, a.one_minus_b1, a.b2, a.one_minus_b2,
+                                                    a.step_size, a.inv_bc2_sqrt, a.eps);
     PLX_LAUNCH_CHECK("adamw_kernel");
     return PLX_OK;
 }
 
-int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, float lr,
-                            float beta1, float beta2, float eps, float weight_decay, int64_t step, uint16_t *param_bf16,
+int plx_adamw_f32_grad_bf16(int64_t n, float *param, const uint16_t *grad, float *exp_avg, float *exp_avg_sq, double lr,
+                            double beta1, double beta2, double eps, double weight_decay, int64_t step, uint16_t *param_bf16,
                             void *stream)
 {
     PLX_REQUIRE(n >= 0 && step >= 1, "adamw: bad size or step (n=%lld step=%lld)", (long long)n, (long long)step);
     if (n == 0) return PLX_OK;
     PLX_REQUIRE(param && grad && exp_avg && exp_avg_sq, "adamw: NULL operand");
-    const double bc1 = 1.0 - std::pow((double)beta1, (double)step);
-    const double bc2 = 1.0 - std::pow((double)beta2, (double)step);
+    PLX_REQUIRE(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0, "adamw: betas must lie in [0, 1)");
+    const AdamScalars a = adam_scalars(lr, beta1, beta2, eps, weight_decay, step);
     const bool v4 = n % 4 == 0 && reinterpret_cast<uintptr_t>(param) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % 8 == 0 &&
                     reinterpret_cast<uintptr_t>(exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(exp_avg_sq) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(param_bf16) % 8 == 0;
     PLX_REQUIRE(plx::ceil_div(v4 ? n / 4 : n, 256) < (1ll << 31), "adamw: tensor too large for one launch");
     const unsigned blocks = (unsigned)plx::ceil_div(v4 ? n / 4 : n, 256);
     hipStream_t st = plx::as_stream(stream);
-    const float decay = 1.0f - lr * weight_decay, step_size = (float)((double)lr / bc1), inv_bc2_sqrt = (float)(1.0 / std::sqrt(bc2));
     if (v4)
-        adamw_grad_bf16_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2,
-                                                             1.0f - beta2, step_size, inv_bc2_sqrt, eps, param_bf16);
+        adamw_grad_bf16_kernel<true><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, a.decay, a.one_minus_b1, a.b2,
+                                                             a.one_minus_b2, a.step_size, a.inv_bc2_sqrt, a.eps, param_bf16);
     else
-        adamw_grad_bf16_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, decay, 1.0f - beta1, beta2,
-                                                              1.0f - beta2, step_size, inv_bc2_sqrt, eps, param_bf16);
+        adamw_grad_bf16_kernel<false><<<blocks, 256, 0, st>>>(n, param, grad, exp_avg, exp_avg_sq, a.decay, a.one_minus_b1, a.b2,
+                                                              a.one_minus_b2, a.step_size, a.inv_bc2_sqrt, a.eps, param_bf16);
     PLX_LAUNCH_CHECK("adamw_grad_bf16_kernel");
     return PLX_OK;
 }

@@ -274,7 +274,7 @@ int main()
     float *d_m = device_alloc<float>(w.size()), *d_v = device_alloc<float>(w.size());
     HIP_OK(hipMemsetAsync(d_m, 0, w.size() * sizeof(float), st));
     HIP_OK(hipMemsetAsync(d_v, 0, w.size() * sizeof(float), st));
-    PLX_OK_OR_DIE(plx_adamw_f32((int64_t)w.size(), d_w, d_gw, d_m, d_v, 3e-3f, 0.9f, 0.999f, 1e-8f, 0.0f, 1, st));
+    PLX_OK_OR_DIE(plx_adamw_f32((int64_t)w.size(), d_w, d_gw, d_m, d_v, 3e-3, 0.9, 0.999, 1e-8, 0.0, 1, st));
     // from the gradient the device holds: the first step moves every weight by lr * sign(g), so a gradient within
     // rounding of zero must not be allowed to differ in sign between the two sides
     const std::vector<float> gw_dev = to_host(d_gw, gw_ref.size());

@@ -28,6 +28,40 @@ def test_library_exports_every_declared_symbol(lib):
     assert sorted(_lib.SIGNATURES) == syms
 
 
+def header_prototypes():
+    """name -> (return type, [parameter types]) as written in the header, comments and names stripped."""
+    text = open(os.path.join(ROOT, "include", "plexus_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = {}
+    for ret, name, params in re.findall(r"^\s*([a-z_0-9 ]+?\*?)\s*\b(plx_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text, flags=re.M | re.S):
+        types = []
+        for prm in [x.strip() for x in params.replace("\n", " ").split(",")]:
+            if prm in ("void", ""):
+                continue
+            types.append("ptr" if "*" in prm else re.sub(r"\s+\w+$", "", prm.replace("const ", "")).strip())
+        protos[name] = (ret.strip(), types)
+    return protos
+
+
+def test_binding_table_matches_the_header_types():
+    """Every ctypes signature has the arity and the scalar types of its C prototype (a float/double or
+    int32/int64 slip corrupts arguments silently)."""
+    scalar = {"int64_t": C.c_int64, "int32_t": C.c_int32, "int": C.c_int, "unsigned": C.c_uint, "float": C.c_float,
+              "double": C.c_double, "size_t": C.c_size_t, "uint64_t": C.c_uint64}
+    rets = {"int": C.c_int, "size_t": C.c_size_t, "int64_t": C.c_int64, "const char *": C.c_char_p, "const char*": C.c_char_p}
+    protos = header_prototypes()
+    assert sorted(protos) == sorted(_lib.SIGNATURES)
+    for name, (ret, types) in protos.items():
+        res, args = _lib.SIGNATURES[name]
+        assert rets[ret] is res, name
+        assert len(args) == len(types), "%s: %d parameters in the header, %d in the binding" % (name, len(types), len(args))
+        for i, (t, a) in enumerate(zip(types, args)):
+            if t == "ptr":
+                assert a is C.c_void_p or issubclass(a, C._Pointer) or a is C.c_char_p, "%s arg %d" % (name, i)
+            else:
+                assert scalar[t] is a, "%s arg %d: header %s, binding %s" % (name, i, t, a)
+
+
 def test_version_and_error_strings(lib):
     assert lib.plx_version() >= 100
     assert lib.plx_error_string(0) == b"ok"
