@@ -229,8 +229,9 @@ class GCNConv(torch.nn.Module):
     Additions: ``association`` selects the order of the two products (see above; the default is the
     reference's); ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (bf16 storage only) drops
     activations after the ReLU in training mode with a counter-based generator keyed by ``dropout_seed``;
-    every training forward uses a fresh offset (``layer_num + 64 * call count``).  The storage type
-    follows the input tensor.
+    every training forward uses a fresh offset (``layer_num + 64 * call count``), which is a host-side
+    counter: a recorded HIP graph replays the mask it was recorded with.  The storage type follows the
+    input tensor.
     """
 
     def __init__(self, in_channels, out_channels, layer_num, weight=None, fuse_relu=False, dropout=0.0, dropout_seed=0,
