@@ -219,6 +219,12 @@ size_t plx_softmax_xent_workspace_bytes(int64_t M, int64_t C);
 int plx_softmax_xent_f32(int64_t M, int64_t C, const float *logits, int64_t ld, const int64_t *labels,
                          int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,
                          float *dlogits, int64_t ldd, void *workspace, size_t workspace_bytes, void *stream);
+/* y[i] = x[i] * (*scale) over a contiguous tensor, `scale` being one float ON THE DEVICE: the multiplication by the
+ * upstream gradient in TensorParallelCrossEntropy.backward (plexus/cross_entropy.py:114), whose scalar autograd
+ * delivers as a device tensor -- reading it in the kernel keeps the host from waiting.  y may alias x.
+ * The bf16 variant takes raw bit patterns and rounds to nearest even. */
+int plx_scale_by_device_scalar_f32(int64_t n, const float *x, const float *scale, float *y, void *stream);
+int plx_scale_by_device_scalar_bf16(int64_t n, const uint16_t *x, const float *scale, uint16_t *y, void *stream);
 /* bf16 logits and gradient, fp32 math and fp32 loss */
 int plx_softmax_xent_bf16(int64_t M, int64_t C, const uint16_t *logits, int64_t ld, const int64_t *labels,
                           int64_t num_nodes, int64_t num_classes, int64_t row_offset, float gscale, float *loss,

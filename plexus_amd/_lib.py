@@ -52,6 +52,8 @@ SIGNATURES = {
     "plx_relu_bwd_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_softmax_xent_workspace_bytes": (_sz, [_i64, _i64]),
     "plx_softmax_xent_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
+    "plx_scale_by_device_scalar_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp]),
+    "plx_scale_by_device_scalar_bf16": (C.c_int, [_i64, _vp, _vp, _vp, _vp]),
     "plx_gcn_norm_csr_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "plx_adamw_f32": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64, _i64, _vp]),
     "plx_adamw_f32_grad_bf16": (C.c_int, [_i64, _vp, _vp, _vp, _vp, _f64, _f64, _f64, _f64, _f64, _i64, _vp, _vp]),

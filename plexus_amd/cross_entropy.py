@@ -28,7 +28,7 @@ class TensorParallelCrossEntropy(torch.autograd.Function):
         timers = get_timers()
         timers.start("cross entropy bwd")
         (dlogits,) = ctx.saved_tensors
-        grad_input = dlogits * grad_output  # plexus/cross_entropy.py:114
+        grad_input = ops.scale_by_scalar(dlogits, grad_output)  # plexus/cross_entropy.py:114
         timers.stop("cross entropy bwd")
         return grad_input, None, None, None, None
 

@@ -246,9 +246,66 @@ int relu_common(bool bwd, int64_t M, int64_t N, const float *in, int64_t ldi, co
     return PLX_OK;
 }
 
+// y[i] = x[i] * (*scale): the upstream gradient of a scalar loss lives on the device and is read there, so the
+// host never waits for it.  T = float (VEC 4) or bf16 bits (VEC 8); one 128-bit item per thread.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) scale_by_device_scalar_kernel(int64_t n, const T *x, const float *__restrict__ scale, T *y)
+{
+    constexpr int kPer = VEC ? 16 / (int)sizeof(T) : 1;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n / kPer) return;
+    const float s = *scale;
+    if constexpr (!VEC) {
+        if constexpr (sizeof(T) == 4)
+            y[i] = x[i] * s;
+        else
+            y[i] = (uint16_t)plx::f32_to_bf16(plx::bf16_to_f32(x[i]) * s);
+    } else if constexpr (sizeof(T) == 4) {
+        const float4 v = load_nt(x + 4 * i);
+        store_nt(y + 4 * i, make_float4(v.x * s, v.y * s, v.z * s, v.w * s));
+    } else {
+        const uint4 v = reinterpret_cast<const uint4 *>(x)[i];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            o[j] = plx::pack_bf16x2(__uint_as_float(w[j] << 16) * s, __uint_as_float(w[j] & 0xffff0000u) * s);
+        reinterpret_cast<uint4 *>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+template <typename T>
+int scale_common(int64_t n, const T *x, const float *scale, T *y, void *stream)
+{
+    PLX_REQUIRE(n >= 0, "scale: negative size");
+    if (n == 0) return PLX_OK;
+    PLX_REQUIRE(x && scale && y, "scale: NULL operand");
+    constexpr int kPer = 16 / (int)sizeof(T);
+    const bool vec = n % kPer == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    const int64_t nblocks = plx::ceil_div(vec ? n / kPer : n, 256);
+    PLX_REQUIRE(nblocks < (1ll << 31), "scale: tensor too large for one launch");
+    hipStream_t st = plx::as_stream(stream);
+    if (vec)
+        scale_by_device_scalar_kernel<T, true><<<(unsigned)nblocks, 256, 0, st>>>(n, x, scale, y);
+    else
+        scale_by_device_scalar_kernel<T, false><<<(unsigned)nblocks, 256, 0, st>>>(n, x, scale, y);
+    PLX_LAUNCH_CHECK("scale_by_device_scalar_kernel");
+    return PLX_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int plx_scale_by_device_scalar_f32(int64_t n, const float *x, const float *scale, float *y, void *stream)
+{
+    return scale_common<float>(n, x, scale, y, stream);
+}
+
+int plx_scale_by_device_scalar_bf16(int64_t n, const uint16_t *x, const float *scale, uint16_t *y, void *stream)
+{
+    return scale_common<uint16_t>(n, x, scale, y, stream);
+}
 
 int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream)
 {

@@ -478,6 +478,8 @@ def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] 
 
 def relu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     _need_gpu(x)
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise TypeError("relu: a 2-D fp32 tensor is expected (bf16 layers fuse the ReLU into the product)")
     if not inplace:
         x = _rowmajor(x)
     y = x if inplace else torch.empty(x.shape, dtype=torch.float32, device=x.device)
@@ -487,6 +489,8 @@ def relu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
 
 def relu_bwd(dy: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _need_gpu(dy, y, out)
+    if dy.dtype != torch.float32 or y.dtype != torch.float32 or dy.shape != y.shape:
+        raise TypeError("relu_bwd: two fp32 tensors of one shape are expected")
     dy, y = _rowmajor(dy), _rowmajor(y)
     dx = out if out is not None else torch.empty(dy.shape, dtype=torch.float32, device=dy.device)
     check(
@@ -524,6 +528,22 @@ def softmax_xent(logits: torch.Tensor, labels: torch.Tensor, num_nodes: int, num
         "plx_softmax_xent",
     )
     return loss, dlogits
+
+
+def scale_by_scalar(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """x * scale for a one-element fp32 device tensor ``scale`` (read on the device; the host does not wait for it)."""
+    _need_gpu(x, scale)
+    if scale.numel() != 1:
+        raise ValueError("scale_by_scalar: the scale must hold one element, got %d" % scale.numel())
+    lib = _lib.load()
+    fn = {torch.float32: lib.plx_scale_by_device_scalar_f32, torch.bfloat16: lib.plx_scale_by_device_scalar_bf16}.get(x.dtype)
+    if fn is None:
+        raise TypeError("scale_by_scalar: unsupported dtype %s" % x.dtype)
+    x = x.contiguous()
+    scale = scale.detach().reshape(1).to(torch.float32)
+    y = torch.empty_like(x)
+    check(fn(x.numel(), x.data_ptr(), scale.data_ptr(), y.data_ptr(), _stream()), "plx_scale_by_device_scalar")
+    return y
 
 
 def gcn_norm_csr(a: CsrMatrix) -> torch.Tensor:

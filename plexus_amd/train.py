@@ -6,12 +6,32 @@ registered, and the optimizer updates the weights and the input features as the 
 validator does (benchmarking/pyg_serial.py:100-104).
 """
 import torch
-import torch.nn.functional as F
 
+from . import ops
 from .cross_entropy import parallel_cross_entropy
 from .gcn_conv import GCNConv
 from .optim import AdamW
 from .utils.timers import get_timers
+
+
+class ReluFunction(torch.autograd.Function):
+    """The F.relu of examples/train.py:77-78 on the library's kernels, for models that keep it outside the layer:
+    forward max(x, 0), backward the upstream gradient where the output is positive."""
+
+    @staticmethod
+    def forward(ctx, x):
+        y = ops.relu(x.detach())
+        ctx.save_for_backward(y)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (y,) = ctx.saved_tensors
+        return ops.relu_bwd(grad_output, y)
+
+
+def relu(x):
+    return ReluFunction.apply(x)
 
 
 class Net(torch.nn.Module):
@@ -34,7 +54,7 @@ class Net(torch.nn.Module):
         for i in range(self.num_gcn_layers):
             x = self.layers[i](x, edge_index_shards)
             if i != self.num_gcn_layers - 1 and not self.fuse_relu:
-                x = F.relu(x)
+                x = relu(x)
         return x
 
 
@@ -72,7 +92,7 @@ def run_epochs(model, optimizer, features, adj_shards, labels, num_nodes, num_cl
         timers.start("epoch " + str(i))
         loss = train(model, optimizer, features, adj_shards, labels, num_nodes, num_classes)
         timers.stop("epoch " + str(i))
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
         if log is not None:
             log("Epoch: {:03d}, Train Loss: {:.4f}".format(i, losses[-1]))
     return losses

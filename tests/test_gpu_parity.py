@@ -368,6 +368,29 @@ def test_softmax_xent_special_cases_and_no_mutation(c):
     assert abs(loss3.item() - closs) <= FP32_TOL * abs(closs) and rel_err(dl3.cpu(), cgrad) <= FP32_TOL
 
 
+def test_upstream_scalar_and_standalone_relu_run_on_the_library():
+    say("loss scaled upstream; ReLU outside the layer")
+    from plexus_amd.cross_entropy import parallel_cross_entropy
+    from plexus_amd.train import relu
+
+    gen = torch.Generator().manual_seed(5)
+    for n, dtype in ((1000 * 48, torch.float32), (1003, torch.float32), (4096, torch.bfloat16), (77, torch.bfloat16)):
+        x = torch.randn(n, generator=gen).to(dtype)
+        got = ops.scale_by_scalar(x.to(DEV), torch.tensor(-2.5, device=DEV))
+        assert got.dtype == dtype and torch.equal(got.cpu(), (x.float() * -2.5).to(dtype))
+    m, c = 1500, 47
+    logits = torch.randn(m, c, generator=gen)
+    y = torch.randint(0, c, (m,), generator=gen)
+    ld = relu(logits.to(DEV).requires_grad_())  # a non-leaf: the gradient flows through relu's backward kernel
+    leaf = ld.grad_fn.next_functions[0][0].variable
+    (parallel_cross_entropy(ld, y.to(DEV), 1, m, c) * 3.0).backward()
+    ref = logits.clone().requires_grad_()
+    (torch.nn.functional.cross_entropy(torch.relu(ref), y) * 3.0).backward()
+    assert rel_err(leaf.grad, ref.grad) <= FP32_TOL
+    with pytest.raises(TypeError):
+        ops.relu(logits.to(DEV).to(torch.bfloat16))
+
+
 def test_gcn_norm_kernel():
     say("gcn_norm_csr")
     g = S.build_graph(1500, "chunglu", 12000, seed=5, device="cpu")
