@@ -247,30 +247,39 @@ int relu_common(bool bwd, int64_t M, int64_t N, const float *in, int64_t ldi, co
 }
 
 // y[i] = x[i] * (*scale): the upstream gradient of a scalar loss lives on the device and is read there, so the
-// host never waits for it.  T = float (VEC 4) or bf16 bits (VEC 8); one 128-bit item per thread.
+// host never waits for it.  T = float or bf16 bits.  VEC: one 128-bit item per thread over the first
+// n - n % kPer elements, and one more thread for the few elements left over; otherwise one element per thread.
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) scale_by_device_scalar_kernel(int64_t n, const T *x, const float *__restrict__ scale, T *y)
 {
-    constexpr int kPer = VEC ? 16 / (int)sizeof(T) : 1;
+    constexpr int kPer = 16 / (int)sizeof(T);
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n / kPer) return;
     const float s = *scale;
-    if constexpr (!VEC) {
+    auto one = [&](int64_t e) {
         if constexpr (sizeof(T) == 4)
-            y[i] = x[i] * s;
+            y[e] = x[e] * s;
         else
-            y[i] = (uint16_t)plx::f32_to_bf16(plx::bf16_to_f32(x[i]) * s);
-    } else if constexpr (sizeof(T) == 4) {
-        const float4 v = load_nt(x + 4 * i);
-        store_nt(y + 4 * i, make_float4(v.x * s, v.y * s, v.z * s, v.w * s));
+            y[e] = (uint16_t)plx::f32_to_bf16(plx::bf16_to_f32(x[e]) * s);
+    };
+    if constexpr (!VEC) {
+        if (i < n) one(i);
     } else {
-        const uint4 v = reinterpret_cast<const uint4 *>(x)[i];
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-        uint32_t o[4];
+        const int64_t items = n / kPer;
+        if (i > items) return;
+        if (i == items) {
+            for (int64_t e = items * kPer; e < n; ++e) one(e);
+        } else if constexpr (sizeof(T) == 4) {
+            const float4 v = load_nt(x + 4 * i);
+            store_nt(y + 4 * i, make_float4(v.x * s, v.y * s, v.z * s, v.w * s));
+        } else {
+            const uint4 v = reinterpret_cast<const uint4 *>(x)[i];
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            uint32_t o[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            o[j] = plx::pack_bf16x2(__uint_as_float(w[j] << 16) * s, __uint_as_float(w[j] & 0xffff0000u) * s);
-        reinterpret_cast<uint4 *>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+            for (int j = 0; j < 4; ++j)
+                o[j] = plx::pack_bf16x2(__uint_as_float(w[j] << 16) * s, __uint_as_float(w[j] & 0xffff0000u) * s);
+            reinterpret_cast<uint4 *>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
     }
 }
 
@@ -281,8 +290,8 @@ int scale_common(int64_t n, const T *x, const float *scale, T *y, void *stream)
     if (n == 0) return PLX_OK;
     PLX_REQUIRE(x && scale && y, "scale: NULL operand");
     constexpr int kPer = 16 / (int)sizeof(T);
-    const bool vec = n % kPer == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
-    const int64_t nblocks = plx::ceil_div(vec ? n / kPer : n, 256);
+    const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    const int64_t nblocks = plx::ceil_div(vec ? n / kPer + 1 : n, 256);
     PLX_REQUIRE(nblocks < (1ll << 31), "scale: tensor too large for one launch");
     hipStream_t st = plx::as_stream(stream);
     if (vec)
