@@ -378,13 +378,21 @@ int softmax_xent_impl(int64_t M, int64_t C, const T *logits, int64_t ld, const i
     a.scale = gscale / (float)num_nodes;
 
     unsigned blocks;
-    if (C >= 2 && C <= 190) {
-        const int R = C <= 47 ? 256 : (C <= 95 ? 128 : 64);  // R * (C | 1) * 4 <= 49,152 bytes of LDS
-        blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, R), kXentMaxBlocks));
+    // Which kernel, from measurements on 2,449,029 rows (fp32, ms): the tiled kernels win up to about 88 classes
+    // (C = 80: 0.67 against 0.71 for a lane group per row), beyond that the lane groups win by far (C = 100: 0.89
+    // against 0.75, C = 172: 2.5 against 0.91).
+    if (C >= 2 && C <= 88) {
         // rows contiguous and tile origins 16-byte aligned (R is a multiple of 8): copy tiles with 128-bit accesses
         const bool contig = C <= 64 && (C & 1) && ld == C && (dlogits == nullptr || ldd == C) &&
                             reinterpret_cast<uintptr_t>(logits) % 16 == 0 && reinterpret_cast<uintptr_t>(dlogits) % 16 == 0;
         const int CP = contig ? (int)C : ((int)C | 1);
+        // rows per tile: 256 or 128 for the vector-copy kernel; the element-copy kernel runs best with tiles of at
+        // most 26 KB, so that six or more workgroups share a compute unit and overlap their copy and row phases
+        // (C = 47 in rows of 48: 0.53 ms with 256 rows, 0.39 with 128; C = 40: 0.44 / 0.29; C = 64: 0.60 / 0.54 with 64)
+        int R = C <= 47 ? 256 : 128;
+        if (!contig)
+            while (R > 32 && (size_t)R * CP * sizeof(float) > 26 * 1024) R >>= 1;
+        blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(M, R), kXentMaxBlocks));
         const size_t shm = (size_t)R * CP * sizeof(float);
         if (contig) launch_tiled_reg<T>(a, C, R, blocks, shm, st);
         else softmax_xent_tiled_kernel<T><<<blocks, 256, shm, st>>>(a, R, CP);
