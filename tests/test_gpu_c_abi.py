@@ -28,3 +28,28 @@ def test_layer_roundtrip_source_uses_only_the_public_header():
     includes = [line.split()[1] for line in src.splitlines() if line.startswith("#include")]
     assert includes == ["<hip/hip_runtime.h>", "<algorithm>", "<cmath>", "<cstdint>", "<cstdio>", "<cstdlib>", "<vector>",
                         '"plexus_hip.h"']
+
+
+@pytest.mark.gpu
+def test_the_reference_side_binding_stub_replaces_torch_sparse_mm():
+    """plexus_amd/utils/hip_ops.py is the ctypes stub meant to be copied into the reference tree; it binds the library
+    on its own (no other module of this package) and stands in for torch.sparse.mm on a torch CSR tensor."""
+    import importlib
+
+    import torch
+
+    from plexus_amd import _lib
+
+    print("[case] reference-side ctypes stub", flush=True)
+    os.environ.setdefault("PLEXUS_HIP_LIB", _lib.LIB_PATH)
+    stub = importlib.import_module("plexus_amd.utils.hip_ops")
+    gen = torch.Generator().manual_seed(0)
+    n, d = 3000, 40
+    dense = (torch.rand(n, n, generator=gen) < 0.004).float() * torch.rand(n, n, generator=gen)
+    a_cpu = dense.to_sparse_csr()
+    h = torch.randn(n, d, generator=gen)
+    a = a_cpu.to("cuda")
+    stub.prepare(a)
+    y = stub.sparse_mm(a, h.to("cuda")).cpu()
+    ref = torch.sparse.mm(a_cpu, h)
+    assert ((y - ref).abs().max() / ref.abs().max()).item() <= 1e-5
