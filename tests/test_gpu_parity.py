@@ -918,6 +918,28 @@ def test_config1_ten_epochs_with_auto_association():
         assert abs(l - r64) <= FP32_TOL * abs(r64)
 
 
+def test_spmm_from_a_line_aligned_copy_of_h_gives_the_same_bits():
+    say("spmm: staging of H into line-aligned rows")
+    from plexus_amd import _lib
+
+    g = S.build_graph(3000, "chunglu", 40000, seed=9, device="cpu", gamma=2.1)  # about 27 entries per column of H
+    a = to_dev(g, seg_len=128)
+    lib = _lib.load()
+    for d, staged in ((47, True), (602, True), (100, False), (128, False)):
+        seg_only = a.n_segments * ((d + 3) // 4 * 4) * 4
+        need = int(lib.plx_spmm_workspace_bytes(a._plan, d))
+        assert (need > seg_only) == staged, (d, need, seg_only)
+        h = torch.randn(3000, d, generator=torch.Generator().manual_seed(d)).to(DEV)
+        y = ops.spmm(a, h)  # whole matrix: gathers from the copy when the workspace has room for it
+        y_rows = ops.chunked_spmm(a, h, max_rows_per_chunk=1100)  # row ranges never stage
+        assert torch.equal(y, y_rows)
+        assert rel_err(y.cpu(), oracle_spmm64(g, h.cpu())) <= FP32_TOL
+        # an operand that is already line-aligned is used where it lies
+        hp = torch.zeros(3000, (d + 31) // 32 * 32, device=DEV)
+        hp[:, :d] = h
+        assert torch.equal(ops.spmm(a, hp[:, :d]), y)
+
+
 def test_row_chunked_spmm_is_bit_identical_and_hands_chunks_on():
     say("row-chunked SpMM (blocked aggregation)")
     import plexus_amd
