@@ -113,10 +113,11 @@ int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
 /* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len */
 int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
-/* bytes of scratch an SpMM of width D needs: fp32 partial sums of the split rows, plus -- when every row of H is
- * gathered at least 16 times on average and rows of D fp32 elements would straddle more 128-byte lines than they
- * have to -- room for a copy of H in rows that start on lines, which whole-matrix products then gather from
- * (0.2 ms of copying against 3 ms saved at K = 232,965, D = 602).  0 if neither applies.  The result is unchanged. */
+/* bytes of scratch an SpMM of width D needs: fp32 partial sums of the split rows, plus -- when rows of D fp32
+ * elements laid end to end straddle more 128-byte lines than they have to and every row of H is gathered often
+ * enough to repay a copy -- room for a copy of H in rows that start on lines, which whole-matrix products then
+ * gather from (0.2 ms of copying against 3 ms saved at K = 232,965, D = 602, 492 gathers per row).  0 if neither
+ * applies.  The result is unchanged. */
 size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D);
 
 /* fp32 values, fp32 H and Y. */

@@ -445,12 +445,16 @@ int64_t offset_granule(uintptr_t base, int64_t pitch_bytes)
 // leading dimension (elements) of the staged copy, or 0 when staging does not pay
 int64_t staged_ld(int64_t K, int64_t nnz, int64_t D, int64_t elem, uintptr_t base, int64_t ldh)
 {
-    if (K <= 0 || nnz < 16 * K) return 0;  // each row of H must be gathered often enough to repay the copy
+    if (K <= 0) return 0;
     const int64_t row_bytes = D * elem;
     const int64_t g = offset_granule(base, ldh * elem);
     if (g == kLine) return 0;  // rows already start on lines
     const double aligned = (double)((row_bytes + kLine - 1) / kLine);
-    if (mean_lines(row_bytes, g) - aligned < 0.3) return 0;
+    const double saved = mean_lines(row_bytes, g) - aligned;  // lines per gathered row
+    if (saved < 0.3) return 0;
+    // the copy reads and writes H once; the gathers save `saved` lines each.  Stage when the saving is at least three
+    // times the bytes of a row per row of H (a copy streams, a gather does not: margin for that)
+    if ((double)nnz * saved * (double)kLine < 3.0 * (double)K * (double)row_bytes) return 0;
     return (row_bytes + kLine - 1) / kLine * kLine / elem;
 }
 

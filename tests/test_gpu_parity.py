@@ -922,10 +922,12 @@ def test_spmm_from_a_line_aligned_copy_of_h_gives_the_same_bits():
     say("spmm: staging of H into line-aligned rows")
     from plexus_amd import _lib
 
-    g = S.build_graph(3000, "chunglu", 40000, seed=9, device="cpu", gamma=2.1)  # about 27 entries per column of H
+    g = S.build_graph(3000, "chunglu", 40000, seed=9, device="cpu", gamma=2.1)
+    per_row_of_h = g.nnz / 3000  # about 27: enough to repay the copy of 188-byte rows, not that of 2,408-byte rows
+    assert 15 < per_row_of_h < 60
     a = to_dev(g, seg_len=128)
     lib = _lib.load()
-    for d, staged in ((47, True), (602, True), (100, False), (128, False)):
+    for d, staged in ((47, True), (602, False), (100, False), (128, False), (24, True)):
         seg_only = a.n_segments * ((d + 3) // 4 * 4) * 4
         need = int(lib.plx_spmm_workspace_bytes(a._plan, d))
         assert (need > seg_only) == staged, (d, need, seg_only)
