@@ -48,7 +48,8 @@ class CsrMatrix:
 
     Built from a torch sparse-CSR tensor (``from_torch``) or from raw arrays.  The plan (row binning
     and the split of long rows into segments) is computed once; the int32 arrays are owned here and
-    outlive it.
+    outlive it.  The scratch of the products is cached on the object, so products of one matrix must
+    be ordered (one stream, or events between streams); different matrices are independent.
     """
 
     def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, val: torch.Tensor, shape, seg_len: int = 0):
