@@ -14,16 +14,9 @@ tune_gemm = False
 _initialized = False
 
 
-def init(
-    G_intra_r: int = 1,
-    G_intra_c: int = 1,
-    G_intra_d: int = 1,
-    gpus_per_node: Optional[int] = None,
-    enable_internal_timers: bool = False,
-    block_aggregation: bool = False,
-    overlap_aggregation: bool = False,
-    tune_gemms: bool = False,
-) -> None:
+def init(G_intra_r: int = 1, G_intra_c: int = 1, G_intra_d: int = 1, gpus_per_node: Optional[int] = None,
+         enable_internal_timers: bool = False, block_aggregation: bool = False, overlap_aggregation: bool = False,
+         tune_gemms: bool = False) -> None:
     """Initialise the (one-GPU) runtime.
 
     Arguments keep the reference's meaning.  ``G_intra_r/c/d`` must all be 1.
