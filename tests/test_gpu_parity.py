@@ -942,6 +942,24 @@ def test_spmm_from_a_line_aligned_copy_of_h_gives_the_same_bits():
         assert torch.equal(ops.spmm(a, hp[:, :d]), y)
 
 
+def test_spmm_staging_with_bf16_rows_and_dense_reuse():
+    say("spmm: staging of bf16 rows and of 2,408-byte fp32 rows under heavy reuse")
+    g = S.build_graph(2000, "uniform", 0, seed=11, device="cpu", exact_pairs=100000)  # about 100 entries per column of H
+    assert g.nnz / 2000 > 90
+    a = to_dev(g, seg_len=64)
+    d = 602
+    from plexus_amd import _lib
+    assert int(_lib.load().plx_spmm_workspace_bytes(a._plan, d)) >= 2000 * 2432 + a.n_segments * 604 * 4  # room for the copy
+    for dtype, tol in ((torch.float32, FP32_TOL), (torch.bfloat16, 2.0 ** -8)):
+        h = torch.randn(2000, d, generator=torch.Generator().manual_seed(1)).to(dtype).to(DEV)
+        y = ops.spmm(a, h)  # contiguous rows: staged into line-aligned rows first
+        pitch = 640  # rows that already start on 128-byte lines are gathered where they lie
+        hp = torch.zeros(2000, pitch, device=DEV, dtype=dtype)
+        hp[:, :d] = h
+        assert torch.equal(ops.spmm(a, hp[:, :d]), y)
+        assert rel_err(y.float().cpu(), oracle_spmm64(g, h.float().cpu())) <= tol
+
+
 def test_row_chunked_spmm_is_bit_identical_and_hands_chunks_on():
     say("row-chunked SpMM (blocked aggregation)")
     import plexus_amd
