@@ -160,8 +160,9 @@ int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
  * rounding of an fp32 product), which costs 2.7 times less matrix-core time than the fp32 MFMA and leaves the
  * products bound by HBM.  Same arguments and meaning as plx_gemm_nn_f32 / plx_gemm_nt_f32 (same reference call
  * sites) plus a workspace of plx_gemm_f32_split_workspace_bytes(N, K) bytes (16-byte aligned) for the pieces of
- * B.  Requires K > 0; for N or K above 128 also K % 4 == 0 and A (and mask) 16-byte aligned with leading
- * dimensions that are multiples of 4 (PLX_ERR_INVALID otherwise -- the caller then uses the entry points above). */
+ * B.  Requires K > 0; for N or K above 128 also an even K and A (and mask) 8-byte aligned with even leading
+ * dimensions -- 128-bit loads when all of these are multiples of 4 elements / 16 bytes, pairs of 64-bit loads
+ * otherwise (PLX_ERR_INVALID for odd shapes -- the caller then uses the entry points above). */
 size_t plx_gemm_f32_split_workspace_bytes(int64_t N, int64_t K);
 int plx_gemm_nn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                           int64_t ldc, unsigned flags, void *workspace, size_t workspace_bytes, void *stream);

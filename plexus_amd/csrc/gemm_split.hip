@@ -96,10 +96,11 @@ __device__ __forceinline__ floatx16 mfma6(bf16x8 a0, bf16x8 a1, bf16x8 a2, bf16x
 // ------------------------------------------------------------------------------------------------
 // NT form.  Workgroups are persistent: workgroup b takes the row panels b, b + gridDim.x, ... and, per panel,
 // every column tile; the steps (panel, column tile, chunk) form one software pipeline in which the global
-// loads of step q + 1 are in flight while the MFMAs of step q run.  Requires A (and mask) 16-byte aligned
-// with leading dimensions that are multiples of 4, and K % 4 == 0.
+// loads of step q + 1 are in flight while the MFMAs of step q run.  AVEC = 4: A (and mask) 16-byte aligned with
+// leading dimensions that are multiples of 4 and K % 4 == 0, read with 128-bit loads.  AVEC = 2: everything a
+// multiple of 2 elements / 8 bytes (rows of 602 elements), read with pairs of 64-bit loads.
 // ------------------------------------------------------------------------------------------------
-template <int TN, bool MASKED>
+template <int TN, bool MASKED, int AVEC>
 __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitArgs g)
 {
     constexpr int BN = 32 * TN;
@@ -144,8 +145,29 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
         for (int p = 0; p < kAVec; ++p) {
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f), m = v;
             if (32 * p < rows_left && k < K) {
-                v = *reinterpret_cast<const float4 *>(pa);
-                if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
+                if constexpr (AVEC == 4) {
+                    v = *reinterpret_cast<const float4 *>(pa);
+                    if constexpr (MASKED) m = *reinterpret_cast<const float4 *>(pm);
+                } else {  // K is even: a pair lies inside the row or past its end as a whole
+                    const float2 lo = *reinterpret_cast<const float2 *>(pa);
+                    v.x = lo.x;
+                    v.y = lo.y;
+                    if constexpr (MASKED) {
+                        const float2 mlo = *reinterpret_cast<const float2 *>(pm);
+                        m.x = mlo.x;
+                        m.y = mlo.y;
+                    }
+                    if (k + 2 < K) {
+                        const float2 hi = *reinterpret_cast<const float2 *>(pa + 2);
+                        v.z = hi.x;
+                        v.w = hi.y;
+                        if constexpr (MASKED) {
+                            const float2 mhi = *reinterpret_cast<const float2 *>(pm + 2);
+                            m.z = mhi.x;
+                            m.w = mhi.y;
+                        }
+                    }
+                }
             }
             dst[p] = v;
             if constexpr (MASKED) mdst[p] = m;
@@ -461,17 +483,18 @@ int launch_resident_tn(const SplitArgs &g, int tn, unsigned blocks, hipStream_t 
 
 int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
 
-template <bool MASKED>
+template <bool MASKED, int AVEC>
 void launch_nt(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
 {
     switch (tn) {
-        case 1: gemm_split_nt_kernel<1, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
-        case 2: gemm_split_nt_kernel<2, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
-        default: gemm_split_nt_kernel<4, MASKED><<<blocks, kThreads, 0, st>>>(g); break;
+        case 1: gemm_split_nt_kernel<1, MASKED, AVEC><<<blocks, kThreads, 0, st>>>(g); break;
+        case 2: gemm_split_nt_kernel<2, MASKED, AVEC><<<blocks, kThreads, 0, st>>>(g); break;
+        default: gemm_split_nt_kernel<4, MASKED, AVEC><<<blocks, kThreads, 0, st>>>(g); break;
     }
 }
 
 bool aligned16(const void *p, int64_t ld) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0); }
+bool aligned8(const void *p, int64_t ld) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % 8 == 0 && ld % 2 == 0); }
 
 int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
 
@@ -487,9 +510,10 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     const int tn = pick_tn(N);
     const int64_t Np = round_up(N, 32 * tn), Kp = round_up(std::max<int64_t>(K, 1), kBK);
     const bool vec = aligned16(A, lda) && aligned16(mask, ldmask) && K % 4 == 0;
+    const bool vec2 = aligned8(A, lda) && aligned8(mask, ldmask) && K % 2 == 0;
     const bool resident = Np <= kRMaxN && Kp <= kRMaxK;  // this kernel also reads A element by element
-    PLX_REQUIRE(vec || resident,
-                "%s: for weights beyond 128 x 128, A and mask must be 16-byte aligned with leading dimensions and K multiples of 4", who);
+    PLX_REQUIRE(vec || vec2 || resident,
+                "%s: for weights beyond 128 x 128, A and mask must be 8-byte aligned with leading dimensions and K multiples of 2", who);
     const size_t need = (size_t)3 * Np * Kp * sizeof(uint16_t);
     if (workspace == nullptr || workspace_bytes < need)
         return plx::fail(PLX_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -510,10 +534,11 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
         return PLX_OK;
     }
     const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, kBM), 2 * 256);
-    if (mask != nullptr)
-        launch_nt<true>(g, tn, blocks, st);
-    else
-        launch_nt<false>(g, tn, blocks, st);
+    if (vec) {
+        if (mask != nullptr) launch_nt<true, 4>(g, tn, blocks, st); else launch_nt<false, 4>(g, tn, blocks, st);
+    } else {
+        if (mask != nullptr) launch_nt<true, 2>(g, tn, blocks, st); else launch_nt<false, 2>(g, tn, blocks, st);
+    }
     PLX_LAUNCH_CHECK("gemm_split_nt_kernel");
     return PLX_OK;
 }

@@ -317,7 +317,7 @@ def _split_ok(n: int, k: int, *mats) -> bool:
         return False
     if n <= 128 and k <= 128:  # the kernel for small weights takes any alignment
         return True
-    return k % 4 == 0 and all(t is None or (t.data_ptr() % 16 == 0 and _ld(t) % 4 == 0) for t in mats)
+    return k % 2 == 0 and all(t is None or (t.data_ptr() % 8 == 0 and _ld(t) % 2 == 0) for t in mats)
 
 
 def _split_ws(n: int, k: int, device):

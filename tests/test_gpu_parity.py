@@ -245,7 +245,7 @@ def test_split_gemm_is_taken_and_keeps_fp32_accuracy_on_hard_inputs():
     ws = torch.empty(need, dtype=torch.uint8, device=DEV)
     stream = torch.cuda.current_stream().cuda_stream
     assert lib.plx_gemm_nn_f32_split(m, n, k, ad.data_ptr(), k, bd.data_ptr(), n, cd.data_ptr(), n, 0, ws.data_ptr(), need - 1, stream) == _lib.PLX_ERR_WORKSPACE
-    # weights up to 128 x 128: any alignment and any K (element loads); beyond that the operands must allow 128-bit loads
+    # weights up to 128 x 128: any alignment and any K (element loads); beyond that the operands must allow 64-bit loads
     assert lib.plx_gemm_nn_f32_split(m - 1, n, k - 3, ad.data_ptr() + 4, k, bd.data_ptr(), n, cd.data_ptr(), n, 0, ws.data_ptr(), need, stream) == 0
     flat = ai.reshape(-1)[1:1 + (m - 1) * k].reshape(m - 1, k)[:, :k - 3]
     assert torch.equal(cd[:m - 1].cpu(), flat @ bi[:k - 3])
@@ -254,7 +254,28 @@ def test_split_gemm_is_taken_and_keeps_fp32_accuracy_on_hard_inputs():
     need2 = int(lib.plx_gemm_f32_split_workspace_bytes(n2, k2))
     ws2 = torch.empty(need2, dtype=torch.uint8, device=DEV)
     assert lib.plx_gemm_nn_f32_split(m, n2, k2, a2.data_ptr() + 4, k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == _lib.PLX_ERR_INVALID
-    assert lib.plx_gemm_nn_f32_split(m, n2, k2 - 2, a2.data_ptr(), k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == _lib.PLX_ERR_INVALID
+    assert lib.plx_gemm_nn_f32_split(m, n2, k2 - 3, a2.data_ptr(), k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == _lib.PLX_ERR_INVALID
+    assert lib.plx_gemm_nn_f32_split(m, n2, k2 - 2, a2.data_ptr() + 8, k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == 0
+
+
+@pytest.mark.parametrize("m,n,k", [(1500, 128, 602), (700, 200, 150), (333, 130, 258)])
+def test_split_gemm_with_64_bit_loads(m, n, k):
+    """Contraction lengths that are even but not multiples of 4 (rows of 602 elements are 8-byte aligned only): the
+    split kernels read them with pairs of 64-bit loads."""
+    say("split gemm, K %% 4 == 2: %dx%dx%d" % (m, n, k))
+    assert ops.SPLIT_GEMM and k % 4 == 2
+    gen = torch.Generator().manual_seed(k)
+    a, w, g = torch.randn(m, k, generator=gen), torch.randn(k, n, generator=gen), torch.randn(m, n, generator=gen)
+    assert ops._split_ok(n, k, a.to(DEV))
+    out = ops.gemm_nn(a.to(DEV), w.to(DEV), relu=True).cpu()
+    assert rel_err(out, torch.relu(a.double() @ w.double())) <= FP32_TOL
+    mask = torch.relu(torch.randn(m, n, generator=gen))
+    dagg = ops.gemm_nt(g.to(DEV), w.to(DEV), mask=mask.to(DEV)).cpu()  # contraction over n: aligned or not, as n falls
+    assert rel_err(dagg, (g.double() * (mask > 0)) @ w.double().t()) <= FP32_TOL
+    # contraction over k with a mask of k columns
+    g2, mask2 = torch.randn(m, k, generator=gen), torch.relu(torch.randn(m, k, generator=gen))
+    out2 = ops.gemm_nt(g2.to(DEV), w.t().contiguous().to(DEV), mask=mask2.to(DEV)).cpu()
+    assert rel_err(out2, (g2.double() * (mask2 > 0)) @ w.double()) <= FP32_TOL
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(3000, 128, 96), (777, 48, 128), (2049, 200, 40)])
