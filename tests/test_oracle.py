@@ -413,3 +413,129 @@ def test_partition_files_and_loader_restatement_vs_dense_slicing(tmp_path, parts
     yp = torch.zeros(big, dtype=torch.int64)
     yp[:n] = pg["y_2"] if layers % 2 == 0 else pg["y"]
     assert torch.equal(labels, yp[ranks[lg] * ls:(ranks[lg] + 1) * ls])
+
+
+# ---- the bf16-storage restatement (OracleNetBf16): pinned against OracleNet and against autograd ----
+def _ring_graph(n, dtype):
+    """Row i holds columns i-1, i, i+2 (mod n) with value 1: three entries per row and per column, not symmetric."""
+    rows = torch.arange(n).repeat_interleave(3)
+    cols = (rows + torch.tensor([-1, 0, 2]).repeat(n)) % n
+    a = torch.sparse_coo_tensor(torch.stack([rows, cols]), torch.ones(3 * n, dtype=dtype), (n, n)).to_sparse_csr()
+    return a, a.transpose(0, 1).to_sparse_csr()
+
+
+def test_bf16_oracle_equals_fp32_oracle_when_rounding_is_the_identity():
+    """Small-integer operands: every stored tensor is exactly representable in bf16, every rounding is the identity and
+    there is no dropout, so the bf16 restatement must give OracleNet's numbers bit for bit (forward, grad_x, grad_w).
+    A transposed weight, a mask taken from the wrong tensor or a misplaced product changes an integer somewhere."""
+    n, dims = 40, [5, 4, 3]
+    gen = torch.Generator().manual_seed(4)
+    for dtype in (torch.float32, torch.float64):
+        a, a_t = _ring_graph(n, dtype)
+        x = torch.randint(-1, 2, (n * dims[0],), generator=gen).to(dtype)
+        ws = [torch.randint(-1, 2, (dims[i] * dims[i + 1],), generator=gen).to(dtype) for i in range(2)]
+        g_logits = torch.randint(-1, 2, (n, dims[-1]), generator=gen).to(dtype)
+        ref = po.OracleNet(ws, dims)
+        out_ref = ref.forward(x, [(a, a_t)])
+        gx_ref, gw_ref = ref.backward(g_logits)
+        # precondition: everything the bf16 path stores survives the rounding unchanged
+        for agg, _, _, pre in ref._saved:
+            assert torch.equal(po.rb(agg), agg) and torch.equal(po.rb(pre), pre)
+        assert torch.equal(po.rb(gx_ref), gx_ref) and (ref._saved[0][3] > 0).any() and (ref._saved[0][3] < 0).any()
+        net = po.OracleNetBf16(ws, dims, dropout_p=0.0)
+        out = net.forward(x, [(a, a_t)])
+        gx, gw = net.backward(g_logits)
+        assert torch.equal(out, out_ref)
+        assert torch.equal(gx.reshape(-1), gx_ref.reshape(-1))
+        for u, v in zip(gw, gw_ref):
+            assert torch.equal(u, v) and u.abs().sum() > 0
+
+
+class _RoundBoth(torch.autograd.Function):
+    """bf16 rounding of a stored tensor: the value is rounded on the way forward and its gradient on the way back."""
+
+    @staticmethod
+    def forward(ctx, t):
+        return po.rb(t)
+
+    @staticmethod
+    def backward(ctx, g):
+        return po.rb(g)
+
+
+def _bf16_forward_autograd(x, ws, dims, a, p, keeps):
+    """The forward of OracleNetBf16 as a differentiable graph: weights rounded straight-through, stored activations
+    through _RoundBoth, the dropout keep-mask a constant factor."""
+    h = _RoundBoth.apply(x)
+    for i, w in enumerate(ws):
+        w2 = w.reshape(dims[i], dims[i + 1])
+        w_st = w2 + (po.rb(w2) - w2).detach()  # value rb(w), gradient passed to w unchanged
+        agg = _RoundBoth.apply(torch.sparse.mm(a, h.reshape(a.shape[1], dims[i])))
+        out = torch.mm(agg, w_st)
+        if i != len(ws) - 1:
+            out = F.relu(out)
+            if p > 0:
+                out = out * keeps[i] / (1.0 - p)
+        h = _RoundBoth.apply(out)
+    return h
+
+
+@pytest.mark.parametrize("p", [0.0, 0.5])
+def test_bf16_oracle_backward_equals_autograd_over_its_forward(p):
+    """Hand backward of OracleNetBf16 == torch.autograd over the same forward (fp64; power-of-two dropout scale, so both
+    orders of applying it give the same bits).  Fails if 1/(1-p) is missing or doubled in grad_w or grad_agg, if the
+    mask comes from a tensor that ignores dropout, or if a weight is transposed."""
+    n, dims, seed = 70, [9, 7, 6, 4], 5
+    a = small_graph(n=n, pairs=350, seed=21).double()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(n * dims[0], generator=gen, dtype=torch.float64)
+    ws = [torch.randn(dims[i] * dims[i + 1], generator=gen, dtype=torch.float64) for i in range(3)]
+    g_logits = torch.randn(n, dims[-1], generator=gen, dtype=torch.float64)
+    offsets = [11, 12, 13]
+    keeps = [torch.from_numpy(po.dropout_keep_mask(n * dims[i + 1], seed, offsets[i], p).reshape(n, dims[i + 1])).double()
+             for i in range(2)]
+
+    net = po.OracleNetBf16(ws, dims, dropout_p=p, seed=seed)
+    out = net.forward(x, [(a, a_t)], offsets=offsets)
+    gx, gw = net.backward(g_logits)
+
+    xs = x.clone().requires_grad_()
+    wt = [w.clone().requires_grad_() for w in ws]
+    out_ag = _bf16_forward_autograd(xs, wt, dims, a, p, keeps)
+    assert torch.equal(out, out_ag.detach())
+    grads = torch.autograd.grad(out_ag, [xs] + wt, g_logits)
+    scale = lambda t: t.abs().max()
+    assert (gx.reshape(-1) - grads[0]).abs().max() <= 1e-13 * scale(grads[0])
+    for u, v in zip(gw, grads[1:]):
+        assert (u - v).abs().max() <= 1e-13 * scale(v) and scale(v) > 0
+    if p > 0:  # the mask really dropped something, and dropped units carry no gradient
+        assert 0.3 < keeps[0].mean() < 0.7
+        assert (net._saved[0][2][keeps[0] == 0] == 0).all()
+
+
+def test_bf16_oracle_dropout_scale_appears_once():
+    """One hidden layer, p = 0.5: grad_w of the hidden layer and the gradient handed to the aggregation are exactly
+    1/(1-p) = 2 times what the same network gives when the kept units are selected by a 0/1 mask without rescaling
+    (computed here from the saved tensors with plain products)."""
+    n, dims, p, seed = 50, [6, 5, 3], 0.5, 2
+    a = small_graph(n=n, pairs=260, seed=31).double()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn(n * dims[0], generator=gen, dtype=torch.float64)
+    ws = [torch.randn(dims[i] * dims[i + 1], generator=gen, dtype=torch.float64) for i in range(2)]
+    g_logits = torch.randn(n, dims[-1], generator=gen, dtype=torch.float64)
+    net = po.OracleNetBf16(ws, dims, dropout_p=p, seed=seed)
+    net.forward(x, [(a, a_t)], offsets=[3, 4])
+    gx, gw = net.backward(g_logits)
+    keep = torch.from_numpy(po.dropout_keep_mask(n * dims[1], seed, 3, p).reshape(n, dims[1])).double()
+    agg0, _, out0, _ = net._saved[0]
+    agg1 = net._saved[1][0]
+    w0, w1 = (po.rb(w.reshape(dims[i], dims[i + 1])) for i, w in enumerate(ws))
+    pre0 = agg0 @ w0
+    assert torch.equal(out0, po.rb(F.relu(pre0) * keep * 2.0))
+    g1 = po.rb(g_logits)
+    assert torch.allclose(gw[1], (agg1.t() @ g1).reshape(-1), rtol=1e-13, atol=0)  # last layer: no scale at all
+    g_h = po.rb(a_t.to_dense() @ po.rb(g1 @ w1.t())) * ((pre0 > 0).double() * keep)  # unscaled, 0/1 selection
+    assert torch.allclose(gw[0], 2.0 * (agg0.t() @ g_h).reshape(-1), rtol=1e-12, atol=1e-14)
+    assert torch.allclose(gx.reshape(n, dims[0]), po.rb(a_t.to_dense() @ po.rb(2.0 * (g_h @ w0.t()))), rtol=1e-12, atol=1e-14)
