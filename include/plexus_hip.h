@@ -131,6 +131,18 @@ int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H
 int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const float *H,
                           int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
                           void *stream);
+/* The whole-matrix fp32 product for callers that CANNOT ALLOCATE device memory or bring a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same kernels and the same bits as plx_spmm_csr_f32, but the partial sums of the split rows live in a static device
+ * array of PLX_SPMM_STATIC_SCRATCH_BYTES (32 MiB, held by every GPU the library runs on until the process ends) and
+ * H is never copied into line-aligned rows.  The call allocates nothing; the array's device address is looked up on
+ * the first call on each device (make that call outside a capture).  A plan whose split rows need more than the
+ * array holds -- segments x ceil(D / 4) x 16 bytes -- is refused with PLX_ERR_WORKSPACE.  All calls on one GPU share
+ * the array: calls that may overlap there (different streams or host threads) race, so order them. */
+#define PLX_SPMM_STATIC_SCRATCH_BYTES (32u << 20)
+size_t plx_spmm_static_scratch_bytes(void);
+int plx_spmm_csr_f32_static(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
+                            int64_t ldy, void *stream);
 /* Diagnostic for the benchmark, not part of the path: performs about n_gathers reads of uniformly random rows
  * (D fp32 each, D in {16, 32, 64, 128, 256}) of `table` with the SpMM's load shape and nothing else, so that
  * timing it gives the memory system's ceiling for this access pattern on a table of this size.

@@ -17,9 +17,15 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
+
+// Scratch of plx_spmm_csr_f32_static: fp32 partial rows of the split rows.  Every GPU the library runs on holds its own
+// copy of this array, at its own address, until the process ends.
+constexpr size_t kStaticScratchBytes = PLX_SPMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace {
 
@@ -518,9 +524,11 @@ int launch_for_vec(const SpmmArgs &a, int lpr, int nacc, dim3 grid, hipStream_t 
     }
 }
 
+// `may_stage` = false: the workspace holds the partial rows of the split rows and nothing else (H is gathered where
+// it lies; same values in the same order, so the same result)
 template <typename T>
 int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const T *H, int64_t ldh,
-              int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
+              int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream, bool may_stage = true)
 {
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
     PLX_REQUIRE(row_begin >= 0 && row_begin <= row_end && row_end <= plan->M, "spmm: row range [%lld, %lld) outside [0, %lld)",
@@ -530,7 +538,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
-    const size_t need = plx_spmm_workspace_bytes(plan, D);
+    const size_t need = may_stage ? plx_spmm_workspace_bytes(plan, D) : (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
     if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return plx::fail(PLX_ERR_WORKSPACE, "spmm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     PLX_REQUIRE(need == 0 || (reinterpret_cast<uintptr_t>(workspace) % 16) == 0, "spmm: workspace not 16-byte aligned");
@@ -548,7 +556,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     // query reserves it for contiguous fp32 rows); the partial rows of split rows follow the staged copy.
     const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
     char *ws_base = static_cast<char *>(workspace);
-    if (row_begin == 0 && row_end == plan->M) {
+    if (may_stage && row_begin == 0 && row_end == plan->M) {
         const int64_t ld_st = staged_ld(plan->K, plan->nnz, D, (int64_t)sizeof(T), reinterpret_cast<uintptr_t>(H), ldh);
         const size_t st_bytes = (size_t)plan->K * (size_t)ld_st * sizeof(T);
         const size_t pad = ws_base ? (size_t)((kLine - reinterpret_cast<uintptr_t>(ws_base) % kLine) % kLine) : 0;
@@ -628,6 +636,29 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
         spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)D, Y, ldy);
         PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
     }
+    return PLX_OK;
+}
+
+// ---- the product without a caller's workspace: partial rows of the split rows in a static device array ----
+// In host code `scratch` is only a handle of the symbol; the address of the array on a device comes from
+// hipGetSymbolAddress with that device current, once per device (every device has its own copy).
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int static_scratch(void **out)
+{
+    int dev = -1;
+    PLX_HIP_CHECK(hipGetDevice(&dev));
+    PLX_REQUIRE(dev >= 0 && dev < kMaxDevices, "spmm_static: device ordinal %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        PLX_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        PLX_REQUIRE(ptr != nullptr, "spmm_static: hipGetSymbolAddress returned NULL");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
     return PLX_OK;
 }
 
@@ -820,6 +851,27 @@ int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t 
                           void *stream)
 {
     return spmm_impl<float>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+size_t plx_spmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int plx_spmm_csr_f32_static(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
+                            int64_t ldy, void *stream)
+{
+    PLX_REQUIRE(plan != nullptr, "spmm_static: plan is NULL");
+    PLX_REQUIRE(D >= 0 && D <= (1ll << 21), "spmm_static: bad feature width D=%lld (at most 2,097,152)", (long long)D);
+    const size_t need = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+    if (need > kStaticScratchBytes)
+        return plx::fail(PLX_ERR_WORKSPACE,
+                         "spmm_static: the %lld segments of the split rows need %zu bytes of partial sums at D=%lld, the static "
+                         "scratch holds %zu; use plx_spmm_csr_f32 with a workspace",
+                         (long long)plan->n_seg, need, (long long)D, kStaticScratchBytes);
+    void *ptr = nullptr;
+    const int rc = static_scratch(&ptr);
+    if (rc != PLX_OK) return rc;
+    // every partial row is written in full (columns < D) by its segment task before the reduction reads it, so nothing
+    // of an earlier call has to be cleared
+    return spmm_impl<float>(plan, 0, plan->M, val, H, ldh, D, Y, ldy, ptr, kStaticScratchBytes, stream, /*may_stage=*/false);
 }
 
 int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int64_t D, int64_t n_gathers, int64_t *gathers_done,
