@@ -414,20 +414,21 @@ def adamw_step(params, grads, state, lr=3e-3, betas=(0.9, 0.999), eps=1e-8, weig
         p.addcdiv_(m, denom, value=-lr / (1 - b1**t))
 
 
-def train_epochs(x0, weights, dims, adj_shards, labels, num_nodes, num_classes, epochs=10, lr=3e-3):
+def train_epochs(x0, weights, dims, adj_shards, labels, num_nodes, num_classes, epochs=10, lr=3e-3, masks_of_epoch=None):
     """examples/train.py:83-112,164-193: zero_grad -> fwd -> CE -> bwd -> AdamW over weights and features.
 
-    Returns the loss of every epoch and the final (features, weights).
+    Returns the loss of every epoch and the final (features, weights).  ``masks_of_epoch(e)`` (optional) gives the
+    ReLU masks the backward pass of epoch e uses in place of its own (see OracleNet.backward).
     """
     net = OracleNet(weights, dims)
     x = x0.clone().reshape(-1)
     state = {}
     losses = []
-    for _ in range(epochs):
+    for e in range(epochs):
         logits = net.forward(x, adj_shards)
         loss, softmax, onehot = cross_entropy_forward(logits, labels, num_nodes, num_classes)
         g = cross_entropy_backward(softmax, onehot.to(softmax.dtype), num_nodes)
-        gx, gws = net.backward(g)
+        gx, gws = net.backward(g, None if masks_of_epoch is None else masks_of_epoch(e))
         adamw_step(net.weights + [x], gws + [gx], state, lr=lr)
         losses.append(float(loss))
     return losses, x, net.weights
@@ -545,3 +546,25 @@ class OracleNetBf16:
             grad_agg = rb(scale * torch.mm(g, torch.t(w)))
             g = rb(torch.sparse.mm(a_t, grad_agg))
         return g, grads_w
+
+
+def train_epochs_bf16(x0, weights, dims, adj_shards, labels, num_nodes, num_classes, epochs=10, lr=3e-3, dropout_p=0.0,
+                      seed=0, offsets_of_epoch=None):
+    """The epoch loop of train_epochs (examples/train.py:83-112,164-193) over the bf16-storage network: the trained
+    tensors (weights, input features) stay in the working precision, the network reads their bf16 roundings, the
+    gradient of the features arrives rounded to bf16, the weight gradients do not.  ``offsets_of_epoch(e)`` gives the
+    dropout offsets of the layers in epoch e.
+    """
+    net = OracleNetBf16(weights, dims, dropout_p=dropout_p, seed=seed)
+    x = x0.clone().reshape(-1)
+    state = {}
+    losses = []
+    for e in range(epochs):
+        offsets = offsets_of_epoch(e) if offsets_of_epoch is not None else None
+        logits = net.forward(x, adj_shards, offsets)
+        loss, softmax, onehot = cross_entropy_forward(logits, labels, num_nodes, num_classes)
+        g = cross_entropy_backward(softmax, onehot.to(softmax.dtype), num_nodes)
+        gx, gws = net.backward(g)
+        adamw_step(net.weights + [x], gws + [gx.reshape(-1)], state, lr=lr)
+        losses.append(float(loss))
+    return losses, x, net.weights

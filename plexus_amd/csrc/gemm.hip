@@ -114,6 +114,50 @@ struct Tile {
     }
 };
 
+// Second level of the sum over rows in the TN product.  ON = false: no state, no code.
+constexpr int kFlushChunks = 8;  // 8 chunks of 32 rows = 128 accumulation steps of the 32x32x2 MFMA
+template <bool ON, int TN>
+struct TotalsTN {
+    __device__ __forceinline__ void chunk_done(floatx16 (&)[TN], int &) {}
+    __device__ __forceinline__ void finish(floatx16 (&)[TN]) {}
+};
+template <int TN>
+struct TotalsTN<true, TN> {
+    float tot[TN][16];
+    __device__ __forceinline__ TotalsTN()
+    {
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) tot[t][v] = 0.f;
+    }
+    __device__ __forceinline__ void flush(floatx16 (&acc)[TN])
+    {
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                tot[t][v] += acc[t][v];
+                acc[t][v] = 0.f;
+            }
+    }
+    __device__ __forceinline__ void chunk_done(floatx16 (&acc)[TN], int &since_flush)
+    {
+        if (++since_flush == kFlushChunks) {  // uniform over the workgroup
+            since_flush = 0;
+            flush(acc);
+        }
+    }
+    // leaves the totals in acc for the common store code
+    __device__ __forceinline__ void finish(floatx16 (&acc)[TN])
+    {
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[t][v] += tot[t][v];
+    }
+};
+
 template <int MODE, int TN>
 __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
 {
@@ -171,6 +215,11 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
+    // TN sums over the rows of the matrices, thousands of them per workgroup: every kFlushChunks chunks the accumulators
+    // of the matrix cores are added into a second set of totals and cleared, so that the rounding error grows with
+    // sqrt(kFlushChunks * 16) + sqrt(chunks / kFlushChunks) steps instead of sqrt(chunks * 16)
+    TotalsTN<MODE == kTN, TN> tot;
+
     int buf = 0;
     if (kbeg < kend) {
         fetch(kbeg);
@@ -179,6 +228,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     }
     __syncthreads();
 
+    int since_flush = 0;
     for (int64_t k0 = kbeg; k0 < kend; k0 += kBK) {
         const bool more = k0 + kBK < kend;
         if (more) fetch(k0 + kBK);
@@ -223,9 +273,11 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
             at.stash(a_buf(buf ^ 1));
             bt.stash(b_buf(buf ^ 1));
         }
+        tot.chunk_done(acc, since_flush);
         __syncthreads();
         buf ^= 1;
     }
+    tot.finish(acc);
 
     // accumulator register v of a lane is C[8 (v / 4) + 4 h + v % 4][lane % 32] of the 32 x 32 tile
     float *out;
@@ -271,7 +323,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
 // ~8 vector-ALU instructions per MFMA, which is what keeps its MFMA pipe half idle.
 // ---------------------------------------------------------------------------------------------------
 template <int MODE, int TN, bool MASKED>
-__global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g)
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm_f32_vec_kernel(const GemmArgs g)
 {
     constexpr int BN = 32 * TN;
     constexpr bool kAX = (MODE != kTN);
@@ -403,6 +455,8 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
+    TotalsTN<MODE == kTN, TN> tot;  // second-level totals of the long sum over rows (see gemm_f32_kernel)
+    int since_flush = 0;
     int buf = 0;
     if (kbeg < kend) {
         fetch();
@@ -442,9 +496,11 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_vec_kernel(const GemmArgs g
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[m], b[t][m], acc[t], 0, 0, 0);
         }
         if (more) stash(buf ^ 1);
+        tot.chunk_done(acc, since_flush);
         __syncthreads();
         buf ^= 1;
     }
+    tot.finish(acc);
 
     float *out;
     int64_t ldo, nrows, ncols;
@@ -494,12 +550,12 @@ __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ 
 {
     // 16 output elements per workgroup, 16 interleaved chains per element (chain j adds the partial tiles
     // j, j + 16, ... in order); the chains are then added in chain order: the same sum whatever the timing
-    __shared__ float part[16][17];
+    __shared__ double part[16][17];
     const int e_local = threadIdx.x & 15;
     const int chain = threadIdx.x >> 4;
     const int64_t e = (int64_t)blockIdx.x * 16 + e_local;
     const int64_t total = rows * cols;
-    float s = 0.f;
+    double s = 0.0;  // the partial tiles are added in fp64 and the sum is rounded once
     int64_t r = 0, c = 0;
     if (e < total) {
         r = e / cols;
@@ -509,21 +565,21 @@ __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ 
         int i = chain;
         for (; i + 48 < splits; i += 64) {  // four loads in flight per chain
             const float v0 = p[0], v1 = p[step], v2 = p[2 * step], v3 = p[3 * step];
-            s = (((s + v0) + v1) + v2) + v3;
+            s = (((s + (double)v0) + (double)v1) + (double)v2) + (double)v3;
             p += 4 * step;
         }
         for (; i < splits; i += 16) {
-            s += p[0];
+            s += (double)p[0];
             p += step;
         }
     }
     part[chain][e_local] = s;
     __syncthreads();
     if (chain == 0 && e < total) {
-        float t = part[0][e_local];
+        double t = part[0][e_local];
 #pragma unroll
         for (int j = 1; j < 16; ++j) t += part[j][e_local];
-        C[r * ldc + c] = t;
+        C[r * ldc + c] = (float)t;
     }
 }
 

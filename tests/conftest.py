@@ -49,6 +49,7 @@ def assert_parity(x, ref32, ref64, tol=FP32_TOL, what=""):
     e32 = rel_err(x, ref32)
     e64 = rel_err(x, ref64)
     ref_gap = rel_err(ref32, ref64)
+    print("%s: rel err vs fp32 oracle %.2e, vs fp64 oracle %.2e (fp32 oracle vs fp64 oracle %.2e)" % (what, e32, e64, ref_gap), flush=True)
     assert e32 <= tol or e64 <= tol or e64 <= ref_gap, (
         "%s: rel err vs fp32 oracle %.3e, vs fp64 oracle %.3e, fp32-vs-fp64 oracle gap %.3e" % (what, e32, e64, ref_gap)
     )

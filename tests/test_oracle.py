@@ -539,3 +539,35 @@ def test_bf16_oracle_dropout_scale_appears_once():
     g_h = po.rb(a_t.to_dense() @ po.rb(g1 @ w1.t())) * ((pre0 > 0).double() * keep)  # unscaled, 0/1 selection
     assert torch.allclose(gw[0], 2.0 * (agg0.t() @ g_h).reshape(-1), rtol=1e-12, atol=1e-14)
     assert torch.allclose(gx.reshape(n, dims[0]), po.rb(a_t.to_dense() @ po.rb(2.0 * (g_h @ w0.t()))), rtol=1e-12, atol=1e-14)
+
+
+def test_bf16_epoch_loop_matches_autograd_training():
+    """train_epochs_bf16 == the same bf16-storage model (rounded values, rounded stored gradients, constant dropout masks)
+    trained by torch autograd + F.cross_entropy + torch.optim.AdamW, in fp64."""
+    n, dims, p, seed, epochs = 70, [9, 7, 6, 4], 0.5, 5, 3
+    a = small_graph(n=n, pairs=350, seed=21).double()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    gen = torch.Generator().manual_seed(8)
+    x0 = torch.randn(n * dims[0], generator=gen, dtype=torch.float64)
+    ws = [torch.randn(dims[i] * dims[i + 1], generator=gen, dtype=torch.float64) * 0.3 for i in range(3)]
+    labels = torch.randint(0, dims[-1], (n,), generator=gen)
+    offs = lambda e: [i + 64 * e for i in range(3)]
+    losses, xf, wf = po.train_epochs_bf16(x0, ws, dims, [(a, a_t)], labels, n, dims[-1], epochs=epochs, dropout_p=p, seed=seed,
+                                          offsets_of_epoch=offs)
+    xs = x0.clone().requires_grad_()
+    wt = [w.clone().requires_grad_() for w in ws]
+    opt = torch.optim.AdamW(wt + [xs], lr=3e-3, weight_decay=0.0)
+    ref_losses = []
+    for e in range(epochs):
+        keeps = [torch.from_numpy(po.dropout_keep_mask(n * dims[i + 1], seed, offs(e)[i], p).reshape(n, dims[i + 1])).double()
+                 for i in range(2)]
+        opt.zero_grad()
+        loss = F.cross_entropy(_bf16_forward_autograd(xs, wt, dims, a, p, keeps), labels)
+        loss.backward()
+        opt.step()
+        ref_losses.append(float(loss.detach()))
+    assert np.allclose(losses, ref_losses, rtol=1e-12, atol=0)
+    assert torch.allclose(xf, xs.detach(), rtol=0, atol=1e-12)
+    for u_, v_ in zip(wf, wt):
+        assert torch.allclose(u_, v_.detach(), rtol=0, atol=1e-12)
+    assert losses[0] != losses[1]
