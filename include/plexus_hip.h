@@ -175,8 +175,9 @@ int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
  * B.  Requires K > 0; for N or K above 128 also an even K and A (and mask) 8-byte aligned with even leading
  * dimensions -- 128-bit loads when all of these are multiples of 4 elements / 16 bytes, pairs of 64-bit loads
  * otherwise (PLX_ERR_INVALID for odd shapes -- the caller then uses the entry points above).
- * Non-finite inputs, and finite ones whose bf16 rounding overflows (above 3.39e38), come out as NaN where the
- * fp32 kernels above give Inf. */
+ * Inf, NaN and finite values of 3.3895e38 or more (whose bf16 rounding overflows) behave as in the fp32 kernels
+ * above: an operand that holds one raises a flag on the device and the product is redone by the fp32 MFMA kernel (a
+ * launch that is always enqueued and returns at once otherwise). */
 size_t plx_gemm_f32_split_workspace_bytes(int64_t N, int64_t K);
 int plx_gemm_nn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                           int64_t ldc, unsigned flags, void *workspace, size_t workspace_bytes, void *stream);

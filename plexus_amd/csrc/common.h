@@ -31,6 +31,13 @@ constexpr int kWave = 64;
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// fp32 MFMA products that run only if one of n_run_if device words is non-zero (gemm.hip); same arguments as
+// plx_gemm_nn_f32 / plx_gemm_nt_f32 otherwise
+int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                   int64_t ldc, unsigned flags, const unsigned *run_if, int n_run_if, void *stream);
+int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream);
+
 }  // namespace plx
 
 #define PLX_HIP_CHECK(expr)                                                                            \

@@ -51,7 +51,19 @@ struct GemmArgs {
     int64_t ws_ld, ws_slab;
     unsigned flags;
     int a_vec, b_vec, m_vec;  // 1 when 128-bit global loads of that operand are legal
+    // when set, the launch does nothing unless one of these n_run_if device words (a few at most) is non-zero: the
+    // fp32 redo of a split product whose operands turned out to hold Inf / NaN
+    const unsigned *run_if;
+    int n_run_if;
 };
+
+__device__ __forceinline__ bool guard_says_skip(const GemmArgs &g)
+{
+    if (g.run_if == nullptr) return false;
+    unsigned any = 0;
+    for (int i = 0; i < g.n_run_if; ++i) any |= g.run_if[i];
+    return any == 0;
+}
 
 // ROWS x COLS tile of a row-major source, fetched as float4 per thread, zero-filled outside the source
 template <int ROWS, int COLS, int STRIDE>
@@ -172,6 +184,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     using BTile = Tile<(kBX ? BN : kBK), (kBX ? kBK : BN), kBStride>;
 
     __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+    if (guard_says_skip(g)) return;
     auto a_buf = [&](int i) { return lds + i * kASize; };
     auto b_buf = [&](int i) { return lds + 2 * kASize + i * kBSize; };
 
@@ -338,6 +351,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
     constexpr int kAPer = (kARows + kAPass - 1) / kAPass, kBPer = (kBRows + kBPass - 1) / kBPass;
 
     __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+    if (guard_says_skip(g)) return;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -634,12 +648,8 @@ int64_t tn_splits(int64_t M, int64_t N, int64_t K)
     return std::max<int64_t>(1, std::min(want, by_rows));
 }
 
-}  // namespace
-
-extern "C" {
-
-int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
-                    float *C, int64_t ldc, unsigned flags, void *stream)
+int gemm_nn_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                 int64_t ldc, unsigned flags, const unsigned *run_if, int n_run_if, void *stream)
 {
     int rc = check_common("gemm_nn", M, N, K, A, B, C);
     if (rc != PLX_OK) return rc < 0 ? rc : PLX_OK;
@@ -648,6 +658,7 @@ int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
     g.A = A; g.B = B; g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.flags = flags;
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb);
+    g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
     dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
     launch_gemm<kNN>(g, tn, grid, plx::as_stream(stream));
@@ -655,8 +666,8 @@ int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
     return PLX_OK;
 }
 
-int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
-                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *stream)
+int gemm_nt_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                 int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream)
 {
     int rc = check_common("gemm_nt", M, N, K, A, B, C);
     if (rc != PLX_OK) return rc < 0 ? rc : PLX_OK;
@@ -666,11 +677,42 @@ int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
     g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
     g.M = M; g.N = N; g.K = K;
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
+    g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
     dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
     launch_gemm<kNT>(g, tn, grid, plx::as_stream(stream));
     PLX_LAUNCH_CHECK("gemm_f32_kernel<NT>");
     return PLX_OK;
+}
+
+}  // namespace
+
+// the same two products, launched so that they run only if a device flag is set (used by the split products)
+namespace plx {
+int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                   int64_t ldc, unsigned flags, const unsigned *run_if, int n_run_if, void *stream)
+{
+    return gemm_nn_impl(M, N, K, A, lda, B, ldb, C, ldc, flags, run_if, n_run_if, stream);
+}
+int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream)
+{
+    return gemm_nt_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, run_if, n_run_if, stream);
+}
+}  // namespace plx
+
+extern "C" {
+
+int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, unsigned flags, void *stream)
+{
+    return gemm_nn_impl(M, N, K, A, lda, B, ldb, C, ldc, flags, nullptr, 0, stream);
+}
+
+int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *mask, int64_t ldmask, void *stream)
+{
+    return gemm_nt_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, nullptr, 0, stream);
 }
 
 size_t plx_gemm_tn_workspace_bytes(int64_t M, int64_t N, int64_t K)

@@ -44,6 +44,7 @@ struct SplitArgs {
     int64_t M, N, K;
     int64_t Np, Kp;
     unsigned flags;
+    unsigned *nonfinite;  // device word raised when an operand holds a value the split cannot carry
     int a_vec;  // A (and mask) 16-byte aligned, leading dimensions and K multiples of 4: 128-bit loads
     // TN form
     const float *B;
@@ -53,7 +54,8 @@ struct SplitArgs {
     int64_t ws_ld, ws_slab;
 };
 
-// x = p0 + p1 + p2 exactly (bf16 pieces, round to nearest even each); pieces of 2 values packed per word
+// x = p0 + p1 + p2 exactly (bf16 pieces, round to nearest even each); pieces of 2 values packed per word.  Holds for
+// every value that needs_care() does not name.
 __device__ __forceinline__ void split2(float x, float y, uint32_t &p0, uint32_t &p1, uint32_t &p2)
 {
     p0 = plx::pack_bf16x2(x, y);
@@ -63,12 +65,26 @@ __device__ __forceinline__ void split2(float x, float y, uint32_t &p0, uint32_t 
     p2 = plx::pack_bf16x2(sx, sy);
 }
 
+// Values the split cannot carry: Inf and NaN (Inf times a zero piece is NaN, where the fp32 product gives Inf), and finite
+// values of 0x7f7f8000 (3.3895e38) or more in magnitude, whose rounding to bf16 overflows.  One compare per element
+// (NaN fails the "less than").  A kernel that meets one raises the flag word of its call, and the whole product is then
+// redone by the fp32 MFMA kernel.
+__device__ __forceinline__ int needs_care(float x) { return !(fabsf(x) < 3.3895313892515355e38f) ? 1 : 0; }
+__device__ __forceinline__ int needs_care(const float4 &v) { return needs_care(v.x) | needs_care(v.y) | needs_care(v.z) | needs_care(v.w); }
+
+// One flag word behind the planes in the workspace: cleared by split_planes_kernel, raised by the product kernel
+// when it meets such a value in either operand (it sees every element of both; in the planes of the small operand
+// all of them show as Inf / NaN first pieces).
+constexpr size_t kFlagBytes = 256;
+
 // the three bf16 planes of a small fp32 matrix, optionally transposed: P[p][n][k] = piece p of X(n, k) with
-// X(n, k) = B[k][n] (transpose) or B[n][k]; zero outside N x K
+// X(n, k) = B[k][n] (transpose) or B[n][k]; zero outside N x K.  Also clears the flag word.
 __global__ void __launch_bounds__(256) split_planes_kernel(const float *__restrict__ B, int64_t ldb, int transpose, int64_t N,
-                                                           int64_t K, int64_t Np, int64_t Kp, uint16_t *__restrict__ P)
+                                                           int64_t K, int64_t Np, int64_t Kp, uint16_t *__restrict__ P,
+                                                           unsigned *__restrict__ flag)
 {
     const int64_t total = Np * Kp;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *flag = 0u;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t n = i / Kp, k = i % Kp;
         float x = 0.f;
@@ -79,6 +95,15 @@ __global__ void __launch_bounds__(256) split_planes_kernel(const float *__restri
         P[total + i] = (uint16_t)p1;
         P[2 * total + i] = (uint16_t)p2;
     }
+}
+
+// true if one of the eight bf16 values of a first-plane vector is Inf or NaN
+__device__ __forceinline__ bool plane0_nonfinite(const u32x4 &v)
+{
+    uint32_t t = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t |= (v[i] & 0x7f807f80u) + 0x00800080u;
+    return (t & 0x80008000u) != 0u;
 }
 
 // six piece products of one 32 x 32 x 16 block, smallest terms first
@@ -185,10 +210,13 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
 
     // B items of this thread: (plane, row, 16-byte vector) -> offset inside a chunk of the planes / inside LDS
     int b_goff[kBVec], b_loff[kBVec];
+    bool b_plane0[kBVec];
+    bool b_first_pass = true;
 #pragma unroll
     for (int j = 0; j < kBVec; ++j) {
         const int id = min((int)threadIdx.x + j * kThreads, kBItems - 1);  // surplus threads repeat the last item
         const int plane = id / (BN * 4), rem = id % (BN * 4);
+        b_plane0[j] = plane == 0;
         b_goff[j] = (int)(plane * g.Np * g.Kp + (int64_t)(rem >> 2) * g.Kp + (rem & 3) * 8);  // planes hold < 2^31 elements
         b_loff[j] = 3 * kAPlane + plane * kBPlane + (rem >> 2) * kS + (rem & 3) * 8;
     }
@@ -198,13 +226,22 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
         const uint16_t *pb = g.Bp + ((int64_t)b_ct * BN) * g.Kp + b_kc * kBK;
 #pragma unroll
         for (int j = 0; j < kBVec; ++j) rb[j] = *reinterpret_cast<const u32x4 *>(pb + b_goff[j]);
+        if (b_first_pass) {  // every chunk of the planes passes here once per workgroup: look for Inf / NaN in plane 0
+#pragma unroll
+            for (int j = 0; j < kBVec; ++j)
+                if (b_plane0[j] && __builtin_expect(plane0_nonfinite(rb[j]), 0)) *g.nonfinite = 1u;
+        }
         if (++b_kc == n_kc) {
             b_kc = 0;
-            if (++b_ct == n_ct) b_ct = 0;
+            if (++b_ct == n_ct) {
+                b_ct = 0;
+                b_first_pass = false;
+            }
         }
     };
     uint16_t *const a_dst = lds + rt * kS + kq * 4;
     auto stash = [&](const float4(&a)[kAVec], const float4(&am)[kAVec]) __attribute__((always_inline)) {
+        int care = 0;
 #pragma unroll
         for (int p = 0; p < kAVec; ++p) {
             float4 v = a[p];
@@ -212,6 +249,7 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
                 const float4 m = am[p];
                 v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
             }
+            care |= needs_care(v);
             uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
             split2(v.x, v.y, lo0, lo1, lo2);
             split2(v.z, v.w, hi0, hi1, hi2);
@@ -220,6 +258,7 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_split_nt_kernel(const SplitA
             *reinterpret_cast<uint2 *>(dst + kAPlane) = make_uint2(lo1, hi1);
             *reinterpret_cast<uint2 *>(dst + 2 * kAPlane) = make_uint2(lo2, hi2);
         }
+        if (__builtin_expect(care, 0)) *g.nonfinite = 1u;
 #pragma unroll
         for (int j = 0; j < kBVec; ++j)
             if ((int)threadIdx.x + j * kThreads < kBItems) *reinterpret_cast<u32x4 *>(lds + b_loff[j]) = rb[j];
@@ -331,8 +370,9 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
         for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
             const int plane = id / ((int)g.Np * vec_per_row), rem = id % ((int)g.Np * vec_per_row);
             const int row = rem / vec_per_row, q = rem % vec_per_row;
-            *reinterpret_cast<u32x4 *>(bres + plane * kBPlane + row * kRBS + q * 8) =
-                *reinterpret_cast<const u32x4 *>(g.Bp + ((int64_t)plane * g.Np + row) * g.Kp + q * 8);
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(g.Bp + ((int64_t)plane * g.Np + row) * g.Kp + q * 8);
+            *reinterpret_cast<u32x4 *>(bres + plane * kBPlane + row * kRBS + q * 8) = v;
+            if (plane == 0 && __builtin_expect(plane0_nonfinite(v), 0)) *g.nonfinite = 1u;  // Inf / NaN in the small operand
         }
     }
     __syncthreads();
@@ -405,6 +445,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     auto step = [&](int kc, float4(&cur)[2], float4(&mcur)[2]) __attribute__((always_inline)) {
         const bool live = kc < n_kc;
         if (live) {
+            int care = 0;
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
                 float4 v = cur[p];
@@ -412,6 +453,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                     const float4 m = mcur[p];
                     v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
                 }
+                care |= needs_care(v);
                 uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
                 split2(v.x, v.y, lo0, lo1, lo2);
                 split2(v.z, v.w, hi0, hi1, hi2);
@@ -420,6 +462,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                 *reinterpret_cast<uint2 *>(dst + kRAPlane) = make_uint2(lo1, hi1);
                 *reinterpret_cast<uint2 *>(dst + 2 * kRAPlane) = make_uint2(lo2, hi2);
             }
+            if (__builtin_expect(care, 0)) *g.nonfinite = 1u;
         }
         fetch(cur, mcur);
         if (live) {
@@ -514,24 +557,35 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     const bool resident = Np <= kRMaxN && Kp <= kRMaxK;  // this kernel also reads A element by element
     PLX_REQUIRE(vec || vec2 || resident,
                 "%s: for weights beyond 128 x 128, A and mask must be 8-byte aligned with leading dimensions and K multiples of 2", who);
-    const size_t need = (size_t)3 * Np * Kp * sizeof(uint16_t);
+    const size_t plane_bytes = (size_t)3 * Np * Kp * sizeof(uint16_t);  // a multiple of 16
+    const size_t need = plane_bytes + kFlagBytes;
     if (workspace == nullptr || workspace_bytes < need)
         return plx::fail(PLX_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
     PLX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, "%s: workspace must be 16-byte aligned", who);
     hipStream_t st = plx::as_stream(stream);
     uint16_t *planes = static_cast<uint16_t *>(workspace);
+    unsigned *flag_words = reinterpret_cast<unsigned *>(static_cast<char *>(workspace) + plane_bytes);
     split_planes_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(Np * Kp, 256), 4096), 256, 0, st>>>(B, ldb, transpose_b, N, K, Np,
-                                                                                                    Kp, planes);
+                                                                                                    Kp, planes, flag_words);
     PLX_LAUNCH_CHECK("split_planes_kernel");
+    // Inf / NaN / values next to FLT_MAX in either operand: the split product is then meaningless and the fp32 MFMA
+    // kernel redoes it.  That
+    // launch is always enqueued and returns at once unless the flag word is set.
+    auto redo = [&]() {
+        if (transpose_b)
+            return plx::gemm_nn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, flags, flag_words, 1, stream);
+        return plx::gemm_nt_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, flag_words, 1, stream);
+    };
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags; g.a_vec = vec;
+    g.nonfinite = flag_words;
     if (resident) {
         const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
         const int rc = mask != nullptr ? launch_resident_tn<true>(g, tn, blocks, st) : launch_resident_tn<false>(g, tn, blocks, st);
         if (rc != PLX_OK) return rc;
         PLX_LAUNCH_CHECK("gemm_split_nt_resident_kernel");
-        return PLX_OK;
+        return redo();
     }
     const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, kBM), 2 * 256);
     if (vec) {
@@ -540,7 +594,7 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
         if (mask != nullptr) launch_nt<true, 2>(g, tn, blocks, st); else launch_nt<false, 2>(g, tn, blocks, st);
     }
     PLX_LAUNCH_CHECK("gemm_split_nt_kernel");
-    return PLX_OK;
+    return redo();
 }
 
 }  // namespace
@@ -551,7 +605,7 @@ size_t plx_gemm_f32_split_workspace_bytes(int64_t N, int64_t K)
 {
     if (N <= 0 || K < 0) return 0;
     const int64_t Np = round_up(N, 32 * pick_tn(N)), Kp = round_up(std::max<int64_t>(K, 1), kBK);
-    return (size_t)3 * Np * Kp * sizeof(uint16_t);
+    return (size_t)3 * Np * Kp * sizeof(uint16_t) + kFlagBytes;
 }
 
 int plx_gemm_nn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,

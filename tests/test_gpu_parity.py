@@ -240,7 +240,7 @@ def test_split_gemm_is_taken_and_keeps_fp32_accuracy_on_hard_inputs():
     assert torch.equal(wide[:, 3:3 + n].cpu(), ai @ bi) and (wide[:, :3] == 0).all() and (wide[:, 3 + n:] == 0).all()
     lib = _lib.load()
     need = int(lib.plx_gemm_f32_split_workspace_bytes(n, k))
-    assert need == 3 * 64 * 128 * 2
+    assert need == 3 * 64 * 128 * 2 + 256  # three bf16 planes of the weight and the flag words of the Inf / NaN check
     ad, bd, cd = ai.to(DEV), bi.to(DEV), torch.empty(m, n, device=DEV)
     ws = torch.empty(need, dtype=torch.uint8, device=DEV)
     stream = torch.cuda.current_stream().cuda_stream
@@ -256,6 +256,85 @@ def test_split_gemm_is_taken_and_keeps_fp32_accuracy_on_hard_inputs():
     assert lib.plx_gemm_nn_f32_split(m, n2, k2, a2.data_ptr() + 4, k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == _lib.PLX_ERR_INVALID
     assert lib.plx_gemm_nn_f32_split(m, n2, k2 - 3, a2.data_ptr(), k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == _lib.PLX_ERR_INVALID
     assert lib.plx_gemm_nn_f32_split(m, n2, k2 - 2, a2.data_ptr() + 8, k2, b2.data_ptr(), n2, c2.data_ptr(), n2, 0, ws2.data_ptr(), need2, stream) == 0
+
+
+@pytest.mark.parametrize("k,n", [(128, 128), (100, 47), (256, 256), (602, 130)])  # resident kernel, chunked kernel, 64-bit loads
+def test_fp32_products_with_inf_nan_and_values_near_overflow_agree_with_torch(k, n):
+    """Inf, NaN and finite values whose bf16 rounding would overflow, in either operand: the default (split) products
+    give what torch.mm gives -- Inf where it gives Inf, NaN where NaN, the same finite numbers elsewhere."""
+    say("fp32 products with Inf / NaN / 3.4e38, K=%d N=%d" % (k, n))
+    gen = torch.Generator().manual_seed(k + n)
+    m = 700
+    big = 3.4e38  # above 0x7f7f8000: rounds to Inf in bf16
+    a0 = torch.randn(m, k, generator=gen)
+    w0 = torch.randn(k, n, generator=gen) * 0.1
+
+    def same(got, ref, what):
+        got, ref = got.cpu(), ref.cpu()
+        assert torch.equal(torch.isnan(got), torch.isnan(ref)), what + ": NaN pattern"
+        assert torch.equal(torch.isinf(got), torch.isinf(ref)) and torch.equal(got[torch.isinf(ref)], ref[torch.isinf(ref)]), what + ": Inf pattern"
+        fin = torch.isfinite(ref)
+        assert rel_err(got[fin], ref[fin]) <= FP32_TOL, what
+
+    def both_paths(fn):
+        keep = ops.SPLIT_GEMM
+        try:
+            ops.SPLIT_GEMM = True
+            y_split = fn()
+            ops.SPLIT_GEMM = False
+            y_mfma = fn()
+        finally:
+            ops.SPLIT_GEMM = keep
+        return y_split, y_mfma
+
+    cases = []
+    # the large operand: one special value per row, in rows 0..3 (the rest of row 1 cleared: whether a sum of finite
+    # terms next to 3.4e38 overflows depends on the order of summation)
+    a = a0.clone()
+    a[1, :] = 0.0
+    a[0, 3], a[1, 5], a[2, 7], a[3, 9] = float("inf"), big, float("nan"), float("-inf")
+    cases.append(("special values in A", a, w0))
+    # finite but huge everywhere in one row: no Inf may appear that fp32 does not produce
+    a = a0.clone()
+    a[10, :] = 0.0
+    a[10, 1] = big
+    a[11, :] = 0.0
+    a[11, 2] = -big
+    w = w0.clone()
+    w[1, :] = 0.5
+    w[2, :] = 2.0  # -3.4e38 * 2 overflows to -Inf in fp32 as well
+    cases.append(("huge finite values", a, w))
+    # the small operand
+    w = w0.clone()
+    w[2, 1], w[4, 3] = float("inf"), float("nan")
+    w[6, 5] = big
+    a = a0.clone()
+    a[:, 6] = a[:, 6].clamp(-0.9, 0.9)  # 3.4e38 * a stays finite; the other terms of these sums are tiny beside it
+    cases.append(("special values in W", a, w))
+    for what, a, w in cases:
+        ad, wd = a.to(DEV), w.to(DEV)
+        ref = torch.mm(ad, wd)
+        y_split, y_mfma = both_paths(lambda: ops.gemm_nn(ad, wd))
+        same(y_split, ref, what + " (NN, split)")
+        same(y_mfma, ref, what + " (NN, fp32 MFMA)")
+        same(y_split, torch.mm(a, w), what + " (NN, split vs host)")
+        # NT form with the ReLU mask: GRAD_AGG = (G * [mask > 0]) . W^T with W stored (n_out = k here, n_in = n): use W^T of the above
+        wt = wd.t().contiguous()  # [n, k]
+        mask = torch.randn(m, k, generator=gen).to(DEV)
+        mask[0:12] = 1.0  # keep the special rows
+        ref_nt = torch.mm(torch.where(mask > 0, ad, torch.zeros_like(ad)), wt.t())
+        z_split, z_mfma = both_paths(lambda: ops.gemm_nt(ad, wt, mask=mask))
+        same(z_split, ref_nt, what + " (NT + mask, split)")
+        same(z_mfma, ref_nt, what + " (NT + mask, fp32 MFMA)")
+        # a special value under a zero of the mask does not exist for the product
+        mask2 = mask.clone()
+        mask2[0:12] = -1.0
+        clean = torch.where(mask2 > 0, ad, torch.zeros_like(ad))
+        z2, _ = both_paths(lambda: ops.gemm_nt(ad, wt, mask=mask2))
+        same(z2, torch.mm(clean, wt.t()), what + " (NT, special rows masked out)")
+    # and a clean product right after a flagged one (the flag words are cleared per call)
+    y_split, _ = both_paths(lambda: ops.gemm_nn(a0.to(DEV), w0.to(DEV)))
+    assert torch.isfinite(y_split).all() and rel_err(y_split, torch.mm(a0, w0)) <= FP32_TOL
 
 
 @pytest.mark.parametrize("m,n,k", [(1500, 128, 602), (700, 200, 150), (333, 130, 258)])
