@@ -152,6 +152,10 @@ int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int
 /* fp32 values, bf16 H and Y (raw uint16 bit patterns), fp32 accumulation, round-to-nearest-even store. */
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
                       uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
+/* rows [row_begin, row_end) of the bf16 product, as plx_spmm_csr_rows_f32 (plexus/gcn_conv.py:67-128) */
+int plx_spmm_csr_rows_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const uint16_t *H,
+                           int64_t ldh, int64_t D, uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                           void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Dense products of the layer (all replace tuned_matmul -> torch.mm, plexus/utils/matmul_tuning.py:94-95)

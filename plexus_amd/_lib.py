@@ -43,6 +43,7 @@ SIGNATURES = {
     "plx_spmm_csr_f32_static": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
     "plx_diag_random_gather_f32": (C.c_int, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_i64), _vp, _vp]),
     "plx_spmm_csr_bf16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_spmm_csr_rows_bf16": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_gemm_nn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp]),
     "plx_gemm_f32_split_workspace_bytes": (_sz, [_i64, _i64]),
     "plx_gemm_nn_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp, _sz, _vp]),

@@ -38,6 +38,19 @@ int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
 int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                    int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream);
 
+#if defined(__HIPCC__)
+// Orders the LDS accesses of one wavefront for the compiler: lanes that exchange data through a tile private to their
+// wavefront (no workgroup barrier) put this between the stores of one phase and the loads of the next.  The hardware
+// executes a wavefront's LDS instructions in order; this keeps the compiler from reordering them.  No instruction
+// besides what the fence needs at wavefront scope.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+#endif
+
 }  // namespace plx
 
 #define PLX_HIP_CHECK(expr)                                                                            \

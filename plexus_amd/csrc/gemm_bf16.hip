@@ -358,6 +358,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 *reinterpret_cast<uint4 *>(a_dst + 8 * j) = MASKED ? mask8(cur[j], mcur[MASKED ? j : 0]) : cur[j];
+            plx::wave_lds_fence();  // the chunk other lanes stored is read below
         }
         fetch(cur, mcur);
         if (live) {
@@ -370,6 +371,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
                 }
             }
+            plx::wave_lds_fence();  // the next position (or the epilogue) overwrites the private tile
         }
     };
 
@@ -391,8 +393,10 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
             for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
                 for (int v = 0; v < 8; ++v) cs[(8 * (v / 4) + 4 * h + (v % 4)) * kRCS + li] = acc[t][8 * pass + v];
+                plx::wave_lds_fence();  // staged by all lanes, read back transposed
                 const float4 lo = *reinterpret_cast<const float4 *>(cs + srow * kRCS + scq * 8);
                 const float4 hi = *reinterpret_cast<const float4 *>(cs + srow * kRCS + scq * 8 + 4);
+                plx::wave_lds_fence();  // before the next pass (or the next panel's chunks) overwrites the tile
                 const int64_t row = panel * 32 + 16 * pass + srow;
                 const int col = t * 32 + scq * 8;
                 if (row < g.M && col < N) {

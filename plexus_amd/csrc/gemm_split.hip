@@ -463,6 +463,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                 *reinterpret_cast<uint2 *>(dst + 2 * kRAPlane) = make_uint2(lo2, hi2);
             }
             if (__builtin_expect(care, 0)) *g.nonfinite = 1u;
+            plx::wave_lds_fence();  // the pieces other lanes stored are read below
         }
         fetch(cur, mcur);
         if (live) {
@@ -477,6 +478,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                 const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bk + t * 32 * kRBS + 2 * kBPlane);
                 acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
             }
+            plx::wave_lds_fence();  // the next position overwrites the private tile
         }
     };
 

@@ -907,4 +907,11 @@ int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_
     return spmm_impl<uint16_t>(plan, 0, plan ? plan->M : 0, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
 }
 
+int plx_spmm_csr_rows_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const uint16_t *H,
+                           int64_t ldh, int64_t D, uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                           void *stream)
+{
+    return spmm_impl<uint16_t>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
 }  // extern "C"

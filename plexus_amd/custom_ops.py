@@ -8,11 +8,13 @@ without a graph break.  They run the same entry points of libplexus_hip in the s
 bit-identical to the autograd-function path.
 
 A CSR matrix travels as its three arrays plus its shape; the prepared form (int32 indices, row plan) is looked up
-in a cache keyed by the arrays' addresses and built on first use.
+in a small least-recently-used cache keyed by the arrays' addresses and built on first use; an entry holds the
+arrays it was made from, so their addresses cannot pass to another matrix while it lives.
 
     out  = gcn_conv(x, A, At, weight, d_in, d_out, fuse_relu)      # A, At: ops.CsrMatrix or torch CSR tensors
     loss = cross_entropy(logits, target, num_nodes, num_classes)
 """
+import collections
 from typing import Tuple
 
 import torch
@@ -20,7 +22,21 @@ from torch import Tensor
 
 from . import ops
 
-_PLANS = {}
+
+class _Entry:
+    """A prepared matrix and the caller's arrays it was made from.  Holding the arrays keeps their memory from being
+    freed and handed to another matrix while their addresses are the key; their version counters tell an in-place
+    edit from an unchanged tensor."""
+
+    __slots__ = ("rowptr", "col", "val", "versions", "csr")
+
+    def __init__(self, rowptr, col, val, csr):
+        self.rowptr, self.col, self.val, self.csr = rowptr, col, val, csr
+        self.versions = (rowptr._version, col._version, val._version)
+
+
+_PLANS = collections.OrderedDict()  # least recently used first
+MAX_PLANS = 16  # a prepared matrix keeps its index arrays and its scratch (which can hold a copy of H) on the device
 
 
 def clear_plan_cache() -> None:
@@ -28,13 +44,26 @@ def clear_plan_cache() -> None:
     _PLANS.clear()
 
 
+def _remember(key, entry) -> None:
+    _PLANS[key] = entry
+    _PLANS.move_to_end(key)
+    while len(_PLANS) > MAX_PLANS:
+        _PLANS.popitem(last=False)
+
+
 def _prepared(rowptr: Tensor, col: Tensor, val: Tensor, rows: int, cols: int) -> ops.CsrMatrix:
     key = (rowptr.data_ptr(), col.data_ptr(), val.data_ptr(), int(rows), int(cols), int(col.numel()))
-    a = _PLANS.get(key)
-    if a is None:
-        a = ops.CsrMatrix(rowptr, col, val, (int(rows), int(cols)))
-        _PLANS[key] = a
-    return a
+    e = _PLANS.get(key)
+    if e is not None and (e.rowptr._version, e.col._version) != e.versions[:2]:
+        e = None  # the structure was edited in place: a new plan
+    if e is None:
+        e = _Entry(rowptr, col, val, ops.CsrMatrix(rowptr, col, val, (int(rows), int(cols))))
+    elif e.val._version != e.versions[2]:
+        if e.csr.val.data_ptr() != e.val.data_ptr():  # the prepared matrix holds a converted copy of the values: refresh it
+            e.csr.val = e.val.to(torch.float32).contiguous()
+        e.versions = e.versions[:2] + (e.val._version,)
+    _remember(key, e)
+    return e.csr
 
 
 def _parts(a):
@@ -42,7 +71,8 @@ def _parts(a):
     into the cache under its own arrays, so it is not prepared twice."""
     a = ops.as_csr(a)
     key = (a.rowptr.data_ptr(), a.col.data_ptr(), a.val.data_ptr(), a.shape[0], a.shape[1], a.nnz)
-    _PLANS.setdefault(key, a)
+    if key not in _PLANS:
+        _remember(key, _Entry(a.rowptr, a.col, a.val, a))
     return a.rowptr, a.col, a.val, a.shape[0], a.shape[1]
 
 

@@ -74,7 +74,7 @@ class GCNConvFunction(torch.autograd.Function):
         H = x.detach().reshape(local_features_shape)
 
         timers.start("AGG = A * H")
-        if plx.block_agg and not bf16:
+        if plx.block_agg:
             # blocked aggregation (plexus/gcn_conv.py:184-185): same rows, one launch per chunk of <= 1 M rows
             AGG = ops.chunked_spmm(A, H)
         else:

@@ -39,6 +39,13 @@ def _rowmajor(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def _need_fp32(who: str, **tensors) -> None:
+    """The fp32 entry points read raw pointers: anything but float32 would be misread without an error."""
+    for name, t in tensors.items():
+        if t is not None and t.dtype != torch.float32:
+            raise TypeError("%s: %s must be float32, got %s" % (who, name, t.dtype))
+
+
 def _ld(t: torch.Tensor) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
 
@@ -283,24 +290,25 @@ def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk
     a = as_csr(a)
     _need_gpu(h)
     h = _rowmajor(h)
-    if h.dtype != torch.float32:
-        raise TypeError("chunked_spmm: fp32 only")
+    lib = _lib.load()
+    fn = {torch.float32: lib.plx_spmm_csr_rows_f32, torch.bfloat16: lib.plx_spmm_csr_rows_bf16}.get(h.dtype)
+    if fn is None:
+        raise TypeError("chunked_spmm: unsupported dtype %s" % h.dtype)
     m, k = a.shape
     if h.shape[0] != k:
         raise ValueError("chunked_spmm: A is %dx%d but H has %d rows" % (m, k, h.shape[0]))
     d = h.shape[1]
-    y = torch.empty((m, d), dtype=torch.float32, device=h.device)
+    y = torch.empty((m, d), dtype=h.dtype, device=h.device)
     ws, ws_bytes = a._workspace(d)
-    lib = _lib.load()
     num_chunks = max(1, (m + max_rows_per_chunk - 1) // max_rows_per_chunk)
     rows_per_chunk = m // num_chunks
     for i in range(num_chunks):
         start = i * rows_per_chunk
         end = m if i == num_chunks - 1 else (i + 1) * rows_per_chunk
         check(
-            lib.plx_spmm_csr_rows_f32(a._plan, start, end, a.val.data_ptr(), h.data_ptr(), _ld(h), d, y.data_ptr(), _ld(y),
-                                      ws.data_ptr() if ws is not None else None, ws_bytes, _stream()),
-            "plx_spmm_csr_rows_f32",
+            fn(a._plan, start, end, a.val.data_ptr(), h.data_ptr(), _ld(h), d, y.data_ptr(), _ld(y),
+               ws.data_ptr() if ws is not None else None, ws_bytes, _stream()),
+            "plx_spmm_csr_rows",
         )
         if on_chunk is not None:
             on_chunk(i, (start, end), y)
@@ -328,6 +336,7 @@ def _split_ws(n: int, k: int, device):
 def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix."""
     _need_gpu(a, b, out)
+    _need_fp32("gemm_nn", a=a, b=b)
     a, b = _rowmajor(a), _rowmajor(b)
     m, k = a.shape
     k2, n = b.shape
@@ -358,6 +367,7 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """C = (A * [mask > 0]).B^T with B stored [N x K]."""
     _need_gpu(a, b, mask)
+    _need_fp32("gemm_nt", a=a, b=b, mask=mask)
     a, b = _rowmajor(a), _rowmajor(b)
     m, k = a.shape
     n, k2 = b.shape
@@ -389,6 +399,7 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
 def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """C[K x N] = A[M x K]^T.(B * [mask > 0])[M x N]."""
     _need_gpu(a, b, mask)
+    _need_fp32("gemm_tn", a=a, b=b, mask=mask)
     a, b = _rowmajor(a), _rowmajor(b)
     m, k = a.shape
     m2, n = b.shape

@@ -94,3 +94,55 @@ def test_dispatcher_checks_and_tracing_without_graph_breaks():
     traced = compiled(xd)
     (g_traced,) = torch.autograd.grad(traced, xd)
     assert torch.equal(eager, traced) and torch.equal(g_eager, g_traced)
+
+
+@pytest.mark.gpu
+def test_plan_cache_never_serves_another_matrix_and_sees_in_place_edits():
+    """The prepared form of a matrix is cached under the addresses of the caller's arrays.  int64 indices (what torch CSR
+    tensors carry) and non-fp32 values are converted to copies, so the caller's arrays can be dropped while the entry
+    lives: a later matrix of the same shape and entry count must still get its own product, an in-place edit of the
+    values must be seen, and the cache stays bounded."""
+    print("[case] plan cache of the custom operators: freed arrays, same-size successor, in-place edit, bound", flush=True)
+    dev = "cuda"
+    co.clear_plan_cache()
+    n, d_in, d_out, nnz = 400, 16, 8, 3000
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, d_in, generator=gen)
+    w = torch.randn(d_in, d_out, generator=gen)
+
+    def random_csr(seed):
+        g = torch.Generator().manual_seed(seed)
+        flat = torch.randperm(n * n, generator=g)[:nnz].sort().values  # nnz distinct positions: every matrix has exactly nnz entries
+        rows, cols = flat // n, flat % n
+        rowptr = torch.zeros(n + 1, dtype=torch.int64)
+        rowptr[1:] = torch.cumsum(torch.bincount(rows, minlength=n), 0)
+        return rowptr, cols, torch.rand(nnz, generator=g, dtype=torch.float64) + 0.5
+
+    def run(rowptr, col, val):
+        out, _ = torch.ops.plexus_amd.gcn_conv(x.to(dev).reshape(-1), rowptr, col, val, rowptr, col, val, n, n, w.to(dev).reshape(-1),
+                                               d_in, d_out, False)
+        return out.cpu()
+
+    def expect(rowptr, col, val):
+        a = torch.sparse_csr_tensor(rowptr, col, val.float(), size=(n, n))
+        return torch.mm(torch.sparse.mm(a, x), w)
+
+    for seed in range(3):  # each round drops the previous arrays before allocating arrays of the same sizes
+        rowptr, col, val = random_csr(seed)
+        rd, cd, vd = rowptr.to(dev), col.to(dev), val.to(dev)
+        assert torch.allclose(run(rd, cd, vd), expect(rowptr, col, val), rtol=1e-5, atol=1e-5), "matrix %d" % seed
+        if seed == 2:  # values edited in place (the prepared matrix holds an fp32 copy of these fp64 values)
+            vd.mul_(2.0)
+            assert torch.allclose(run(rd, cd, vd), 2.0 * expect(rowptr, col, val), rtol=1e-5, atol=1e-5)
+            cd.copy_(torch.flip(cd, [0]) * 0 + cd)  # an in-place write that leaves the structure as it is: still a valid plan
+            assert torch.allclose(run(rd, cd, vd), 2.0 * expect(rowptr, col, val), rtol=1e-5, atol=1e-5)
+        del rd, cd, vd
+    keep = []
+    for seed in range(co.MAX_PLANS + 3):
+        rowptr, col, val = random_csr(100 + seed)
+        keep.append((rowptr.to(dev), col.to(dev), val.to(dev)))
+        run(*keep[-1])
+    assert len(co._PLANS) == co.MAX_PLANS
+    rowptr, col, val = random_csr(100)  # evicted meanwhile: prepared again, same result
+    assert torch.allclose(run(*keep[0]), expect(rowptr, col, val), rtol=1e-5, atol=1e-5)
+    co.clear_plan_cache()

@@ -1090,6 +1090,42 @@ def test_row_chunked_spmm_is_bit_identical_and_hands_chunks_on():
     plexus_amd.init()
     for u, v in zip(*outs):
         assert torch.equal(u, v)
+    # bf16 storage: the same row ranges of the bf16 product, bit for bit, alone and through the layer
+    hb = h.to(torch.bfloat16)
+    full_b = ops.spmm(a, hb)
+    assert full_b.dtype == torch.bfloat16 and torch.equal(ops.chunked_spmm(a, hb, max_rows_per_chunk=700), full_b)
+    outs = []
+    for blocked in (False, True):
+        plexus_amd.init(block_aggregation=blocked)
+        layer = GCNConv(36, 8, 1, weight=w, fuse_relu=True)
+        x = hb.clone().requires_grad_()
+        o = layer(x, [(a, to_dev(g, True))])
+        o.float().sum().backward()
+        outs.append((o.detach(), x.grad, layer.weight.grad))
+    plexus_amd.init()
+    for u, v in zip(*outs):
+        assert torch.equal(u, v)
+
+
+def test_fp32_wrappers_reject_other_dtypes():
+    say("dtype checks of the fp32 products")
+    a = torch.randn(64, 16, device=DEV)
+    b = torch.randn(16, 8, device=DEV)
+    g = torch.randn(64, 8, device=DEV)
+    for bad in (a.double(), a.half(), a.to(torch.bfloat16)):
+        with pytest.raises(TypeError, match="float32"):
+            ops.gemm_nn(bad, b)
+        with pytest.raises(TypeError, match="float32"):
+            ops.gemm_tn(bad, g)
+    with pytest.raises(TypeError, match="float32"):
+        ops.gemm_nn(a, b.double())
+    with pytest.raises(TypeError, match="mask must be float32"):
+        ops.gemm_nt(g, b, mask=g > 0)
+    with pytest.raises(TypeError, match="mask must be float32"):
+        ops.gemm_tn(a, g, mask=(g > 0))
+    with pytest.raises(TypeError):
+        ops.chunked_spmm(ops.CsrMatrix(torch.zeros(65, dtype=torch.int64, device=DEV), torch.zeros(0, dtype=torch.int64, device=DEV),
+                                       torch.zeros(0, device=DEV), (64, 64)), a.double())
 
 
 def test_device_csr_transpose_matches_host_construction():
