@@ -113,11 +113,19 @@ int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
 /* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len */
 int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
+/* Column slicing of H.  When the rows of H taken whole overflow the last-level cache while a 256-byte slice of every row
+ * stays in it, and every row is gathered often, whole-matrix products run as passes over 256-byte column slices
+ * (233 K rows, 492 entries per row, 602 fp32 columns: 31.0 -> 18.4 ms).  The choice depends on the plan, the width and
+ * the element size only, and every product of a sliced shape -- whole matrix or row range, sliced in place, from a
+ * line-aligned copy, or in one pass when neither is possible -- sums each element in the same order, so they agree bit
+ * for bit.  mode 0: decide by that rule (the default); 1: slice whenever a row exceeds 256 bytes; -1: never. */
+int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
 /* bytes of scratch an SpMM of width D needs: fp32 partial sums of the split rows, plus -- when rows of D fp32
  * elements laid end to end straddle more 128-byte lines than they have to and every row of H is gathered often
  * enough to repay a copy -- room for a copy of H in rows that start on lines, which whole-matrix products then
  * gather from (0.2 ms of copying against 3 ms saved at K = 232,965, D = 602, 492 gathers per row).  0 if neither
- * applies.  The result is unchanged. */
+ * applies; for a sliced shape (above) whose contiguous rows do not start on 128-byte lines, room for that copy as well.
+ * The result does not depend on whether the copy is used. */
 size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D);
 
 /* fp32 values, fp32 H and Y. */

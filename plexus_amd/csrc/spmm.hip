@@ -50,6 +50,7 @@ struct SpmmArgs {
     int32_t row_begin;
     int32_t row_end;
     int32_t seg_base;  // index of the first segment task in the plan's tables
+    int32_t y_vec;     // 1: rows of Y take VEC-wide stores; 0: element stores, each guarded by the width D
 };
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
@@ -170,6 +171,9 @@ __device__ __forceinline__ void store_f32(float *p, const float (&v)[VEC])
     }
 }
 
+__device__ __forceinline__ void store_elem(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store_elem(uint16_t *p, float v) { *p = (uint16_t)f32_to_bf16(v); }
+
 // value of `x` held by lane `src`; `src` differs between lane groups when G > 1
 template <int G>
 __device__ __forceinline__ int pick_i(int x, int src)
@@ -185,13 +189,18 @@ __device__ __forceinline__ float pick_f(float x, int src)
     return __int_as_float(pick_i<G>(__float_as_int(x), src));
 }
 
-template <typename TIN, typename TOUT, int VEC, int LPR, int NACC>
+// R > 1: every lane group keeps R accumulator sets ("chains") and entry number q of a task (counted from the task's
+// first entry) goes to chain q mod (G * R) -- group q mod G, set (q / G) mod R.  The chains are added pairwise in the
+// order a kernel with G * R lane groups adds its groups, so the sum has the same bits as that kernel's.
+template <typename TIN, typename TOUT, int VEC, int LPR, int NACC, int R = 1>
 __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
 {
     constexpr int G = kWave / LPR;
     static_assert(G == 1 || NACC == 1, "several accumulator vectors only with one group");
-    // gathers kept in flight per lane = U * NACC
-    constexpr int U = (G >= 8) ? 1 : (G == 4) ? 2 : (G == 2) ? 4 : (NACC <= 2 ? 4 : (NACC <= 4 ? 2 : 1));
+    static_assert((R & (R - 1)) == 0 && R >= 1 && G * R <= kWave, "chains per group: a power of two");
+    // gathers kept in flight per lane = U * NACC; U is a multiple of R so that the chain of a load is known statically
+    constexpr int U0 = (G >= 8) ? 1 : (G == 4) ? 2 : (G == 2) ? 4 : (NACC <= 2 ? 4 : (NACC <= 4 ? 2 : 1));
+    constexpr int U = U0 > R ? U0 : R;
     constexpr int TILE = LPR * VEC * NACC;
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -232,11 +241,13 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
         off[k] = ok[k] ? e : 0;
     }
 
-    float acc[NACC][VEC];
+    float acc[R][NACC][VEC];
 #pragma unroll
-    for (int k = 0; k < NACC; ++k)
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[k][e] = 0.f;
+        for (int k = 0; k < NACC; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[r][k][e] = 0.f;
 
     const TIN *__restrict__ Hp = static_cast<const TIN *>(p.H);
 
@@ -270,44 +281,83 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
 #pragma unroll
                 for (int k = 0; k < NACC; ++k)
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) acc[k][e] = fmaf(v[u], h[u][k][e], acc[k][e]);
+                    for (int e = 0; e < VEC; ++e) acc[u % R][k][e] = fmaf(v[u], h[u][k][e], acc[u % R][k][e]);
         }
-        for (; i < n; i += G) {
-            const int src = i + g;
-            const int c = pick_i<G>(cl, src & (kWave - 1));
-            const float v = pick_f<G>(vl, src & (kWave - 1));
-            if (src < n) {
-                const TIN *row = Hp + (int64_t)c * p.ldh;
+        if constexpr (R == 1) {
+            for (; i < n; i += G) {
+                const int src = i + g;
+                const int c = pick_i<G>(cl, src & (kWave - 1));
+                const float v = pick_f<G>(vl, src & (kWave - 1));
+                if (src < n) {
+                    const TIN *row = Hp + (int64_t)c * p.ldh;
 #pragma unroll
-                for (int k = 0; k < NACC; ++k) {
-                    float h[VEC];
-                    VecIO<TIN, VEC>::load(row + off[k], h);
+                    for (int k = 0; k < NACC; ++k) {
+                        float h[VEC];
+                        VecIO<TIN, VEC>::load(row + off[k], h);
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) acc[k][e] = fmaf(v, h[e], acc[k][e]);
+                        for (int e = 0; e < VEC; ++e) acc[0][k][e] = fmaf(v, h[e], acc[0][k][e]);
+                    }
+                }
+            }
+        } else {
+            // fewer than G * U entries are left; i is a multiple of G * U, so step u continues chain u mod R
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int src = i + u * G + g;
+                const int c = pick_i<G>(cl, src & (kWave - 1));
+                const float v = pick_f<G>(vl, src & (kWave - 1));
+                if (src < n) {
+                    const TIN *row = Hp + (int64_t)c * p.ldh;
+#pragma unroll
+                    for (int k = 0; k < NACC; ++k) {
+                        float h[VEC];
+                        VecIO<TIN, VEC>::load(row + off[k], h);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[u % R][k][e] = fmaf(v, h[e], acc[u % R][k][e]);
+                    }
                 }
             }
         }
     }
 
-    // combine the G group sums: group g ^ 1, g ^ 2, ... (fixed order)
+    // combine the G group sums: group g ^ 1, g ^ 2, ... (fixed order), chain set by chain set
     if constexpr (G > 1) {
 #pragma unroll
-        for (int o = LPR; o < kWave; o <<= 1)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[0][e] += __shfl_xor(acc[0][e], o, kWave);
+            for (int o = LPR; o < kWave; o <<= 1)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[r][0][e] += __shfl_xor(acc[r][0][e], o, kWave);
     }
+    // then the chain sets, continuing the same pairwise order
+#pragma unroll
+    for (int s = 1; s < R; s <<= 1)
+#pragma unroll
+        for (int r = 0; r < R; r += 2 * s)
+#pragma unroll
+            for (int k = 0; k < NACC; ++k)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[r][k][e] += acc[r + s][k][e];
 
     if (g == 0) {
         if (to_ws) {
             float *dst = p.ws + out_row * p.ldws;
 #pragma unroll
             for (int k = 0; k < NACC; ++k)
-                if (ok[k]) store_f32<VEC>(dst + off[k], acc[k]);
+                if (ok[k]) store_f32<VEC>(dst + off[k], acc[0][k]);
         } else {
             TOUT *dst = static_cast<TOUT *>(p.Y) + out_row * p.ldy;
+            if (p.y_vec) {
 #pragma unroll
-            for (int k = 0; k < NACC; ++k)
-                if (ok[k]) VecIO<TOUT, VEC>::store(dst + off[k], acc[k]);
+                for (int k = 0; k < NACC; ++k)
+                    if (ok[k]) VecIO<TOUT, VEC>::store(dst + off[k], acc[0][k]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < NACC; ++k)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (ok[k] && off[k] + e < p.D) store_elem(dst + off[k] + e, acc[0][k][e]);
+            }
         }
     }
 }
@@ -491,14 +541,15 @@ struct plx_spmm_plan {
     int32_t *tables;  // device: long_rows[n_long] | seg_first[n_long+1] | seg_begin[n_seg] | seg_end[n_seg]
     const int32_t *long_rows, *seg_first, *seg_begin, *seg_end;
     std::vector<int32_t> h_long_rows, h_seg_first;  // host copies, to cut row ranges out of the plan
+    int slicing = 0;  // 0: column slices of H where the cost model says so, 1: whenever rows exceed a slice, -1: never
 };
 
 namespace {
 
-template <typename TIN, typename TOUT, int VEC, int LPR, int NACC>
+template <typename TIN, typename TOUT, int VEC, int LPR, int NACC, int R = 1>
 void launch_variant(const SpmmArgs &a, dim3 grid, hipStream_t st)
 {
-    spmm_csr_kernel<TIN, TOUT, VEC, LPR, NACC><<<grid, 256, 0, st>>>(a);
+    spmm_csr_kernel<TIN, TOUT, VEC, LPR, NACC, R><<<grid, 256, 0, st>>>(a);
 }
 
 template <typename TIN, typename TOUT, int VEC>
@@ -524,6 +575,55 @@ int launch_for_vec(const SpmmArgs &a, int lpr, int nacc, dim3 grid, hipStream_t 
     }
 }
 
+// the one-pass kernel summing in the order of the column-sliced product (kSliceChains chains): lpr 32 -> two lane
+// groups with two chains each, lpr 64 -> one group with four chains and at most two accumulator vectors
+template <typename TIN, typename TOUT, int VEC>
+int launch_chained(const SpmmArgs &a, int lpr, int nacc, dim3 grid, hipStream_t st)
+{
+    if (lpr == 32) { launch_variant<TIN, TOUT, VEC, 32, 1, 2>(a, grid, st); return 0; }
+    if (lpr == 64 && nacc == 1) { launch_variant<TIN, TOUT, VEC, 64, 1, 4>(a, grid, st); return 0; }
+    if (lpr == 64 && nacc == 2) { launch_variant<TIN, TOUT, VEC, 64, 2, 4>(a, grid, st); return 0; }
+    return -1;
+}
+
+// ---- column slices of H ----
+// A wide H is gathered in passes over slices of kSliceBytes per row when its rows, taken whole, overflow the last-level
+// cache while one slice of every row stays in it: on a 233 K-row graph with 492 entries per row, 602 fp32 columns take
+// 31.0 ms in one pass and 18.4 ms in ten passes over 64-column slices (a pass re-reads the index and value arrays, 8 of
+// the 264 bytes an entry then costs).  A slice is one quarter of a wavefront's 64 x 16 bytes, so a pass runs with four
+// lane groups; products that cannot be sliced in place (row ranges, operands that are not line-aligned and have no
+// room to be copied) use the one-pass kernel with the same four chains per sum, hence the same bits.
+constexpr int64_t kSliceBytes = 256;
+constexpr int kSliceChains = 4;
+
+bool sliced_plan(const plx_spmm_plan *plan, int64_t D, int64_t elem)
+{
+    const int64_t row_bytes = D * elem;
+    if (row_bytes <= kSliceBytes || plan->K <= 0 || plan->M <= 0 || plan->slicing < 0) return false;
+    if (plan->slicing > 0) return true;
+    if (plan->K * row_bytes <= (64ll << 20)) return false;     // whole rows stay cached as they are
+    if (plan->K * kSliceBytes > (128ll << 20)) return false;   // not even a slice of every row would
+    return plan->nnz >= 32 * plan->K && plan->nnz >= 32 * plan->M;  // every row of H is gathered often, rows of A are long
+}
+
+// Slices are read with 16-byte loads from line-aligned rows; a last slice that is not a multiple of 16 bytes wide is
+// read past its width, which is safe inside the padded rows of a staged copy but not inside a caller's tensor.
+bool sliceable_in_place(uintptr_t base, int64_t ldh, int64_t D, int64_t elem)
+{
+    return offset_granule(base, ldh * elem) == kLine && (D * elem) % 16 == 0;
+}
+
+// leading dimension (elements) of the staged copy of H that a whole-matrix product of this plan and width wants, or 0:
+// line-aligned rows either because column slices need them or because alignment alone repays the copy
+int64_t wanted_stage_ld(const plx_spmm_plan *plan, int64_t D, int64_t elem, uintptr_t base, int64_t ldh)
+{
+    if (sliced_plan(plan, D, elem)) {
+        if (sliceable_in_place(base, ldh, D, elem)) return 0;
+        return (D * elem + kLine - 1) / kLine * kLine / elem;
+    }
+    return staged_ld(plan->K, plan->nnz, D, elem, base, ldh);
+}
+
 // `may_stage` = false: the workspace holds the partial rows of the split rows and nothing else (H is gathered where
 // it lies; same values in the same order, so the same result)
 template <typename T>
@@ -538,26 +638,24 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
-    const size_t need = may_stage ? plx_spmm_workspace_bytes(plan, D) : (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+    const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+    const size_t need = may_stage ? plx_spmm_workspace_bytes(plan, D) : seg_bytes;
     if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return plx::fail(PLX_ERR_WORKSPACE, "spmm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     PLX_REQUIRE(need == 0 || (reinterpret_cast<uintptr_t>(workspace) % 16) == 0, "spmm: workspace not 16-byte aligned");
     hipStream_t st = plx::as_stream(stream);
 
     constexpr int kMaxVec = 16 / (int)sizeof(T);
-    auto widest = [&](const T *h, int64_t ld_h) {
-        int v = kMaxVec;
-        while (v > 1 && (D % v || ld_h % v || ldy % v || reinterpret_cast<uintptr_t>(h) % (v * sizeof(T)) ||
-                         reinterpret_cast<uintptr_t>(Y) % (v * sizeof(T))))
-            v >>= 1;
-        return v;
-    };
+    constexpr int64_t kElem = (int64_t)sizeof(T);
+    const bool whole = row_begin == 0 && row_end == plan->M;
+    const bool sliced = sliced_plan(plan, D, kElem);
+
     // Whole-matrix products stage H into line-aligned rows when that pays and the workspace has the room (the size
     // query reserves it for contiguous fp32 rows); the partial rows of split rows follow the staged copy.
-    const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
     char *ws_base = static_cast<char *>(workspace);
-    if (may_stage && row_begin == 0 && row_end == plan->M) {
-        const int64_t ld_st = staged_ld(plan->K, plan->nnz, D, (int64_t)sizeof(T), reinterpret_cast<uintptr_t>(H), ldh);
+    bool h_is_staged = false;  // H points at the copy: rows on 128-byte lines, padded to whole lines
+    if (may_stage && whole) {
+        const int64_t ld_st = wanted_stage_ld(plan, D, kElem, reinterpret_cast<uintptr_t>(H), ldh);
         const size_t st_bytes = (size_t)plan->K * (size_t)ld_st * sizeof(T);
         const size_t pad = ws_base ? (size_t)((kLine - reinterpret_cast<uintptr_t>(ws_base) % kLine) % kLine) : 0;
         if (ld_st > 0 && ws_base != nullptr && workspace_bytes >= pad + st_bytes + seg_bytes) {
@@ -576,32 +674,20 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
             PLX_LAUNCH_CHECK("stage_rows_kernel");
             H = staged;
             ldh = ld_st;
+            h_is_staged = true;
             ws_base += pad + st_bytes;  // a multiple of 128 bytes past an aligned address
         }
-    }
-    int vec = widest(H, ldh);
-    const int64_t units = D / vec;
-    int lpr = 4;
-    while (lpr < kWave && lpr < units) lpr <<= 1;
-    int nacc = 1, tiles = 1;
-    if (lpr == kWave) {
-        const int64_t chunks = plx::ceil_div(units, kWave);
-        tiles = (int)plx::ceil_div(chunks, 8);
-        nacc = (int)plx::ceil_div(chunks, tiles);
     }
 
     SpmmArgs a;
     a.rowptr = plan->rowptr;
     a.col = plan->col;
     a.val = val;
-    a.H = H;
-    a.Y = Y;
     a.ws = reinterpret_cast<float *>(ws_base);
     a.seg_begin = plan->seg_begin;
     a.seg_end = plan->seg_end;
     a.ldh = ldh;
     a.ldy = ldy;
-    a.ldws = ws_ld(D);
     // split rows inside the range, and their segments
     const auto lr_begin = plan->h_long_rows.begin(), lr_end = plan->h_long_rows.end();
     const int64_t q0 = std::lower_bound(lr_begin, lr_end, (int32_t)row_begin) - lr_begin;
@@ -610,33 +696,90 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     const int64_t s1 = q1 > q0 ? plan->h_seg_first[(size_t)q1] : 0;
     a.M = (int32_t)plan->M;
     a.n_seg = (int32_t)(s1 - s0);
-    a.D = (int32_t)D;
     a.seg_len = plan->seg_len;
     a.row_begin = (int32_t)row_begin;
     a.row_end = (int32_t)row_end;
     a.seg_base = (int32_t)s0;
-
     const int64_t tasks = (row_end - row_begin) + (s1 - s0);
+    auto reduce_split_rows = [&](T *y, int64_t d) -> int {
+        if (q1 > q0) {
+            dim3 rgrid((unsigned)(q1 - q0), (unsigned)plx::ceil_div(d, 64), 1);
+            spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)d, y, ldy);
+            PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
+        }
+        return PLX_OK;
+    };
+
+    // ---- passes over column slices: whole matrix, rows of H (as they lie or as staged) on 128-byte lines ----
+    if (sliced && whole && (h_is_staged || sliceable_in_place(reinterpret_cast<uintptr_t>(H), ldh, D, kElem))) {
+        static_assert(kWave / 16 == kSliceChains, "a slice is covered by 16 lanes, so a pass sums in kSliceChains lane groups");
+        constexpr int64_t kW = kSliceBytes / kElem;  // columns per slice; 16 lanes x 16 bytes cover one
+        const bool y_vec = reinterpret_cast<uintptr_t>(Y) % 16 == 0 && (ldy * kElem) % 16 == 0;
+        a.ldws = ws_ld(kW);
+        dim3 grid((unsigned)plx::ceil_div(tasks, 4), 1, 1);
+        for (int64_t c0 = 0; c0 < D; c0 += kW) {
+            const int64_t w = std::min<int64_t>(kW, D - c0);
+            a.H = H + c0;
+            a.Y = Y + c0;
+            a.D = (int32_t)w;
+            a.y_vec = (y_vec && w % kMaxVec == 0) ? 1 : 0;  // a ragged last slice loads past its width (inside the padded row) and stores by element
+            launch_variant<T, T, kMaxVec, 16, 1>(a, grid, st);
+            PLX_LAUNCH_CHECK("spmm_csr_kernel (column slice)");
+            const int rc = reduce_split_rows(Y + c0, w);
+            if (rc != PLX_OK) return rc;
+        }
+        return PLX_OK;
+    }
+
+    auto widest = [&](const T *h, int64_t ld_h) {
+        int v = kMaxVec;
+        while (v > 1 && (D % v || ld_h % v || ldy % v || reinterpret_cast<uintptr_t>(h) % (v * sizeof(T)) ||
+                         reinterpret_cast<uintptr_t>(Y) % (v * sizeof(T))))
+            v >>= 1;
+        return v;
+    };
+    int vec = widest(H, ldh);
+    const int64_t units = D / vec;
+    int lpr = 4;
+    while (lpr < kWave && lpr < units) lpr <<= 1;
+    int nacc = 1, tiles = 1;
+    if (lpr == kWave) {
+        const int64_t chunks = plx::ceil_div(units, kWave);
+        tiles = (int)plx::ceil_div(chunks, sliced ? 2 : 8);  // the chained kernel keeps four sums per accumulator vector
+        nacc = (int)plx::ceil_div(chunks, tiles);
+    }
+    a.H = H;
+    a.Y = Y;
+    a.ldws = ws_ld(D);
+    a.D = (int32_t)D;
+    a.y_vec = 1;
+
     dim3 grid((unsigned)plx::ceil_div(tasks, 4), (unsigned)tiles, 1);
     int rc = -1;
-    switch (vec) {
-        case 1: rc = launch_for_vec<T, T, 1>(a, lpr, nacc, grid, st); break;
-        case 2: rc = launch_for_vec<T, T, 2>(a, lpr, nacc, grid, st); break;
-        case 4: rc = launch_for_vec<T, T, 4>(a, lpr, nacc, grid, st); break;
-        case 8:
-            if constexpr (kMaxVec == 8) rc = launch_for_vec<T, T, 8>(a, lpr, nacc, grid, st);
-            break;
-        default: break;
+    if (sliced) {  // one pass, summed in the order of the sliced product
+        switch (vec) {
+            case 1: rc = launch_chained<T, T, 1>(a, lpr, nacc, grid, st); break;
+            case 2: rc = launch_chained<T, T, 2>(a, lpr, nacc, grid, st); break;
+            case 4: rc = launch_chained<T, T, 4>(a, lpr, nacc, grid, st); break;
+            case 8:
+                if constexpr (kMaxVec == 8) rc = launch_chained<T, T, 8>(a, lpr, nacc, grid, st);
+                break;
+            default: break;
+        }
+    } else {
+        switch (vec) {
+            case 1: rc = launch_for_vec<T, T, 1>(a, lpr, nacc, grid, st); break;
+            case 2: rc = launch_for_vec<T, T, 2>(a, lpr, nacc, grid, st); break;
+            case 4: rc = launch_for_vec<T, T, 4>(a, lpr, nacc, grid, st); break;
+            case 8:
+                if constexpr (kMaxVec == 8) rc = launch_for_vec<T, T, 8>(a, lpr, nacc, grid, st);
+                break;
+            default: break;
+        }
     }
-    if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "spmm: no kernel for vec=%d lpr=%d nacc=%d", vec, lpr, nacc);
+    if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "spmm: no kernel for vec=%d lpr=%d nacc=%d%s", vec, lpr, nacc, sliced ? " (chained)" : "");
     PLX_LAUNCH_CHECK("spmm_csr_kernel");
-
-    if (q1 > q0) {
-        dim3 rgrid((unsigned)(q1 - q0), (unsigned)plx::ceil_div(D, 64), 1);
-        spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)D, Y, ldy);
-        PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
-    }
-    return PLX_OK;
+    return reduce_split_rows(Y, D);
 }
 
 // ---- the product without a caller's workspace: partial rows of the split rows in a static device array ----
@@ -835,9 +978,17 @@ size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)
     const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
     // room for the line-aligned copy of H, decided for contiguous fp32 rows (an operand laid out otherwise is staged
     // only if it fits what the caller brought)
-    const int64_t ld_st = staged_ld(plan->K, plan->nnz, D, 4, 0, D);
+    const int64_t ld_st = wanted_stage_ld(plan, D, 4, 0, D);
     if (ld_st == 0) return seg_bytes;
     return (size_t)kLine + (size_t)plan->K * (size_t)ld_st * sizeof(float) + seg_bytes;
+}
+
+int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_set_slicing: plan is NULL");
+    PLX_REQUIRE(mode >= -1 && mode <= 1, "plan_set_slicing: mode must be -1, 0 or 1");
+    plan->slicing = mode;
+    return PLX_OK;
 }
 
 int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,

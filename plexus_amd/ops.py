@@ -122,6 +122,12 @@ class CsrMatrix:
     def size(self, dim: int) -> int:
         return self.shape[dim]
 
+    def set_slicing(self, mode: int) -> None:
+        """Column slicing of H in the products of this matrix: 0 = where the library's rule says so (the default),
+        1 = whenever a row of H exceeds 256 bytes, -1 = never.  The result of a product does not depend on how it was
+        sliced, only on the mode."""
+        check(_lib.load().plx_spmm_plan_set_slicing(self._plan, int(mode)), "plx_spmm_plan_set_slicing")
+
     def _workspace(self, d: int):
         need = int(_lib.load().plx_spmm_workspace_bytes(self._plan, d))
         if need == 0:

@@ -1042,6 +1042,55 @@ def test_spmm_from_a_line_aligned_copy_of_h_gives_the_same_bits():
         assert torch.equal(ops.spmm(a, hp[:, :d]), y)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_spmm_in_column_slices_agrees_bit_for_bit_with_its_one_pass_form(dtype):
+    """Products of a sliced shape: passes over 256-byte column slices of H (in place when its rows lie on 128-byte lines,
+    else from a staged copy), and the one-pass kernel that sums in the same order (row ranges, operands that can be
+    neither sliced in place nor copied).  All of them must give the same bits, and the oracle's numbers."""
+    say("spmm in column slices, %s" % dtype)
+    from plexus_amd import _lib
+
+    lib = _lib.load()
+    g = S.build_graph(3000, "chunglu", 40000, seed=5, device="cpu", gamma=2.1)
+    tol = FP32_TOL if dtype == torch.float32 else 2.0 ** -8
+    per16 = 4 if dtype == torch.float32 else 8
+    widths = [128, 602, 130, 72, 256, 1433] if dtype == torch.float32 else [256, 200, 136, 602]
+    for seg_len in (64, 1024):
+        a = to_dev(g, seg_len=seg_len)
+        plain = to_dev(g, seg_len=seg_len)
+        plain.set_slicing(-1)
+        a.set_slicing(1)
+        assert a.n_long_rows > 0
+        for d in widths:
+            h_host = torch.randn(3000, d, generator=torch.Generator().manual_seed(d)).to(dtype)
+            h = h_host.to(DEV)
+            y = ops.spmm(a, h)  # whole matrix: sliced in place (rows on lines, whole 16-byte units) or from a copy
+            assert rel_err(y.float().cpu(), oracle_spmm64(g, h_host.float())) <= tol
+            # row ranges never slice: one pass with the same four chains per sum
+            assert torch.equal(ops.chunked_spmm(a, h, max_rows_per_chunk=700), y), (d, seg_len)
+            # an operand off the lines and no room to copy it (the entry point without a workspace): one pass again
+            if dtype == torch.float32 and a.n_segments * ((d + 3) // 4) * 16 <= (32 << 20):
+                y2 = torch.full((3000, d), float("nan"), device=DEV)
+                flat = torch.zeros(3000 * d + 1, device=DEV)
+                h_off = flat[1:].view(3000, d)
+                h_off.copy_(h)
+                _lib.check(lib.plx_spmm_csr_f32_static(a._plan, a.val.data_ptr(), h_off.data_ptr(), d, d, y2.data_ptr(), d,
+                                                       torch.cuda.current_stream().cuda_stream), "plx_spmm_csr_f32_static")
+                assert torch.equal(y2, y), (d, seg_len)
+            # H and Y as column slabs of wider matrices; Y rows off 16-byte boundaries
+            wide_h = torch.zeros(3000, d + 32 * per16, device=DEV, dtype=dtype)
+            wide_h[:, 32 * per16 // 2: 32 * per16 // 2 + d] = h
+            wide_y = torch.zeros(3000, d + 3, device=DEV, dtype=dtype)
+            ops.spmm(a, wide_h[:, 32 * per16 // 2: 32 * per16 // 2 + d], out=wide_y[:, 1:1 + d])
+            assert torch.equal(wide_y[:, 1:1 + d], y) and (wide_y[:, 0] == 0).all() and (wide_y[:, 1 + d:] == 0).all(), (d, seg_len)
+            # the unsliced product differs in summation order only
+            assert rel_err(ops.spmm(plain, h).float(), y.float()) <= (1e-6 if dtype == torch.float32 else 2.0 ** -7)
+    # the rule itself: this small matrix is not sliced unless told to, the 233 K-row benchmark matrix would be
+    auto = to_dev(g)
+    h = torch.randn(3000, 602, generator=torch.Generator().manual_seed(1)).to(DEV)
+    assert torch.equal(ops.spmm(auto, h), ops.spmm(plain, h))
+
+
 def test_spmm_staging_with_bf16_rows_and_dense_reuse():
     say("spmm: staging of bf16 rows and of 2,408-byte fp32 rows under heavy reuse")
     g = S.build_graph(2000, "uniform", 0, seed=11, device="cpu", exact_pairs=100000)  # about 100 entries per column of H
