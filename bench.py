@@ -343,15 +343,22 @@ def main():
     stats = g.degree_stats()
     torch.cuda.synchronize()
     gen_s = time.time() - t0
-    # preparation, timed apart from the hot path: int64 -> int32 indices + row plan, and the device-side transpose
-    t_prep = time.time()
-    a = ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape, args.seg_len)
-    torch.cuda.synchronize()
-    prep_plan_ms = (time.time() - t_prep) * 1e3
-    t_prep = time.time()
-    at = ops.csr_transpose(a, args.seg_len)
-    torch.cuda.synchronize()
-    prep_transpose_ms = (time.time() - t_prep) * 1e3
+    # preparation, timed apart from the hot path: int64 -> int32 indices + row plan, and the device-side transpose.
+    # Each is run twice and the second run is reported: the first call into the library also loads its code object
+    # and makes the allocator fetch fresh memory (about 25 ms each, once per process; kept as *_first_call).
+    def timed_twice(fn):
+        out, ms = None, []
+        for _ in range(2):
+            del out
+            torch.cuda.synchronize()
+            t_prep = time.time()
+            out = fn()
+            torch.cuda.synchronize()
+            ms.append((time.time() - t_prep) * 1e3)
+        return out, ms[1], ms[0]
+
+    a, prep_plan_ms, prep_plan_first_ms = timed_twice(lambda: ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape, args.seg_len))
+    at, prep_transpose_ms, prep_transpose_first_ms = timed_twice(lambda: ops.csr_transpose(a, args.seg_len))
     assert torch.equal(at.col, g.col_t.to(torch.int32)) and torch.equal(at.val, g.val_t)  # same as the generator's own transpose
     nnz = g.nnz
     bf16 = args.config == 5
@@ -554,6 +561,7 @@ def main():
         "random_gather_ceiling": gather_ceiling,
         "spmm_D%d" % d_side: spmm[d_side],
         "prep_ms": {"narrow_indices_and_plan": prep_plan_ms, "device_transpose_and_plan": prep_transpose_ms,
+                    "narrow_indices_and_plan_first_call": prep_plan_first_ms, "device_transpose_and_plan_first_call": prep_transpose_first_ms,
                     "gcn_norm_from_edge_list": prep_norm_ms, "double_permutation": prep_perm_ms},
         "epoch_ms": epoch_ms,
         "epoch_ms_transform_first_option": epoch_ms_tf,

@@ -103,8 +103,9 @@ int plx_spmm_segments_host(int64_t M, const int32_t *rowptr_host, int32_t seg_le
  * ---------------------------------------------------------------------------------------- */
 typedef struct plx_spmm_plan plx_spmm_plan;
 
-/* Reads rowptr (M+1 int32 on the device; synchronises `stream`), bins the rows and keeps the
- * segment tables on the device.  Checks once that rowptr runs from 0 to nnz without decreasing and that
+/* Reads rowptr and col on the device (synchronises `stream`; two counters and the two short tables that row-range
+ * products need cross to the host, nothing else), finds the rows to split and keeps their segment tables on the
+ * device.  Checks once that rowptr runs from 0 to nnz without decreasing and that
  * every column index lies in [0, K) (PLX_ERR_INVALID otherwise): the SpMM itself trusts them.
  * rowptr/col are BORROWED: they must outlive the plan and keep their contents.
  * seg_len <= 0 selects the default (1024, or 4096 when rows hold 128 entries or more on average). */
@@ -113,6 +114,10 @@ int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
 /* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len */
 int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
+/* Copies the plan's tables to host arrays (any of them may be NULL): long rows [long rows], seg_first [long rows + 1],
+ * seg_begin / seg_end [segments] -- the layout of plx_spmm_segments_host.  For inspection and tests; synchronous. */
+int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host, int32_t *seg_first_host, int32_t *seg_begin_host,
+                              int32_t *seg_end_host);
 /* Column slicing of H.  When the rows of H taken whole overflow the last-level cache while a 256-byte slice of every row
  * stays in it, and every row is gathered often, whole-matrix products run as passes over 256-byte column slices
  * (233 K rows, 492 entries per row, 602 fp32 columns: 31.0 -> 18.4 ms).  The choice depends on the plan, the width and

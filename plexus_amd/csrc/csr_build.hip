@@ -27,12 +27,6 @@ int bits_for(int64_t n)
     return b;
 }
 
-__global__ void iota_kernel(int64_t n, int32_t *__restrict__ out)
-{
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (int32_t)i;
-}
-
 // a fill kernel rather than a memset node: these calls are stream-ordered and may be recorded into a graph
 __global__ void zero_i32_kernel(int64_t n, int32_t *__restrict__ out)
 {
@@ -53,21 +47,45 @@ __global__ void rowptr_from_sorted_kernel(int64_t n, const KeyT *__restrict__ so
     }
 }
 
-// transposed entry i comes from entry j = perm[i] of the source: its column is the source row of j
-__global__ void transpose_gather_kernel(int64_t nnz, int64_t M, const int32_t *__restrict__ rowptr, const int32_t *__restrict__ perm,
-                                        const float *__restrict__ val, int32_t *__restrict__ col_t, float *__restrict__ val_t)
+// (row, value) of every stored entry as one 64-bit word, row in the upper half: the payload that travels through the
+// sort by column.  A workgroup takes 1,024 consecutive entries; it finds the rows of its first and last entry by
+// binary search once, and each entry then searches only between those (no steps at all inside a long row).
+constexpr int kPackPerBlock = 1024;
+__global__ void __launch_bounds__(256) pack_row_value_kernel(int64_t nnz, int64_t M, const int32_t *__restrict__ rowptr,
+                                                             const float *__restrict__ val, uint64_t *__restrict__ packed)
 {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nnz; i += stride) {
-        const int32_t j = perm[i];
-        // row of entry j: the last r with rowptr[r] <= j
+    __shared__ int32_t bounds[2];
+    const int64_t e0 = (int64_t)blockIdx.x * kPackPerBlock;
+    const int64_t e1 = min(e0 + kPackPerBlock, nnz) - 1;
+    if (threadIdx.x < 2) {
+        const int64_t j = threadIdx.x == 0 ? e0 : e1;
         int64_t lo = 0, hi = M;  // invariant: rowptr[lo] <= j < rowptr[hi]
         while (hi - lo > 1) {
             const int64_t mid = (lo + hi) >> 1;
             if (rowptr[mid] <= j) lo = mid; else hi = mid;
         }
-        col_t[i] = (int32_t)lo;
-        val_t[i] = val[j];
+        bounds[threadIdx.x] = (int32_t)lo;
+    }
+    __syncthreads();
+    const int32_t r_first = bounds[0], r_last = bounds[1];
+    for (int64_t j = e0 + threadIdx.x; j <= e1; j += 256) {
+        int32_t lo = r_first, hi = r_last + 1;  // the row of j is the last r in [r_first, r_last] with rowptr[r] <= j
+        while (hi - lo > 1) {
+            const int32_t mid = lo + ((hi - lo) >> 1);
+            if (rowptr[mid] <= j) lo = mid; else hi = mid;
+        }
+        packed[j] = ((uint64_t)(uint32_t)lo << 32) | (uint64_t)__float_as_uint(val[j]);
+    }
+}
+
+// transposed entry i: its column is the source row, its value the source value
+__global__ void unpack_row_value_kernel(int64_t nnz, const uint64_t *__restrict__ packed, int32_t *__restrict__ col_t, float *__restrict__ val_t)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const uint64_t w = packed[i];
+        col_t[i] = (int32_t)(w >> 32);
+        val_t[i] = __uint_as_float((uint32_t)w);
     }
 }
 
@@ -104,19 +122,19 @@ struct RowOfBlockKey {
 unsigned blocks_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>(plx::ceil_div(n, 256), 256 * 32)); }
 
 struct TransposeLayout {
-    size_t keys_out, idx_in, idx_out, temp, temp_bytes, total;
+    size_t keys_out, pay_in, pay_out, temp, temp_bytes, total;
 };
 
 int transpose_layout(int64_t K, int64_t nnz, TransposeLayout &l)
 {
     size_t temp = 0;
-    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const int32_t *)nullptr, (int32_t *)nullptr, (const int32_t *)nullptr,
-                                             (int32_t *)nullptr, (size_t)nnz, 0, (unsigned)bits_for(K), (hipStream_t)0);
+    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp, (const int32_t *)nullptr, (int32_t *)nullptr, (const uint64_t *)nullptr,
+                                             (uint64_t *)nullptr, (size_t)nnz, 0, (unsigned)bits_for(K), (hipStream_t)0);
     if (e != hipSuccess) return plx::fail(PLX_ERR_HIP, "csr_transpose: radix sort size query failed: %s", hipGetErrorString(e));
     size_t off = 0;
     l.keys_out = off; off += align_up(sizeof(int32_t) * (size_t)nnz);
-    l.idx_in = off;   off += align_up(sizeof(int32_t) * (size_t)nnz);
-    l.idx_out = off;  off += align_up(sizeof(int32_t) * (size_t)nnz);
+    l.pay_in = off;   off += align_up(sizeof(uint64_t) * (size_t)nnz);
+    l.pay_out = off;  off += align_up(sizeof(uint64_t) * (size_t)nnz);
     l.temp = off;     off += align_up(temp);
     l.temp_bytes = temp;
     l.total = off;
@@ -190,18 +208,19 @@ int plx_csr_transpose_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *rowp
     PLX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 256 == 0, "csr_transpose: workspace must be 256-byte aligned");
     char *ws = static_cast<char *>(workspace);
     int32_t *keys_out = reinterpret_cast<int32_t *>(ws + l.keys_out);
-    int32_t *idx_in = reinterpret_cast<int32_t *>(ws + l.idx_in);
-    int32_t *idx_out = reinterpret_cast<int32_t *>(ws + l.idx_out);
+    uint64_t *pay_in = reinterpret_cast<uint64_t *>(ws + l.pay_in);
+    uint64_t *pay_out = reinterpret_cast<uint64_t *>(ws + l.pay_out);
 
-    iota_kernel<<<blocks_for(nnz), 256, 0, st>>>(nnz, idx_in);
-    PLX_LAUNCH_CHECK("iota_kernel");
-    // stable sort by column: within a column the entries keep their source order, i.e. ascending source row
+    pack_row_value_kernel<<<(unsigned)plx::ceil_div(nnz, kPackPerBlock), 256, 0, st>>>(nnz, M, rowptr, val, pay_in);
+    PLX_LAUNCH_CHECK("pack_row_value_kernel");
+    // stable sort by column: within a column the entries keep their source order, i.e. ascending source row; the
+    // (row, value) words travel with the keys, so nothing is gathered afterwards
     size_t temp = l.temp_bytes;
-    PLX_HIP_CHECK(rocprim::radix_sort_pairs(ws + l.temp, temp, col, keys_out, idx_in, idx_out, (size_t)nnz, 0, (unsigned)bits_for(K), st));
+    PLX_HIP_CHECK(rocprim::radix_sort_pairs(ws + l.temp, temp, col, keys_out, pay_in, pay_out, (size_t)nnz, 0, (unsigned)bits_for(K), st));
     rowptr_from_sorted_kernel<int32_t><<<blocks_for(nnz + 1), 256, 0, st>>>(nnz, keys_out, K, rowptr_t, RowOfColumnKey());
     PLX_LAUNCH_CHECK("rowptr_from_sorted_kernel");
-    transpose_gather_kernel<<<blocks_for(nnz), 256, 0, st>>>(nnz, M, rowptr, idx_out, val, col_t, val_t);
-    PLX_LAUNCH_CHECK("transpose_gather_kernel");
+    unpack_row_value_kernel<<<blocks_for(nnz), 256, 0, st>>>(nnz, pay_out, col_t, val_t);
+    PLX_LAUNCH_CHECK("unpack_row_value_kernel");
     return PLX_OK;
 }
 

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "common.h"
+#include "plan_build.h"
 
 // Scratch of plx_spmm_csr_f32_static: fp32 partial rows of the split rows.  Every GPU the library runs on holds its own
 // copy of this array, at its own address, until the process ends.
@@ -418,17 +419,6 @@ __global__ void narrow_i64_kernel(int64_t n, const int64_t *__restrict__ src, in
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) dst[i] = (int32_t)src[i];
-}
-
-// Counts the column indices outside [0, K): the gather of the SpMM trusts them.
-__global__ void __launch_bounds__(256) count_bad_columns_kernel(int64_t nnz, const int32_t *__restrict__ col, int32_t K,
-                                                                unsigned int *__restrict__ n_bad)
-{
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    unsigned int bad = 0;
-    for (; i < nnz; i += stride) bad += (unsigned int)col[i] >= (unsigned int)K ? 1u : 0u;
-    if (bad) atomicAdd(n_bad, bad);
 }
 
 // Diagnostic: what the memory system gives to the access pattern of the SpMM when nothing else is in the
@@ -880,71 +870,33 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
     if (seg_len <= 0) seg_len = (M > 0 && nnz / M >= 128) ? 4096 : 1024;
     hipStream_t st = plx::as_stream(stream);
 
-    std::vector<int32_t> rp((size_t)M + 1);
-    PLX_HIP_CHECK(hipMemcpyAsync(rp.data(), rowptr, sizeof(int32_t) * (size_t)(M + 1), hipMemcpyDeviceToHost, st));
-    PLX_HIP_CHECK(hipStreamSynchronize(st));
-    PLX_REQUIRE(rp[0] == 0 && rp[(size_t)M] == nnz, "plan_create: rowptr[0]=%d rowptr[M]=%d but nnz=%lld", rp[0],
-                rp[(size_t)M], (long long)nnz);
-
-    int64_t nl = 0, ns = 0;
-    int rc = plx_spmm_segments_host(M, rp.data(), seg_len, &nl, &ns, nullptr, nullptr, 0, nullptr, nullptr, 0);
+    // validation and the tables of the split rows, on the device
+    plx::PlanTables t;
+    const int rc = plx::build_plan_tables(M, K, nnz, rowptr, col, seg_len, st, t);
     if (rc != PLX_OK) return rc;
 
-    if (nnz > 0) {  // every column index must name a row of H: one streaming pass, once per matrix
-        unsigned int *d_bad = nullptr, h_bad = 0;
-        PLX_HIP_CHECK(hipMalloc(reinterpret_cast<void **>(&d_bad), sizeof(unsigned int)));
-        hipError_t e = hipMemsetAsync(d_bad, 0, sizeof(unsigned int), st);
-        if (e == hipSuccess) {
-            const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(nnz, 256 * 8), 8192);
-            count_bad_columns_kernel<<<blocks, 256, 0, st>>>(nnz, col, (int32_t)K, d_bad);
-            e = hipGetLastError();
-        }
-        if (e == hipSuccess) e = hipMemcpyAsync(&h_bad, d_bad, sizeof(unsigned int), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess) e = hipStreamSynchronize(st);
-        (void)hipFree(d_bad);
-        if (e != hipSuccess) return plx::fail(PLX_ERR_HIP, "plan_create: column check failed: %s", hipGetErrorString(e));
-        PLX_REQUIRE(h_bad == 0, "plan_create: %u column indices lie outside [0, %lld)", h_bad, (long long)K);
-    }
-
     plx_spmm_plan *p = new (std::nothrow) plx_spmm_plan();
-    if (!p) return plx::fail(PLX_ERR_NOMEM, "plan_create: host allocation failed");
+    if (!p) {
+        if (t.tables) (void)hipFree(t.tables);
+        return plx::fail(PLX_ERR_NOMEM, "plan_create: host allocation failed");
+    }
     p->M = M;
     p->K = K;
     p->nnz = nnz;
     p->rowptr = rowptr;
     p->col = col;
     p->seg_len = seg_len;
-    p->n_long = nl;
-    p->n_seg = ns;
-    p->tables = nullptr;
+    p->n_long = t.n_long;
+    p->n_seg = t.n_seg;
+    p->tables = t.tables;
     p->long_rows = p->seg_first = p->seg_begin = p->seg_end = nullptr;
-    if (nl > 0) {
-        const size_t total = (size_t)nl + (size_t)(nl + 1) + 2 * (size_t)ns;
-        std::vector<int32_t> host(total);
-        int32_t *lr = host.data(), *sf = lr + nl, *sb = sf + nl + 1, *se = sb + ns;
-        rc = plx_spmm_segments_host(M, rp.data(), seg_len, &nl, &ns, lr, sf, nl, sb, se, ns);
-        if (rc != PLX_OK) {
-            delete p;
-            return rc;
-        }
-        hipError_t e = hipMalloc(reinterpret_cast<void **>(&p->tables), total * sizeof(int32_t));
-        if (e != hipSuccess) {
-            delete p;
-            return plx::fail(PLX_ERR_NOMEM, "plan_create: hipMalloc of %zu bytes failed: %s", total * sizeof(int32_t),
-                             hipGetErrorString(e));
-        }
-        e = hipMemcpy(p->tables, host.data(), total * sizeof(int32_t), hipMemcpyHostToDevice);
-        if (e != hipSuccess) {
-            (void)hipFree(p->tables);
-            delete p;
-            return plx::fail(PLX_ERR_HIP, "plan_create: table upload failed: %s", hipGetErrorString(e));
-        }
-        p->h_long_rows.assign(lr, lr + nl);
-        p->h_seg_first.assign(sf, sf + nl + 1);
+    if (t.n_long > 0) {
+        p->h_long_rows = std::move(t.h_long_rows);
+        p->h_seg_first = std::move(t.h_seg_first);
         p->long_rows = p->tables;
-        p->seg_first = p->tables + nl;
-        p->seg_begin = p->seg_first + nl + 1;
-        p->seg_end = p->seg_begin + ns;
+        p->seg_first = p->tables + t.n_long;
+        p->seg_begin = p->seg_first + t.n_long + 1;
+        p->seg_end = p->seg_begin + t.n_seg;
     }
     *out = p;
     return PLX_OK;
@@ -970,6 +922,22 @@ int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what)
         case 5: return plan->seg_len;
         default: return -1;
     }
+}
+
+int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host, int32_t *seg_first_host, int32_t *seg_begin_host,
+                              int32_t *seg_end_host)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_tables_host: plan is NULL");
+    if (plan->n_long == 0) {
+        if (seg_first_host) seg_first_host[0] = 0;
+        return PLX_OK;
+    }
+    const size_t nl = (size_t)plan->n_long, ns = (size_t)plan->n_seg;
+    if (long_rows_host) PLX_HIP_CHECK(hipMemcpy(long_rows_host, plan->long_rows, nl * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (seg_first_host) PLX_HIP_CHECK(hipMemcpy(seg_first_host, plan->seg_first, (nl + 1) * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (seg_begin_host) PLX_HIP_CHECK(hipMemcpy(seg_begin_host, plan->seg_begin, ns * sizeof(int32_t), hipMemcpyDeviceToHost));
+    if (seg_end_host) PLX_HIP_CHECK(hipMemcpy(seg_end_host, plan->seg_end, ns * sizeof(int32_t), hipMemcpyDeviceToHost));
+    return PLX_OK;
 }
 
 size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)

@@ -118,6 +118,36 @@ def test_spmm_plan_rejects_malformed_matrices():
     assert ops.spmm(a, torch.eye(4, device=DEV)).sum().item() == 5.0
 
 
+def test_device_built_plan_tables_equal_the_host_construction():
+    """The tables of the split rows are built on the device (compaction, prefix sum, one workgroup per split row); they
+    must be exactly what the host routine makes of the same row pointers."""
+    say("spmm plan tables: device against host")
+    import ctypes as C
+
+    from plexus_amd import _lib
+
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(0)
+    for m, seg_len in ((5000, 7), (5000, 64), (1, 3), (300, 1), (70000, 16)):
+        lens = torch.randint(0, 40, (m,), generator=gen)
+        lens[torch.randint(0, m, (max(1, m // 50),), generator=gen)] = torch.randint(40, 3000, (max(1, m // 50),), generator=gen)
+        rowptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(lens, 0)]).to(torch.int32)
+        nnz = int(rowptr[-1])
+        col = torch.zeros(nnz, dtype=torch.int32)
+        a = ops.CsrMatrix(rowptr.to(DEV), col.to(DEV), torch.ones(nnz).to(DEV), (m, 4), seg_len)
+        rp = rowptr.numpy()
+        nl, ns = C.c_int64(), C.c_int64()
+        assert lib.plx_spmm_segments_host(m, rp.ctypes.data, seg_len, C.byref(nl), C.byref(ns), None, None, 0, None, None, 0) == 0
+        assert (a.n_long_rows, a.n_segments) == (nl.value, ns.value) and nl.value > 0
+        want = [np.zeros(nl.value, np.int32), np.zeros(nl.value + 1, np.int32), np.zeros(ns.value, np.int32), np.zeros(ns.value, np.int32)]
+        assert lib.plx_spmm_segments_host(m, rp.ctypes.data, seg_len, C.byref(nl), C.byref(ns), want[0].ctypes.data, want[1].ctypes.data,
+                                          nl.value, want[2].ctypes.data, want[3].ctypes.data, ns.value) == 0
+        got = [np.full_like(w, -1) for w in want]
+        _lib.check(lib.plx_spmm_plan_tables_host(a._plan, *[x.ctypes.data for x in got]), "plx_spmm_plan_tables_host")
+        for name, x, w in zip(("long_rows", "seg_first", "seg_begin", "seg_end"), got, want):
+            assert np.array_equal(x, w), (name, m, seg_len)
+
+
 def test_spmm_and_transpose_just_below_the_int32_limit():
     """Maximum size: 2,145,386,496 stored entries (the entry points take fewer than 2^31 - 64), every row split into two
     segments.  The product is checked against fp64 arithmetic by torch in row blocks, the transpose by the adjoint
