@@ -25,10 +25,30 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 FP32_VECTOR_TFLOPS = 157.3
-# Bytes moved between L2 and the memory side per SpMM launch at D = 128 on the full-size workload, from
-# rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain
-# 1 GiB copy: 2.000 and 1.000); the summary is profiles/spmm_csr_config3_fp32_pmc.txt.
-MEASURED_SPMM_TRAFFIC_BYTES = {(2449029, 126149029, 128): 53.9e9}
+# Bytes moved between L2 and the memory side per SpMM launch, from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each
+# scaled by what the same counter reads for a plain 1 GiB copy).  The figures are not kept here: they are read from the
+# trailer of the counter summary under profiles/, which also names the commit it was taken at, and both are reported
+# in the JSON line (roofline.traffic, roofline.traffic_source).
+SPMM_TRAFFIC_PROFILE = os.path.join("profiles", "spmm_csr_config3_fp32_pmc.txt")
+
+
+def measured_spmm_traffic(n, nnz, d):
+    """(bytes per launch or None, where the figure comes from) for the SpMM of an n-row, nnz-entry graph at width d."""
+    import re
+
+    path = os.path.join(ROOT, SPMM_TRAFFIC_PROFILE)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    commit = re.search(r"^\s*taken_at_commit\s*=\s*(\S+)", text, flags=re.M)
+    kernel = re.search(r"^\s*kernel\s*=\s*(.+)$", text, flags=re.M)
+    m = re.search(r"^\s*traffic_bytes_per_launch\[%d,%d,%d\]\s*=\s*([0-9.eE+]+)" % (n, nnz, d), text, flags=re.M)
+    if not m:
+        return None, None
+    source = {"profile": SPMM_TRAFFIC_PROFILE, "commit": commit.group(1) if commit else None,
+              "kernel": kernel.group(1).strip() if kernel else None}
+    return float(m.group(1)), source
 
 
 def spmm_bytes(m, k, nnz, d, elem=4):
@@ -568,7 +588,8 @@ def main():
         "loss_first_last": [losses[0], losses[-1]] if losses else None,
         "roofline": {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": dom["alg_GBps"] / HBM_PEAK_GBPS,
-                     "traffic": None if bf16 else MEASURED_SPMM_TRAFFIC_BYTES.get((n, nnz, 128)),
+                     "traffic": None if bf16 else measured_spmm_traffic(n, nnz, d_main)[0],
+                     "traffic_source": None if bf16 else measured_spmm_traffic(n, nnz, d_main)[1],
                      "kernel": "spmm_csr_kernel (A.H, D=%d, %s)" % (d_main, "bf16" if bf16 else "fp32"),
                      "alg_bytes_per_launch": dom["alg_bytes"],
                      "avg_launch_ms": dom["ms"]},
