@@ -156,12 +156,6 @@ int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t 
 size_t plx_spmm_static_scratch_bytes(void);
 int plx_spmm_csr_f32_static(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
                             int64_t ldy, void *stream);
-/* Diagnostic for the benchmark, not part of the path: performs about n_gathers reads of uniformly random rows
- * (D fp32 each, D in {16, 32, 64, 128, 256}) of `table` with the SpMM's load shape and nothing else, so that
- * timing it gives the memory system's ceiling for this access pattern on a table of this size.
- * *gathers_done receives the exact count. */
-int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int64_t D, int64_t n_gathers, int64_t *gathers_done,
-                               float *sink, void *stream);
 /* fp32 values, bf16 H and Y (raw uint16 bit patterns), fp32 accumulation, round-to-nearest-even store. */
 int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_t *H, int64_t ldh, int64_t D,
                       uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
@@ -233,6 +227,12 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
 /* Y = bf16(X) (transpose = 0, Y is [M x N]) or bf16(X^T) (transpose = 1, Y is [N x M]); X is [M x N] fp32. */
 int plx_cast_f32_bf16(int64_t M, int64_t N, const float *X, int64_t ldx, uint16_t *Y, int64_t ldy, int transpose,
                       void *stream);
+
+/* Copies M rows of row_bytes bytes from one row pitch to another (fp32 or bf16 matrices whose rows are padded
+ * differently; everything a multiple of 2 bytes).  Used where a narrow matrix is padded to 16-byte rows for the SpMM
+ * of a layer that transforms before it aggregates; it has no counterpart in the reference. */
+int plx_copy_rows(int64_t M, int64_t row_bytes, const void *src, int64_t src_pitch_bytes, void *dst, int64_t dst_pitch_bytes,
+                  void *stream);
 
 /* Y = max(X, 0) and dX = dY ⊙ [Y > 0] for callers that keep F.relu outside the layer
  * (examples/train.py:77-78).  Outputs may alias inputs. */

@@ -43,7 +43,6 @@ SIGNATURES = {
     "plx_spmm_csr_rows_f32": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_spmm_static_scratch_bytes": (_sz, []),
     "plx_spmm_csr_f32_static": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
-    "plx_diag_random_gather_f32": (C.c_int, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_i64), _vp, _vp]),
     "plx_spmm_csr_bf16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_spmm_csr_rows_bf16": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_gemm_nn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp]),
@@ -53,6 +52,7 @@ SIGNATURES = {
     "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_copy_rows": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_relu_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_relu_bwd_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_softmax_xent_workspace_bytes": (_sz, [_i64, _i64]),
@@ -68,6 +68,11 @@ SIGNATURES = {
     "plx_gemm_tn_bf16": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz, _vp]),
     "plx_cast_f32_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, C.c_int, _vp]),
     "plx_softmax_xent_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
+}
+
+# include/plexus_hip_diag.h: measurement probes, not part of the path
+DIAG_SIGNATURES = {
+    "plx_diag_random_gather_f32": (C.c_int, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_i64), _vp, _vp]),
 }
 
 PLX_GEMM_RELU = 1
@@ -92,7 +97,7 @@ def load():
                 "(or `python -c 'import __graft_entry__ as g; g.build()'`); there is no CPU fallback"
             )
         lib = C.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
+        for name, (res, args) in list(SIGNATURES.items()) + list(DIAG_SIGNATURES.items()):
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args

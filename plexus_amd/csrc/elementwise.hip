@@ -57,6 +57,18 @@ __global__ void __launch_bounds__(256) relu_kernel(int64_t M, int64_t N, const f
 
 bool aligned4(const void *p, int64_t ld) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && ld % 4 == 0; }
 
+// rows of `row_bytes` bytes from one pitch to another; UNIT = bytes per thread item (16 when everything is 16-byte
+// aligned, else 4 or 2)
+template <typename UNIT>
+__global__ void __launch_bounds__(256) copy_rows_kernel(int64_t M, int64_t units_per_row, const char *__restrict__ src, int64_t src_pitch,
+                                                        char *__restrict__ dst, int64_t dst_pitch)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M * units_per_row) return;
+    const int64_t r = i / units_per_row, c = i % units_per_row;
+    reinterpret_cast<UNIT *>(dst + r * dst_pitch)[c] = reinterpret_cast<const UNIT *>(src + r * src_pitch)[c];
+}
+
 // d^-1/2 of the row sums.  A wavefront sums one row; rows longer than kLongRow entries (the hubs of a power-law
 // graph: one row of the benchmark graph holds 1.1 M entries) are left to the whole workgroup afterwards, with four
 // loads in flight per thread.  Both orders of summation are fixed.
@@ -314,6 +326,28 @@ int plx_scale_by_device_scalar_f32(int64_t n, const float *x, const float *scale
 int plx_scale_by_device_scalar_bf16(int64_t n, const uint16_t *x, const float *scale, uint16_t *y, void *stream)
 {
     return scale_common<uint16_t>(n, x, scale, y, stream);
+}
+
+int plx_copy_rows(int64_t M, int64_t row_bytes, const void *src, int64_t src_pitch_bytes, void *dst, int64_t dst_pitch_bytes,
+                  void *stream)
+{
+    PLX_REQUIRE(M >= 0 && row_bytes >= 0, "copy_rows: negative size");
+    if (M == 0 || row_bytes == 0) return PLX_OK;
+    PLX_REQUIRE(src != nullptr && dst != nullptr, "copy_rows: NULL operand");
+    PLX_REQUIRE(src_pitch_bytes >= row_bytes && dst_pitch_bytes >= row_bytes, "copy_rows: pitch smaller than a row");
+    const uintptr_t all = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes |
+                          (uintptr_t)src_pitch_bytes | (uintptr_t)dst_pitch_bytes;
+    PLX_REQUIRE(all % 2 == 0, "copy_rows: addresses, pitches and the row length must be multiples of 2 bytes");
+    hipStream_t st = plx::as_stream(stream);
+    const char *s = static_cast<const char *>(src);
+    char *d = static_cast<char *>(dst);
+    auto blocks = [&](int64_t unit) { return (unsigned)plx::ceil_div(M * (row_bytes / unit), 256); };
+    PLX_REQUIRE(M * row_bytes / 2 < (1ll << 39), "copy_rows: too large");
+    if (all % 16 == 0) copy_rows_kernel<uint4><<<blocks(16), 256, 0, st>>>(M, row_bytes / 16, s, src_pitch_bytes, d, dst_pitch_bytes);
+    else if (all % 4 == 0) copy_rows_kernel<uint32_t><<<blocks(4), 256, 0, st>>>(M, row_bytes / 4, s, src_pitch_bytes, d, dst_pitch_bytes);
+    else copy_rows_kernel<uint16_t><<<blocks(2), 256, 0, st>>>(M, row_bytes / 2, s, src_pitch_bytes, d, dst_pitch_bytes);
+    PLX_LAUNCH_CHECK("copy_rows_kernel");
+    return PLX_OK;
 }
 
 int plx_relu_f32(int64_t M, int64_t N, const float *X, int64_t ldx, float *Y, int64_t ldy, void *stream)

@@ -22,6 +22,7 @@
 
 #include "common.h"
 #include "plan_build.h"
+#include "plexus_hip_diag.h"
 
 // Scratch of plx_spmm_csr_f32_static: fp32 partial rows of the split rows.  Every GPU the library runs on holds its own
 // copy of this array, at its own address, until the process ends.

@@ -122,10 +122,11 @@ class GCNConvFunction(torch.autograd.Function):
         quantum = 8 if bf16 else 4  # rows of Z padded to 16 bytes so that the gather uses 128-bit loads
         d_pad = (d_out + quantum - 1) // quantum * quantum
         timers.start("OUT = AGG * W")
-        alloc = torch.zeros if d_pad != d_out else torch.empty
-        Z = alloc((H.shape[0], d_pad), dtype=x.dtype, device=H.device)
+        # the padding columns are never written: the SpMM carries them through as columns of their own, and every
+        # consumer reads the first d_out columns only
+        Z = torch.empty((H.shape[0], d_pad), dtype=x.dtype, device=H.device)
         if bf16:
-            Z[:, :d_out].copy_(ops.gemm_nt_bf16(H, ops.cast_bf16(W, transpose=True)))
+            ops.copy_rows(ops.gemm_nt_bf16(H, ops.cast_bf16(W, transpose=True)), Z[:, :d_out])
         else:
             ops.gemm_nn(H, W, out=Z[:, :d_out])
         timers.stop("OUT = AGG * W")
@@ -157,12 +158,17 @@ class GCNConvFunction(torch.autograd.Function):
         quantum = 8 if ctx.bf16 else 4
         d_pad = (d_out + quantum - 1) // quantum * quantum
         m = grad_output.shape[0]
-        alloc = torch.zeros if d_pad != d_out else torch.empty
-        Gp = alloc((m, d_pad), dtype=grad_output.dtype, device=grad_output.device)
-        if ctx.fuse_relu:
-            ops.relu_bwd(grad_output, out, out=Gp[:, :d_out])
+        whole = ops._whole_padded_rows(grad_output) if d_pad != d_out else None
+        if not ctx.fuse_relu and d_pad == d_out and grad_output.is_contiguous():
+            Gp = grad_output
+        elif not ctx.fuse_relu and whole is not None and whole.shape[1] == d_pad:
+            Gp = whole  # the gradient already lies in rows of d_pad elements (the loss writes it in the layout of its logits)
         else:
-            Gp[:, :d_out].copy_(grad_output)
+            Gp = torch.empty((m, d_pad), dtype=grad_output.dtype, device=grad_output.device)
+            if ctx.fuse_relu:
+                ops.relu_bwd(grad_output, out, out=Gp[:, :d_out])
+            else:
+                ops.copy_rows(grad_output, Gp[:, :d_out])
         timers.start("GRAD_H = A.T * GRAD_AGG")
         T = ops.spmm(ctx.adj_t, Gp)[:, :d_out]
         timers.stop("GRAD_H = A.T * GRAD_AGG")

@@ -494,6 +494,20 @@ def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] 
     return c
 
 
+def copy_rows(src: torch.Tensor, dst: torch.Tensor) -> torch.Tensor:
+    """dst[:, :] = src for two row-major matrices of one shape and dtype with any row pitches (no torch kernel)."""
+    _need_gpu(src, dst)
+    if src.shape != dst.shape or src.dtype != dst.dtype or src.dim() != 2:
+        raise ValueError("copy_rows: two 2-D tensors of one shape and dtype expected")
+    src = _rowmajor(src)
+    if dst.shape[1] > 1 and dst.stride(1) != 1:
+        raise ValueError("copy_rows: the rows of the destination must be contiguous")
+    es = src.element_size()
+    m, n = src.shape
+    check(_lib.load().plx_copy_rows(m, n * es, src.data_ptr(), _ld(src) * es, dst.data_ptr(), _ld(dst) * es, _stream()), "plx_copy_rows")
+    return dst
+
+
 def relu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     _need_gpu(x)
     if x.dtype != torch.float32 or x.dim() != 2:
@@ -535,7 +549,13 @@ def softmax_xent(logits: torch.Tensor, labels: torch.Tensor, num_nodes: int, num
     if fn is None:
         raise TypeError("softmax_xent: unsupported dtype %s" % logits.dtype)
     loss = torch.empty(1, dtype=torch.float32, device=logits.device)
-    dlogits = torch.empty((m, c), dtype=logits.dtype, device=logits.device) if want_grad else None
+    dlogits = None
+    if want_grad:
+        # the gradient takes the row pitch of the logits: a consumer that padded its rows (for 16-byte loads) gets it
+        # back in the same layout
+        ld = _ld(logits)
+        dlogits = torch.empty((m, ld), dtype=logits.dtype, device=logits.device)[:, :c] if ld != c else \
+            torch.empty((m, c), dtype=logits.dtype, device=logits.device)
     need = int(lib.plx_softmax_xent_workspace_bytes(m, c))
     ws = torch.empty(need, dtype=torch.uint8, device=logits.device)
     check(
@@ -548,6 +568,17 @@ def softmax_xent(logits: torch.Tensor, labels: torch.Tensor, num_nodes: int, num
     return loss, dlogits
 
 
+def _whole_padded_rows(x: torch.Tensor):
+    """The [rows x pitch] matrix behind a row-major 2-D view whose rows are padded, if the view starts its storage and the
+    storage holds every padded row whole; else None."""
+    if x.dim() != 2 or x.shape[0] == 0 or x.shape[1] == 0 or x.stride(1) != 1 or x.stride(0) <= x.shape[1] or x.storage_offset() != 0:
+        return None
+    m, ld = x.shape[0], x.stride(0)
+    if x.untyped_storage().nbytes() < m * ld * x.element_size():
+        return None
+    return x.as_strided((m, ld), (ld, 1))
+
+
 def scale_by_scalar(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     """x * scale for a one-element fp32 device tensor ``scale`` (read on the device; the host does not wait for it)."""
     _need_gpu(x, scale)
@@ -557,8 +588,13 @@ def scale_by_scalar(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     fn = {torch.float32: lib.plx_scale_by_device_scalar_f32, torch.bfloat16: lib.plx_scale_by_device_scalar_bf16}.get(x.dtype)
     if fn is None:
         raise TypeError("scale_by_scalar: unsupported dtype %s" % x.dtype)
-    x = x.contiguous()
     scale = scale.detach().reshape(1).to(torch.float32)
+    base = _whole_padded_rows(x)
+    if base is not None:  # rows padded to a longer pitch, whole in their storage: scaled with their padding, layout kept
+        yb = torch.empty_like(base)
+        check(fn(base.numel(), base.data_ptr(), scale.data_ptr(), yb.data_ptr(), _stream()), "plx_scale_by_device_scalar")
+        return yb[:, :x.shape[1]]
+    x = x.contiguous()
     y = torch.empty_like(x)
     check(fn(x.numel(), x.data_ptr(), scale.data_ptr(), y.data_ptr(), _stream()), "plx_scale_by_device_scalar")
     return y

@@ -13,8 +13,8 @@ from plexus_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_symbols():
-    text = open(os.path.join(ROOT, "include", "plexus_hip.h")).read()
+def header_symbols(name="plexus_hip.h"):
+    text = open(os.path.join(ROOT, "include", name)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(plx_[a-z0-9_]+)\s*\(", text)))
 
@@ -26,6 +26,11 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(lib, s), "libplexus_hip.so does not export %s" % s
     # and the Python binding table covers exactly the header
     assert sorted(_lib.SIGNATURES) == syms
+    # the measurement probes live in their own header
+    diag = header_symbols("plexus_hip_diag.h")
+    assert sorted(_lib.DIAG_SIGNATURES) == diag and not set(diag) & set(syms)
+    for s in diag:
+        assert hasattr(lib, s), "libplexus_hip.so does not export %s" % s
 
 
 def header_prototypes():
