@@ -32,13 +32,15 @@ def device_csr_pair(g):
     return (ops.CsrMatrix(g.rowptr, g.col, g.val, g.shape), ops.CsrMatrix(g.rowptr_t, g.col_t, g.val_t, (g.shape[1], g.shape[0])))
 
 
-def network_forward_loss_backward(scale, max_flips):
-    """One forward + loss + backward of the three-layer fp32 network, every tensor of it against the oracle."""
+def network_forward_loss_backward(scale, max_flips, g=None, DIMS3=DIMS3):
+    """One forward + loss + backward of a three-layer fp32 network, every tensor of it against the oracle."""
     from plexus_amd.cross_entropy import parallel_cross_entropy
     from plexus_amd.gcn_conv import GCNConv
 
-    g = S.config3_graph(DEV, seed=0, scale=scale)
+    if g is None:
+        g = S.config3_graph(DEV, seed=0, scale=scale)
     n = g.shape[0]
+    assert g.shape[0] == g.shape[1]
     print(g.degree_stats(), flush=True)
     x = S.normal_features(n, DIMS3[0], DEV, seed=1)
     y = S.uniform_labels(n, DIMS3[-1], DEV, seed=2)
@@ -99,6 +101,50 @@ def test_config3_network_forward_loss_backward_at_a_tenth():
 def test_config3_network_forward_loss_backward_full_size():
     say("config 3 network 100-128-128-47 fp32, full size (2.45 M nodes): logits, loss, hidden activations, grad_x, grad_w")
     network_forward_loss_backward(1.0, max_flips=80)
+
+
+def test_config4_rank_block_network_full_size():
+    """One rank's block of a 2 x 2 x 2 grid at its real shape (rows and columns [0, N/2) of a doubly permuted R-MAT graph with
+    N = 8,388,608: 4,194,304 x 4,194,304, about 64 M entries, not symmetric), local widths 64 -> 64 -> 64 -> 24: forward,
+    loss and backward of the three layers against the oracle in fp32 and fp64."""
+    say("config 4 block network 64-64-64-24 fp32, full size")
+    g = S.config4_block(DEV, seed=0, scale=1.0)
+    assert not torch.equal(g.rowptr, g.rowptr_t)
+    network_forward_loss_backward(1.0, max_flips=80, g=g, DIMS3=[64, 64, 64, 24])
+
+
+def test_config5_network_full_size_bf16_dropout():
+    """The bf16-storage 256-256-256-47 network with dropout 0.5 at full size (2.45 M nodes): logits, loss, grad_x and the
+    three grad_w against the bf16-storage oracle, which regenerates the dropout masks from the same seed and offsets."""
+    say("config 5 network 256-256-256-47 bf16 + dropout, full size")
+    from plexus_amd.cross_entropy import parallel_cross_entropy
+    from plexus_amd.train import Net
+
+    dims, seed = [256, 256, 256, 47], 11
+    g = S.config3_graph(DEV, seed=0, scale=1.0)
+    n = g.shape[0]
+    x = S.normal_features(n, dims[0], DEV, seed=1)
+    y = S.uniform_labels(n, dims[-1], DEV, seed=2)
+    ws = S.glorot_weights(dims, seed=0)
+    model = Net(3, dims[0], dims[1], dims[-1], weights=ws, fuse_relu=True, dropout=0.5, dropout_seed=seed)
+    model.train()
+    offsets = [layer.next_dropout_offset() for layer in model.layers]
+    xd = x.to(torch.bfloat16).requires_grad_()
+    logits = model(xd, [device_csr_pair(g)])
+    loss = parallel_cross_entropy(logits, y, 3, n, dims[-1])
+    loss.backward()
+    torch.cuda.synchronize()
+
+    net = po.OracleNetBf16(ws, dims, dropout_p=0.5, seed=seed)
+    ref_logits = net.forward(x.cpu(), [host_csr_pair(g)], offsets)
+    ref_loss, sm, oh = po.cross_entropy_forward(ref_logits, y.cpu(), n, dims[-1])
+    gx_ref, gws_ref = net.backward(po.cross_entropy_backward(sm, oh.float(), n))
+    errs = {"logits": rel_err(logits.float(), ref_logits), "loss": abs(loss.item() - ref_loss.item()) / abs(ref_loss.item()),
+            "grad_x": rel_err(xd.grad.float(), gx_ref.reshape(n, dims[0]))}
+    for i, (layer, gw) in enumerate(zip(model.layers, gws_ref)):
+        errs["grad_w[%d]" % i] = rel_err(layer.weight.grad, gw)
+    print("loss gpu %.6f oracle %.6f; rel errors %s" % (loss.item(), ref_loss.item(), {k: "%.2e" % v for k, v in errs.items()}), flush=True)
+    assert all(v <= BF16_TOL for v in errs.values()), errs
 
 
 def test_config3_ten_epoch_loss_curve():
