@@ -112,7 +112,8 @@ typedef struct plx_spmm_plan plx_spmm_plan;
 int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr,
                          const int32_t *col, int32_t seg_len, void *stream);
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
-/* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len */
+/* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len, 6: hub rows, 7: entries in hub rows,
+ * 8: bytes of the hub pass's tables */
 int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
 /* Copies the plan's tables to host arrays (any of them may be NULL): long rows [long rows], seg_first [long rows + 1],
  * seg_begin / seg_end [segments] -- the layout of plx_spmm_segments_host.  For inspection and tests; synchronous. */
@@ -125,6 +126,22 @@ int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host
  * line-aligned copy, or in one pass when neither is possible -- sums each element in the same order, so they agree bit
  * for bit.  mode 0: decide by that rule (the default); 1: slice whenever a row exceeds 256 bytes; -1: never. */
 int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
+/* The hub pass.  On a power-law graph a third of the entries sit in a few thousand rows; gathered row by row they miss
+ * the cache like every other row.  A plan may carry tables that let those rows ("hub rows": the longest of the split
+ * rows, cut into at most 9,216 parts of at most 8 * seg_len entries) walk the columns together, window after window of
+ * 4,096 columns, one eighth of the columns per XCD, so that a row of H fetched for one of them is found in that XCD's
+ * L2 by the others (2.45 M nodes, 126 M entries, 128 fp32 columns: 7.3 -> 5.7 ms).  The tables cost 5 bytes per entry
+ * of a hub row.  plx_spmm_plan_create builds them by itself where it expects a gain: short rows on average (fewer
+ * than 128 entries, the shapes that do not take column slices), 512-byte rows of H beyond 128 MB in total, an eighth
+ * of the entries in hub rows.  plx_spmm_plan_build_hub builds them for any plan with split rows (synchronises
+ * `stream`).  A product uses the pass when the tables exist, the mode allows it, the shape is not a sliced one, H
+ * as passed spans less than 4 GiB and its base, row pitch and width are multiples of 4 elements; a row range runs the
+ * whole pass if it holds a hub row.  The order of every sum is fixed by the plan: the same operands give the same bits
+ * on every call and in every row range, but not the bits of a product without the pass (the two agree to fp32
+ * rounding).  plx_spmm_csr_f32_static never uses it.
+ * mode 0: use the pass where possible (the default), -1: never. */
+int plx_spmm_plan_build_hub(plx_spmm_plan *plan, void *stream);
+int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode);
 /* bytes of scratch an SpMM of width D needs: fp32 partial sums of the split rows, plus -- when rows of D fp32
  * elements laid end to end straddle more 128-byte lines than they have to and every row of H is gathered often
  * enough to repay a copy -- room for a copy of H in rows that start on lines, which whole-matrix products then

@@ -38,6 +38,8 @@ SIGNATURES = {
     "plx_spmm_plan_info": (_i64, [_vp, C.c_int]),
     "plx_spmm_plan_tables_host": (C.c_int, [_vp, _vp, _vp, _vp, _vp]),
     "plx_spmm_plan_set_slicing": (C.c_int, [_vp, C.c_int]),
+    "plx_spmm_plan_build_hub": (C.c_int, [_vp, _vp]),
+    "plx_spmm_plan_set_hub": (C.c_int, [_vp, C.c_int]),
     "plx_spmm_workspace_bytes": (_sz, [_vp, _i64]),
     "plx_spmm_csr_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_spmm_csr_rows_f32": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),

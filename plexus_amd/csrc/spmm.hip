@@ -22,6 +22,7 @@
 
 #include "common.h"
 #include "plan_build.h"
+#include "spmm_hub.h"
 #include "plexus_hip_diag.h"
 
 // Scratch of plx_spmm_csr_f32_static: fp32 partial rows of the split rows.  Every GPU the library runs on holds its own
@@ -53,6 +54,7 @@ struct SpmmArgs {
     int32_t row_end;
     int32_t seg_base;  // index of the first segment task in the plan's tables
     int32_t y_vec;     // 1: rows of Y take VEC-wide stores; 0: element stores, each guarded by the width D
+    const uint8_t *seg_skip;  // flags over the plan's segments: tasks left to the hub pass (or NULL)
 };
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
@@ -216,6 +218,7 @@ __global__ void __launch_bounds__(256) spmm_csr_kernel(const SpmmArgs p)
     bool to_ws;
     int64_t out_row;
     if (task < p.n_seg) {
+        if (p.seg_skip != nullptr && p.seg_skip[p.seg_base + task]) return;
         a = p.seg_begin[p.seg_base + task];
         b = p.seg_end[p.seg_base + task];
         to_ws = true;
@@ -371,10 +374,12 @@ template <typename TOUT>
 __global__ void __launch_bounds__(256) spmm_reduce_split_rows(const float *__restrict__ ws, int64_t ldws,
                                                               const int32_t *__restrict__ long_rows,
                                                               const int32_t *__restrict__ seg_first, int32_t q_base,
-                                                              int32_t D, TOUT *__restrict__ Y, int64_t ldy)
+                                                              int32_t D, TOUT *__restrict__ Y, int64_t ldy,
+                                                              const uint8_t *__restrict__ long_skip)
 {
     __shared__ float4 part[16][16];
     const int q = q_base + blockIdx.x;
+    if (long_skip != nullptr && long_skip[q]) return;  // a hub row: the hub pass writes it
     const int chain = threadIdx.x >> 4;
     const int l = threadIdx.x & 15;
     const int d = blockIdx.y * 64 + l * 4;
@@ -533,6 +538,8 @@ struct plx_spmm_plan {
     const int32_t *long_rows, *seg_first, *seg_begin, *seg_end;
     std::vector<int32_t> h_long_rows, h_seg_first;  // host copies, to cut row ranges out of the plan
     int slicing = 0;  // 0: column slices of H where the cost model says so, 1: whenever rows exceed a slice, -1: never
+    plx::hub::HubPlan hub;  // tables of the hub pass (empty: no hub pass)
+    int hub_mode = 0;       // 0: hub pass where the tables exist and the operands allow it, -1: never
 };
 
 namespace {
@@ -615,6 +622,14 @@ int64_t wanted_stage_ld(const plx_spmm_plan *plan, int64_t D, int64_t elem, uint
     return staged_ld(plan->K, plan->nnz, D, elem, base, ldh);
 }
 
+// room for the partial sums of the hub pass, or 0 when this plan and width do not use it (column slices and the hub
+// pass answer different shapes of matrix; a product takes one or the other)
+size_t hub_workspace_bytes(const plx_spmm_plan *plan, int64_t D, int64_t elem)
+{
+    if (plan->hub.block == nullptr || plan->hub_mode < 0 || sliced_plan(plan, D, elem)) return 0;
+    return plx::hub::partial_bytes(D);
+}
+
 // `may_stage` = false: the workspace holds the partial rows of the split rows and nothing else (H is gathered where
 // it lies; same values in the same order, so the same result)
 template <typename T>
@@ -630,6 +645,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
     const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+    const size_t hub_bytes = may_stage ? hub_workspace_bytes(plan, D, sizeof(T)) : 0;
     const size_t need = may_stage ? plx_spmm_workspace_bytes(plan, D) : seg_bytes;
     if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return plx::fail(PLX_ERR_WORKSPACE, "spmm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -644,12 +660,14 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     // Whole-matrix products stage H into line-aligned rows when that pays and the workspace has the room (the size
     // query reserves it for contiguous fp32 rows); the partial rows of split rows follow the staged copy.
     char *ws_base = static_cast<char *>(workspace);
+    const T *const H0 = H;  // the operand as the caller passed it
+    const int64_t ldh0 = ldh;
     bool h_is_staged = false;  // H points at the copy: rows on 128-byte lines, padded to whole lines
     if (may_stage && whole) {
         const int64_t ld_st = wanted_stage_ld(plan, D, kElem, reinterpret_cast<uintptr_t>(H), ldh);
         const size_t st_bytes = (size_t)plan->K * (size_t)ld_st * sizeof(T);
         const size_t pad = ws_base ? (size_t)((kLine - reinterpret_cast<uintptr_t>(ws_base) % kLine) % kLine) : 0;
-        if (ld_st > 0 && ws_base != nullptr && workspace_bytes >= pad + st_bytes + seg_bytes) {
+        if (ld_st > 0 && ws_base != nullptr && workspace_bytes >= pad + st_bytes + seg_bytes + hub_bytes) {
             T *staged = reinterpret_cast<T *>(ws_base + pad);
             const unsigned sblocks = (unsigned)plx::ceil_div(plan->K, 4);
             int sv = kMaxVec;
@@ -670,7 +688,31 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
         }
     }
 
+    // ---- the hub pass takes the longest rows when the plan has its tables and the caller's H suits its loads ----
+    // (4-element vectors at 32-bit byte offsets).  The choice looks at the operand as the caller passed it, so a whole
+    // product and a row range of it choose alike, and a row range runs the whole pass when it holds a hub row: the sums
+    // of a hub row are then the same bits whatever range it is computed in and wherever H is gathered from.
+    bool use_hub = false;
+    const T *hub_h = H0;
+    int64_t hub_ldh = ldh0;
+    if (hub_bytes > 0) {
+        const auto &hr = plan->hub.h_rows_sorted;
+        const bool any = std::lower_bound(hr.begin(), hr.end(), (int32_t)row_begin) != std::lower_bound(hr.begin(), hr.end(), (int32_t)row_end);
+        use_hub = any && D % 4 == 0 && ldh0 % 4 == 0 && reinterpret_cast<uintptr_t>(H0) % (4 * sizeof(T)) == 0 &&
+                  plan->K * ldh0 * kElem < plx::hub::kHubMaxBytes;
+        if (h_is_staged && plan->K * ldh * kElem < plx::hub::kHubMaxBytes) {
+            hub_h = H;
+            hub_ldh = ldh;
+        }
+    }
+    float *hub_partial = reinterpret_cast<float *>(ws_base + seg_bytes);  // seg_bytes is a multiple of 16
+    auto hub_pass = [&]() -> int {
+        if (!use_hub) return PLX_OK;
+        return plx::hub::launch(plan->hub, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st);
+    };
+
     SpmmArgs a;
+    a.seg_skip = use_hub ? plan->hub.seg_is_hub : nullptr;
     a.rowptr = plan->rowptr;
     a.col = plan->col;
     a.val = val;
@@ -695,7 +737,8 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     auto reduce_split_rows = [&](T *y, int64_t d) -> int {
         if (q1 > q0) {
             dim3 rgrid((unsigned)(q1 - q0), (unsigned)plx::ceil_div(d, 64), 1);
-            spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)d, y, ldy);
+            spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)d, y, ldy,
+                                                             use_hub ? plan->hub.long_is_hub : nullptr);
             PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
         }
         return PLX_OK;
@@ -770,7 +813,9 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     }
     if (rc != 0) return plx::fail(PLX_ERR_UNSUPPORTED, "spmm: no kernel for vec=%d lpr=%d nacc=%d%s", vec, lpr, nacc, sliced ? " (chained)" : "");
     PLX_LAUNCH_CHECK("spmm_csr_kernel");
-    return reduce_split_rows(Y, D);
+    rc = reduce_split_rows(Y, D);
+    if (rc != PLX_OK) return rc;
+    return hub_pass();
 }
 
 // ---- the product without a caller's workspace: partial rows of the split rows in a static device array ----
@@ -793,6 +838,18 @@ int static_scratch(void **out)
         g_scratch_ptr[dev] = ptr;
     }
     *out = g_scratch_ptr[dev];
+    return PLX_OK;
+}
+
+// the tables of the hub pass, kept when the hub rows hold at least `min_entries` entries
+int build_hub(plx_spmm_plan *p, int64_t min_entries, hipStream_t st)
+{
+    if (p->n_long == 0) return PLX_OK;
+    plx::hub::HubPlan hp;
+    const int rc = plx::hub::build_hub_plan(p->M, p->K, p->nnz, p->rowptr, p->col, p->seg_len, p->n_long, p->n_seg, p->long_rows, p->seg_first,
+                                            p->h_long_rows, min_entries, st, hp);
+    if (rc != PLX_OK) return rc;
+    p->hub = std::move(hp);
     return PLX_OK;
 }
 
@@ -899,13 +956,40 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
         p->seg_begin = p->seg_first + t.n_long + 1;
         p->seg_end = p->seg_begin + t.n_seg;
     }
+    // The hub pass pays where H is far larger than the caches (its rows are then fetched again for almost every
+    // entry), rows are short on average (wide-row matrices take column slices instead) and the long rows hold a good
+    // part of the entries: measured on the 2.45 M-node power-law graph, 128 fp32 columns, 33 % of the entries in hub
+    // rows: 7.3 ms without, 5.7 ms with.
+    if (t.n_long > 0 && M > 0 && nnz / M < 128 && K * 512 >= (128ll << 20)) {
+        const int hrc = build_hub(p, nnz / 8, st);
+        if (hrc != PLX_OK) {
+            plx_spmm_plan_destroy(p);
+            return hrc;
+        }
+    }
     *out = p;
+    return PLX_OK;
+}
+
+int plx_spmm_plan_build_hub(plx_spmm_plan *plan, void *stream)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_build_hub: plan is NULL");
+    if (plan->hub.block != nullptr) return PLX_OK;
+    return build_hub(plan, 1, plx::as_stream(stream));
+}
+
+int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_set_hub: plan is NULL");
+    PLX_REQUIRE(mode >= -1 && mode <= 0, "plan_set_hub: mode must be -1 or 0");
+    plan->hub_mode = mode;
     return PLX_OK;
 }
 
 int plx_spmm_plan_destroy(plx_spmm_plan *plan)
 {
     if (!plan) return PLX_OK;
+    plx::hub::free_hub_plan(plan->hub);
     if (plan->tables) (void)hipFree(plan->tables);
     delete plan;
     return PLX_OK;
@@ -921,6 +1005,9 @@ int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what)
         case 3: return plan->n_long;
         case 4: return plan->n_seg;
         case 5: return plan->seg_len;
+        case 6: return plan->hub.n_rows;
+        case 7: return plan->hub.entries;
+        case 8: return plan->hub.stored * 5;  // bytes of the streams
         default: return -1;
     }
 }
@@ -948,8 +1035,9 @@ size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)
     // room for the line-aligned copy of H, decided for contiguous fp32 rows (an operand laid out otherwise is staged
     // only if it fits what the caller brought)
     const int64_t ld_st = wanted_stage_ld(plan, D, 4, 0, D);
-    if (ld_st == 0) return seg_bytes;
-    return (size_t)kLine + (size_t)plan->K * (size_t)ld_st * sizeof(float) + seg_bytes;
+    const size_t hub_bytes = hub_workspace_bytes(plan, D, 4);
+    if (ld_st == 0) return seg_bytes + hub_bytes;
+    return (size_t)kLine + (size_t)plan->K * (size_t)ld_st * sizeof(float) + seg_bytes + hub_bytes;
 }
 
 int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode)

@@ -1,0 +1,609 @@
+// The rows of A with the most entries ("hub rows"), multiplied window by window.
+//
+// On a power-law graph a third of the entries sit in a few thousand rows.  Taken row by row they gather rows of H
+// from all over the matrix like every other row and miss the cache four times out of five.  Here all of them walk
+// the columns together: the columns are cut into kHubRanges ranges, one per XCD, and every range into windows of
+// kHubWindow columns whose rows of H fit the XCD's L2; the kHubGroups workgroups of a range go through its windows
+// in the same order, each adding the entries that its own rows have in the window, so that a row of H fetched for
+// one hub row is found in L2 by the others that reference it.
+//
+// A hub row is cut into parts of bounded length ("slots": part s of S takes the s-th S-th of the row's entries inside
+// every window), and the slots are dealt over the wavefronts by size.  A workgroup keeps the sums of its slots for its
+// range in LDS for the whole pass; a wavefront owns kHubRowsPerWave of them, so no two wavefronts touch the same sum
+// and nothing needs an atomic or a barrier.  The entries of a slot inside a window are a contiguous run of the CSR
+// arrays (columns are sorted within a row); the plan writes out, for every wavefront, the runs of its slots window
+// after window as one stream of positions.  The partial sums of the kHubRanges ranges of a slot go to memory and a
+// second kernel adds them, slot by slot and range by range, into the row of Y: the order of every sum is fixed by
+// the plan, so the result does not change from call to call or with the row range of the call.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <numeric>
+#include <type_traits>
+#include <vector>
+
+#include "common.h"
+#include "spmm_hub.h"
+
+#ifndef PLX_HUB_U
+#define PLX_HUB_U 8
+#endif
+
+namespace {
+
+using plx::kWave;
+using namespace plx::hub;
+
+struct HubArgs {
+    const int32_t *col;
+    const float *val;
+    const void *H;
+    int64_t ldh;
+    int32_t D, d_read;
+    const int32_t *hub_row;
+    const int64_t *stream_first;
+    const int32_t *stream_total;
+    const int32_t *stream_pos;
+    const uint8_t *stream_run;
+    int32_t n_rows;
+    const int32_t *rows;
+    const int32_t *row_slot_first;
+    const int32_t *row_slots;
+    int32_t row_begin, row_end;
+    float *partial;  // [kHubRanges][kHubSlots][ldp]
+    int64_t ldp;
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const T *p, float (&o)[VEC])
+{
+    static_assert(VEC == 4, "four elements per lane");
+    if constexpr (sizeof(T) == 4) {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        o[0] = t.x;
+        o[1] = t.y;
+        o[2] = t.z;
+        o[3] = t.w;
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        o[0] = __uint_as_float(t.x << 16);
+        o[1] = __uint_as_float(t.x & 0xffff0000u);
+        o[2] = __uint_as_float(t.y << 16);
+        o[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+}
+
+// One wavefront = one stream: the entries of its kHubRowsPerWave slots inside its range of columns, window after
+// window, written out by the plan as positions in the CSR arrays (stream_pos) and slot numbers (stream_run), padded
+// to whole batches of 64.  A batch moves through four stages, one per turn of the loop, so that no load is waited for
+// in the turn that issues it: positions and slots (coalesced) -> column and value of every entry (gathered) -> byte
+// offset of the row of H and value into LDS, run boundaries as a bit mask -> rows of H.  The vector memory pipeline
+// takes as long for a 64-lane load of 8 bytes per lane as for one of 16, so a row of H is read by half a wavefront,
+// 16 bytes per lane: lanes 0-31 go through entries 0-31 of the batch and lanes 32-63 through entries 32-63, U steps
+// at a time, the loads of one set of steps in flight while the set before is added up.  Every turn issues the same
+// loads whatever it finds (past the end of the stream they repeat its last batch), so the counter of outstanding
+// loads the hardware waits on has a fixed meaning.
+template <typename T>
+__global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int VEC = kHubVec;
+    constexpr int TW = kHubTile;  // columns of H covered by a wavefront
+    constexpr int U = PLX_HUB_U;  // steps (two entries each) per set of loads
+    constexpr int kHalf = kWave / 2;
+    static_assert(kHalf == 4 * U, "the 32 steps of a batch are four sets");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int half = lane >> 5;
+    const int range = blockIdx.x % kHubRanges;  // workgroups go to the XCDs in turn
+    const int group = blockIdx.x / kHubRanges;
+    const int dl = (lane & (kHalf - 1)) * VEC;  // this lane's columns inside the tile
+    const int d0 = blockIdx.y * TW + dl;
+    // a lane whose columns lie past the readable width gathers the first columns instead; its sums are never stored
+    const bool ok = d0 + VEC <= p.d_read;
+    const int off = ok ? d0 : 0;
+
+    float *acc = lds + (size_t)wave * kHubRowsPerWave * TW;  // [kHubRowsPerWave][TW], this wavefront's sums
+    uint2 *ring = reinterpret_cast<uint2 *>(lds + (size_t)kWaves * kHubRowsPerWave * TW) + wave * 3 * kWave;  // [3][64] (offset, value)
+    for (int i = lane; i < kHubRowsPerWave * TW; i += kWave) acc[i] = 0.f;
+
+    const int slot0 = (group * kWaves + wave) * kHubRowsPerWave;
+    const int stream = (range * kHubGroups + group) * kWaves + wave;
+    const int64_t sbase = p.stream_first[stream];
+    const int total = p.stream_total[stream];
+    const int nb = (total + kWave - 1) / kWave;  // batches
+    const char *__restrict__ Hb = static_cast<const char *>(p.H);
+    const uint32_t row_bytes = (uint32_t)(p.ldh * (int64_t)sizeof(T));
+    const uint32_t lane_off = (uint32_t)off * (uint32_t)sizeof(T);
+
+    if (nb > 0) {
+        struct Listed { int pos, run; };
+        struct Read { int c, run; float v; };
+        struct Ready { int run; uint64_t starts; int left; const uint2 *mine; };
+        auto list = [&](int k) {
+            const int64_t at = sbase + (int64_t)min(k, nb - 1) * kWave + lane;
+            Listed x;
+            x.pos = p.stream_pos[at];
+            x.run = p.stream_run[at];
+            return x;
+        };
+        auto read = [&](const Listed &x) {
+            Read y;
+            y.c = p.col[x.pos];
+            y.v = p.val[x.pos];
+            y.run = x.run;
+            return y;
+        };
+        int carry_lo = -1, carry_hi = -1;  // slots of entries 31 and 63 of the batch before: where the two halves stand
+        auto ready = [&](const Read &y, int k, int slot) {
+            Ready z;
+            uint2 *dst = ring + slot * kWave;
+            dst[lane] = make_uint2((uint32_t)y.c * row_bytes, __float_as_uint(y.v));
+            int before = __shfl_up(y.run, 1, kWave);
+            if (lane == 0) before = carry_lo;
+            if (lane == kHalf) before = carry_hi;
+            z.left = min(max(total - k * kWave, 0), kWave);
+            z.starts = __ballot(y.run != before && lane < z.left);
+            carry_lo = __builtin_amdgcn_readlane(y.run, kHalf - 1);
+            carry_hi = __builtin_amdgcn_readlane(y.run, kWave - 1);
+            z.run = y.run;
+            z.mine = dst + half * kHalf;
+            plx::wave_lds_fence();
+            return z;
+        };
+        struct Rows { float h[U][VEC]; float v[U]; };
+        auto fetch = [&](const Ready &z, int g, Rows &r) {
+#pragma unroll
+            for (int u = 0; u < U; u += 2) {
+                const uint4 e = *reinterpret_cast<const uint4 *>(z.mine + g * U + u);  // two entries of this half
+                r.v[u] = __uint_as_float(e.y);
+                r.v[u + 1] = __uint_as_float(e.w);
+                load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.x + lane_off)), r.h[u]);
+                load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.z + lane_off)), r.h[u + 1]);
+            }
+        };
+        int cur = -1;  // the slot this half is summing
+        float sum[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) sum[k] = 0.f;
+        // Products are summed in registers while the slot stays the same and added to the slot's sum in LDS when it
+        // changes; the two halves may hold the same slot, so they add to LDS one after the other.
+        auto flush = [&](int run) {
+            if (cur >= 0) {
+                float4 t = *reinterpret_cast<float4 *>(acc + cur * TW + dl);
+                t.x += sum[0];
+                t.y += sum[1];
+                t.z += sum[2];
+                t.w += sum[3];
+                *reinterpret_cast<float4 *>(acc + cur * TW + dl) = t;
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = 0.f;
+            cur = run;
+        };
+        auto consume = [&](const Ready &z, int g, const Rows &r, auto checked) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = g * U + u;
+                const bool lo = (z.starts >> i) & 1, hi = (z.starts >> (kHalf + i)) & 1;
+                if (lo | hi) {
+                    if (lo) {
+                        const int run = __builtin_amdgcn_readlane(z.run, i);
+                        if (half == 0) flush(run);
+                        plx::wave_lds_fence();
+                    }
+                    if (hi) {
+                        const int run = __builtin_amdgcn_readlane(z.run, kHalf + i);
+                        if (half == 1) flush(run);
+                        plx::wave_lds_fence();
+                    }
+                }
+                if (!decltype(checked)::value || half * kHalf + i < z.left) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) sum[k] = fmaf(r.v[u], r.h[u][k], sum[k]);
+                }
+            }
+        };
+        auto add_up = [&](const Ready &z, int g, const Rows &r) {
+            if (z.left == kWave) consume(z, g, r, std::false_type{});
+            else consume(z, g, r, std::true_type{});
+        };
+
+        Rows ra, rb;
+        Listed l0 = list(0), l1 = list(1), l2 = list(2);
+        Read r0 = read(l0), r1 = read(l1);
+        int s_now = 0, s_next = 1, s_free = 2;
+        Ready now = ready(r0, 0, s_now), next = ready(r1, 1, s_next);
+        Read rd = read(l2);
+        Listed li = list(3);
+        fetch(now, 0, ra);
+        for (int k = 0; k < nb; ++k) {
+            const Ready after = ready(rd, k + 2, s_free);
+            rd = read(li);
+            li = list(k + 4);
+            fetch(now, 1, rb);
+            add_up(now, 0, ra);
+            fetch(now, 2, ra);
+            add_up(now, 1, rb);
+            fetch(now, 3, rb);
+            add_up(now, 2, ra);
+            fetch(next, 0, ra);
+            add_up(now, 3, rb);
+            now = next;
+            next = after;
+            const int t = s_now;
+            s_now = s_next;
+            s_next = s_free;
+            s_free = t;
+        }
+        if (half == 0) flush(-1);
+        plx::wave_lds_fence();
+        if (half == 1) flush(-1);
+        plx::wave_lds_fence();
+    }
+
+    // the sums of this range: P[range][slot][ldp]
+    if (half == 0 && ok) {
+        for (int r = 0; r < kHubRowsPerWave; ++r) {
+            if (p.hub_row[slot0 + r] < 0) continue;
+            float *dst = p.partial + ((int64_t)range * kHubSlots + slot0 + r) * p.ldp + blockIdx.y * TW + dl;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+                if (blockIdx.y * TW + dl + k < p.D) dst[k] = acc[r * TW + dl + k];
+        }
+    }
+}
+
+// Y[hub row] = sum over the row's slots (its parts, in order) and, per slot, over the ranges in range order
+template <typename TOUT>
+__global__ void __launch_bounds__(128) spmm_hub_reduce_kernel(const HubArgs p, TOUT *__restrict__ Y, int64_t ldy)
+{
+    const int q = blockIdx.x;
+    const int row = p.rows[q];
+    if (row < p.row_begin || row >= p.row_end) return;
+    const int s0 = p.row_slot_first[q], s1 = p.row_slot_first[q + 1];
+    for (int d = threadIdx.x; d < p.D; d += blockDim.x) {
+        float s = 0.f;
+        for (int i = s0; i < s1; ++i) {
+            const int slot = p.row_slots[i];
+#pragma unroll
+            for (int x = 0; x < kHubRanges; ++x) s += p.partial[((int64_t)x * kHubSlots + slot) * p.ldp + d];
+        }
+        if constexpr (sizeof(TOUT) == 4) {
+            Y[(int64_t)row * ldy + d] = s;
+        } else {
+            uint32_t u = __float_as_uint(s);
+            if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;
+            else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+            Y[(int64_t)row * ldy + d] = (uint16_t)u;
+        }
+    }
+}
+
+// ---- construction of the streams ----
+struct BuildArgs {
+    const int32_t *rowptr;
+    const int32_t *col;
+    const int32_t *hub_row;   // [kHubSlots]
+    const int32_t *hub_part;  // [kHubSlots] part | parts << 16
+    int32_t window, windows_per_range, n_windows;
+    const int64_t *stream_first;  // fill
+    int32_t *stream_total;        // count
+    int32_t *stream_pos;          // fill
+    uint8_t *stream_run;          // fill
+};
+
+// One wavefront per stream.  Lane l follows slot l of the wavefront through the windows of the range: the entries of
+// the slot's row inside a window (found by bisection over the row's sorted columns) and the slot's share of them.
+// FILL = false adds up the stream's length; FILL = true writes the stream: the runs of a window one after the other,
+// 64 entries per step (entry f of the window belongs to the last slot whose exclusive prefix of run lengths is <= f).
+template <bool FILL>
+__global__ void __launch_bounds__(64) hub_streams_kernel(const BuildArgs b)
+{
+    __shared__ int prefix[kWave];
+    __shared__ int delta[kWave];
+    const int lane = threadIdx.x;
+    const int stream = blockIdx.x;
+    const int wave = stream % kWaves, group = (stream / kWaves) % kHubGroups, range = stream / (kWaves * kHubGroups);
+    const int slot = (group * kWaves + wave) * kHubRowsPerWave + min(lane, kHubRowsPerWave - 1);
+    const int row = lane < kHubRowsPerWave ? b.hub_row[slot] : -1;
+    int lo_pos = 0, end_pos = 0, part = 0, parts = 1;
+    if (row >= 0) {
+        lo_pos = b.rowptr[row];
+        end_pos = b.rowptr[row + 1];
+        part = b.hub_part[slot] & 0xffff;
+        parts = b.hub_part[slot] >> 16;
+    }
+    auto first_at_least = [&](int from, int64_t target) {  // first position in [from, end_pos] whose column is >= target
+        int lo = from, hi = end_pos;
+        while (lo < hi) {
+            const int mid = lo + ((hi - lo) >> 1);
+            if ((int64_t)b.col[mid] < target) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    };
+    const int w_begin = range * b.windows_per_range, w_end = min(w_begin + b.windows_per_range, b.n_windows);
+    int p0 = row >= 0 ? first_at_least(lo_pos, (int64_t)w_begin * b.window) : 0;
+    int64_t length = 0;  // of this lane's runs (count) / of the stream so far (fill)
+    const int64_t base = FILL ? b.stream_first[stream] : 0;
+    for (int w = w_begin; w < w_end; ++w) {
+        int p1 = p0;
+        if (row >= 0) p1 = w + 1 == b.n_windows ? end_pos : first_at_least(p0, (int64_t)(w + 1) * b.window);
+        const int64_t n_all = p1 - p0;
+        const int begin = p0 + (int)(n_all * part / parts), end = p0 + (int)(n_all * (part + 1) / parts);
+        p0 = p1;
+        const int n = row >= 0 ? end - begin : 0;
+        if constexpr (!FILL) {
+            length += n;
+        } else {
+            int incl = n;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const int t = __shfl_up(incl, o, kWave);
+                if (lane >= o) incl += t;
+            }
+            const int total = __shfl(incl, kWave - 1, kWave);
+            __syncthreads();
+            prefix[lane] = incl - n;
+            delta[lane] = begin - (incl - n);
+            __syncthreads();
+            for (int f = lane; f < total; f += kWave) {
+                int lo = 0, hi = kHubRowsPerWave;  // prefix[lo] <= f < prefix[hi] (prefix[kHubRowsPerWave ..] = total)
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (prefix[mid] <= f) lo = mid; else hi = mid;
+                }
+                b.stream_pos[base + length + f] = f + delta[lo];
+                b.stream_run[base + length + f] = (uint8_t)lo;
+            }
+            length += total;
+        }
+    }
+    if constexpr (!FILL) {
+        int64_t sum = length;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+        if (lane == 0) b.stream_total[stream] = (int32_t)sum;
+    } else {
+        // padding up to a whole batch: a valid position (entry 0 of the matrix), a slot number no wavefront has
+        const int64_t padded = (length + kWave - 1) / kWave * kWave;
+        for (int64_t f = length + lane; f < padded; f += kWave) {
+            b.stream_pos[base + f] = 0;
+            b.stream_run[base + f] = 255;
+        }
+    }
+}
+
+// flags of the hub rows among the split rows of the plan and of their segments; one workgroup per hub row
+__global__ void __launch_bounds__(64) hub_flags_kernel(int32_t n_long, const int32_t *__restrict__ long_rows, const int32_t *__restrict__ seg_first,
+                                                       const int32_t *__restrict__ rows, uint8_t *__restrict__ long_is_hub,
+                                                       uint8_t *__restrict__ seg_is_hub)
+{
+    const int32_t row = rows[blockIdx.x];
+    int lo = 0, hi = n_long;  // position of the row among the split rows (it is one of them)
+    while (lo < hi) {
+        const int mid = lo + ((hi - lo) >> 1);
+        if (long_rows[mid] < row) lo = mid + 1; else hi = mid;
+    }
+    if (threadIdx.x == 0) long_is_hub[lo] = 1;
+    for (int s = seg_first[lo] + threadIdx.x; s < seg_first[lo + 1]; s += blockDim.x) seg_is_hub[s] = 1;
+}
+
+__global__ void __launch_bounds__(256) row_lengths_kernel(int64_t n, const int32_t *__restrict__ rowptr, const int32_t *__restrict__ rows,
+                                                          int32_t *__restrict__ len)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) len[i] = rowptr[rows[i] + 1] - rowptr[rows[i]];
+}
+
+struct DeviceBlock {  // freed on every way out
+    void *p = nullptr;
+    ~DeviceBlock()
+    {
+        if (p) (void)hipFree(p);
+    }
+};
+
+size_t lds_bytes() { return ((size_t)kWaves * kHubRowsPerWave * kHubTile) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2); }
+
+template <typename T>
+int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st)
+{
+    const size_t shm = lds_bytes();
+    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_hub_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm));
+    dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, kHubTile), 1);
+    spmm_hub_kernel<T><<<grid, kThreads, shm, st>>>(a);
+    PLX_LAUNCH_CHECK("spmm_hub_kernel");
+    spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 128, 0, st>>>(a, static_cast<T *>(Y), ldy);
+    PLX_LAUNCH_CHECK("spmm_hub_reduce_kernel");
+    return PLX_OK;
+}
+
+}  // namespace
+
+namespace plx {
+namespace hub {
+
+size_t partial_bytes(int64_t D) { return (size_t)kHubRanges * kHubSlots * (size_t)(ceil_div(D, kHubTile) * kHubTile) * sizeof(float); }
+
+void free_hub_plan(HubPlan &hp)
+{
+    if (hp.block) (void)hipFree(hp.block);
+    hp = HubPlan();
+}
+
+int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, const int32_t *col, int32_t seg_len, int64_t n_long,
+                   int64_t n_seg, const int32_t *long_rows, const int32_t *seg_first, const std::vector<int32_t> &h_long_rows,
+                   int64_t min_entries, hipStream_t st, HubPlan &out)
+{
+    (void)M;
+    out = HubPlan();
+    if (n_long <= 0 || K <= 0 || nnz <= 0) return PLX_OK;
+
+    // lengths of the split rows, to the host
+    std::vector<int32_t> len((size_t)n_long);
+    {
+        DeviceBlock d_len;
+        PLX_HIP_CHECK(hipMalloc(&d_len.p, sizeof(int32_t) * (size_t)n_long));
+        row_lengths_kernel<<<(unsigned)ceil_div(n_long, 256), 256, 0, st>>>(n_long, rowptr, long_rows, static_cast<int32_t *>(d_len.p));
+        PLX_LAUNCH_CHECK("row_lengths_kernel");
+        PLX_HIP_CHECK(hipMemcpyAsync(len.data(), d_len.p, sizeof(int32_t) * (size_t)n_long, hipMemcpyDeviceToHost, st));
+        PLX_HIP_CHECK(hipStreamSynchronize(st));
+    }
+    // longest first (ties: lower row first); a row takes ceil(len / part_len) slots, rows are taken while slots last
+    std::vector<int32_t> order((size_t)n_long);
+    std::iota(order.begin(), order.end(), 0);
+    const size_t keep = std::min<size_t>((size_t)n_long, (size_t)kHubSlots);
+    auto longer = [&](int32_t x, int32_t y) { return len[(size_t)x] != len[(size_t)y] ? len[(size_t)x] > len[(size_t)y] : x < y; };
+    std::partial_sort(order.begin(), order.begin() + (ptrdiff_t)keep, order.end(), longer);
+    const int64_t part_len = (int64_t)seg_len * kHubPartFactor;
+    struct Slot { int32_t row, part, parts, q; int64_t size; };
+    std::vector<Slot> slots;
+    std::vector<int32_t> rows, row_slot_first{0};
+    int64_t entries = 0;
+    for (size_t i = 0; i < keep; ++i) {
+        const int32_t q = order[i];
+        const int64_t l = len[(size_t)q];
+        const int64_t parts = ceil_div(l, part_len);
+        if ((int64_t)slots.size() + parts > kHubSlots) continue;  // a shorter row may still fit
+        for (int64_t s = 0; s < parts; ++s) slots.push_back(Slot{h_long_rows[(size_t)q], (int32_t)s, (int32_t)parts, (int32_t)rows.size(), l / parts});
+        rows.push_back(h_long_rows[(size_t)q]);
+        row_slot_first.push_back((int32_t)slots.size());
+        entries += l;
+    }
+    if (rows.empty() || entries < min_entries) return PLX_OK;
+    // the slots by size, dealt over the workgroups first, then over the wavefronts of a workgroup
+    std::vector<int32_t> by_size(slots.size());
+    std::iota(by_size.begin(), by_size.end(), 0);
+    std::stable_sort(by_size.begin(), by_size.end(), [&](int32_t x, int32_t y) { return slots[(size_t)x].size > slots[(size_t)y].size; });
+    std::vector<int32_t> hub_row((size_t)kHubSlots, -1), hub_part((size_t)kHubSlots, 1 << 16), row_slots(slots.size());
+    for (size_t k = 0; k < by_size.size(); ++k) {
+        const Slot &s = slots[(size_t)by_size[k]];
+        const int32_t id = (int32_t)((k % kHubGroups) * (kWaves * kHubRowsPerWave) + ((k / kHubGroups) % kWaves) * kHubRowsPerWave +
+                                     k / (kHubGroups * kWaves));
+        hub_row[(size_t)id] = s.row;
+        hub_part[(size_t)id] = s.part | (s.parts << 16);
+        row_slots[(size_t)row_slot_first[(size_t)s.q] + (size_t)s.part] = id;
+    }
+
+    const int32_t window = kHubWindow;
+    const int32_t wpr = (int32_t)ceil_div(ceil_div(K, kHubRanges), window);
+    const int32_t n_windows = wpr * kHubRanges;
+
+    // the small tables and the stream lengths
+    const size_t n_rows = rows.size(), n_slots = slots.size();
+    auto up16 = [](size_t x) { return (x + 15) / 16 * 16; };
+    const size_t o_hub_row = 0, o_hub_part = o_hub_row + up16(sizeof(int32_t) * kHubSlots), o_rows = o_hub_part + up16(sizeof(int32_t) * kHubSlots),
+                 o_rsf = o_rows + up16(sizeof(int32_t) * n_rows), o_rs = o_rsf + up16(sizeof(int32_t) * (n_rows + 1)),
+                 o_first = o_rs + up16(sizeof(int32_t) * n_slots), o_total = o_first + up16(sizeof(int64_t) * kHubStreams),
+                 o_lflag = o_total + up16(sizeof(int32_t) * kHubStreams), o_sflag = o_lflag + up16((size_t)n_long),
+                 small_bytes = o_sflag + up16((size_t)n_seg);
+    DeviceBlock small;
+    PLX_HIP_CHECK(hipMalloc(&small.p, small_bytes));
+    char *sb = static_cast<char *>(small.p);
+    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_row, hub_row.data(), sizeof(int32_t) * kHubSlots, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_part, hub_part.data(), sizeof(int32_t) * kHubSlots, hipMemcpyHostToDevice, st));
+    BuildArgs b{};
+    b.rowptr = rowptr;
+    b.col = col;
+    b.hub_row = reinterpret_cast<const int32_t *>(sb + o_hub_row);
+    b.hub_part = reinterpret_cast<const int32_t *>(sb + o_hub_part);
+    b.window = window;
+    b.windows_per_range = wpr;
+    b.n_windows = n_windows;
+    b.stream_total = reinterpret_cast<int32_t *>(sb + o_total);
+    hub_streams_kernel<false><<<kHubStreams, 64, 0, st>>>(b);
+    PLX_LAUNCH_CHECK("hub_streams_kernel (count)");
+    std::vector<int32_t> totals((size_t)kHubStreams);
+    PLX_HIP_CHECK(hipMemcpyAsync(totals.data(), sb + o_total, sizeof(int32_t) * kHubStreams, hipMemcpyDeviceToHost, st));
+    PLX_HIP_CHECK(hipStreamSynchronize(st));
+    std::vector<int64_t> first((size_t)kHubStreams);
+    int64_t stored = 0, counted = 0;
+    for (int i = 0; i < kHubStreams; ++i) {
+        first[(size_t)i] = stored;
+        stored += ceil_div(totals[(size_t)i], kWave) * kWave;
+        counted += totals[(size_t)i];
+    }
+    PLX_REQUIRE(counted == entries, "hub plan: the streams hold %lld entries, the hub rows %lld", (long long)counted, (long long)entries);
+
+    // everything in one block: the small tables, then the streams
+    const size_t o_pos = up16(small_bytes), o_run = o_pos + up16(sizeof(int32_t) * (size_t)stored), bytes = o_run + up16((size_t)stored);
+    DeviceBlock block;
+    hipError_t e = hipMalloc(&block.p, bytes);
+    if (e != hipSuccess) return plx::fail(PLX_ERR_NOMEM, "hub plan: hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    char *bb = static_cast<char *>(block.p);
+    PLX_HIP_CHECK(hipMemcpyAsync(bb, sb, o_rows, hipMemcpyDeviceToDevice, st));  // hub_row, hub_part
+    PLX_HIP_CHECK(hipMemcpyAsync(bb + o_rows, rows.data(), sizeof(int32_t) * n_rows, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(bb + o_rsf, row_slot_first.data(), sizeof(int32_t) * (n_rows + 1), hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(bb + o_rs, row_slots.data(), sizeof(int32_t) * n_slots, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(bb + o_first, first.data(), sizeof(int64_t) * kHubStreams, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(bb + o_total, totals.data(), sizeof(int32_t) * kHubStreams, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemsetAsync(bb + o_lflag, 0, o_pos - o_lflag, st));
+    b.hub_row = reinterpret_cast<const int32_t *>(bb + o_hub_row);
+    b.hub_part = reinterpret_cast<const int32_t *>(bb + o_hub_part);
+    b.stream_first = reinterpret_cast<const int64_t *>(bb + o_first);
+    b.stream_total = nullptr;
+    b.stream_pos = reinterpret_cast<int32_t *>(bb + o_pos);
+    b.stream_run = reinterpret_cast<uint8_t *>(bb + o_run);
+    hub_streams_kernel<true><<<kHubStreams, 64, 0, st>>>(b);
+    PLX_LAUNCH_CHECK("hub_streams_kernel (fill)");
+    hub_flags_kernel<<<(unsigned)n_rows, 64, 0, st>>>((int32_t)n_long, long_rows, seg_first, reinterpret_cast<const int32_t *>(bb + o_rows),
+                                                      reinterpret_cast<uint8_t *>(bb + o_lflag), reinterpret_cast<uint8_t *>(bb + o_sflag));
+    PLX_LAUNCH_CHECK("hub_flags_kernel");
+    PLX_HIP_CHECK(hipStreamSynchronize(st));  // the host vectors above are read by the copies
+
+    out.n_rows = (int32_t)n_rows;
+    out.n_slots = (int32_t)n_slots;
+    out.entries = entries;
+    out.stored = stored;
+    out.window = window;
+    out.n_windows = n_windows;
+    out.windows_per_range = wpr;
+    out.block = block.p;
+    block.p = nullptr;
+    out.hub_row = reinterpret_cast<const int32_t *>(bb + o_hub_row);
+    out.rows = reinterpret_cast<const int32_t *>(bb + o_rows);
+    out.row_slot_first = reinterpret_cast<const int32_t *>(bb + o_rsf);
+    out.row_slots = reinterpret_cast<const int32_t *>(bb + o_rs);
+    out.stream_first = reinterpret_cast<const int64_t *>(bb + o_first);
+    out.stream_total = reinterpret_cast<const int32_t *>(bb + o_total);
+    out.stream_pos = reinterpret_cast<const int32_t *>(bb + o_pos);
+    out.stream_run = reinterpret_cast<const uint8_t *>(bb + o_run);
+    out.long_is_hub = reinterpret_cast<const uint8_t *>(bb + o_lflag);
+    out.seg_is_hub = reinterpret_cast<const uint8_t *>(bb + o_sflag);
+    out.h_rows_sorted = rows;
+    std::sort(out.h_rows_sorted.begin(), out.h_rows_sorted.end());
+    return PLX_OK;
+}
+
+int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *H, int64_t ldh, int64_t D, int64_t d_read, bool bf16,
+           int64_t row_begin, int64_t row_end, void *Y, int64_t ldy, float *partial, hipStream_t st)
+{
+    PLX_REQUIRE(hp.block != nullptr && partial != nullptr, "hub pass: no tables or no room for the partial sums");
+    PLX_REQUIRE(d_read % kHubVec == 0 && d_read <= ldh, "hub pass: readable width %lld", (long long)d_read);
+    HubArgs a{};
+    a.col = col;
+    a.val = val;
+    a.H = H;
+    a.ldh = ldh;
+    a.D = (int32_t)D;
+    a.d_read = (int32_t)d_read;
+    a.hub_row = hp.hub_row;
+    a.stream_first = hp.stream_first;
+    a.stream_total = hp.stream_total;
+    a.stream_pos = hp.stream_pos;
+    a.stream_run = hp.stream_run;
+    a.n_rows = hp.n_rows;
+    a.rows = hp.rows;
+    a.row_slot_first = hp.row_slot_first;
+    a.row_slots = hp.row_slots;
+    a.row_begin = (int32_t)row_begin;
+    a.row_end = (int32_t)row_end;
+    a.partial = partial;
+    a.ldp = ceil_div(D, kHubTile) * kHubTile;
+    return bf16 ? launch_t<uint16_t>(a, Y, ldy, st) : launch_t<float>(a, Y, ldy, st);
+}
+
+}  // namespace hub
+}  // namespace plx

@@ -128,6 +128,27 @@ class CsrMatrix:
         sliced, only on the mode."""
         check(_lib.load().plx_spmm_plan_set_slicing(self._plan, int(mode)), "plx_spmm_plan_set_slicing")
 
+    @property
+    def n_hub_rows(self) -> int:
+        """Rows taken by the hub pass (0: this matrix has no hub tables)."""
+        return int(_lib.load().plx_spmm_plan_info(self._plan, 6))
+
+    @property
+    def hub_entries(self) -> int:
+        return int(_lib.load().plx_spmm_plan_info(self._plan, 7))
+
+    def build_hub(self) -> None:
+        """Builds the tables of the hub pass whatever the library's size rule says (it builds them by itself for large
+        power-law matrices): the longest rows then walk the columns together, sharing the rows of H through L2."""
+        check(_lib.load().plx_spmm_plan_build_hub(self._plan, _stream()), "plx_spmm_plan_build_hub")
+        self._ws = None
+
+    def set_hub(self, mode: int) -> None:
+        """0 = products use the hub pass where the tables exist and the operands allow it (the default), -1 = never.
+        With and without the pass a product agrees to fp32 rounding, not bit for bit."""
+        check(_lib.load().plx_spmm_plan_set_hub(self._plan, int(mode)), "plx_spmm_plan_set_hub")
+        self._ws = None
+
     def _workspace(self, d: int):
         need = int(_lib.load().plx_spmm_workspace_bytes(self._plan, d))
         if need == 0:

@@ -1123,6 +1123,104 @@ def test_spmm_in_column_slices_agrees_bit_for_bit_with_its_one_pass_form(dtype):
     assert torch.equal(ops.spmm(auto, h), ops.spmm(plain, h))
 
 
+def _hub_matrix(seed, n=3000, pairs=40000, seg_len=16):
+    g = S.build_graph(n, "chunglu", pairs, seed=seed, device="cpu", gamma=2.1)
+    a = to_dev(g, seg_len=seg_len)
+    assert a.n_hub_rows == 0  # too small for the library to build the tables by itself
+    a.build_hub()
+    return g, a
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d", [4, 100, 128, 260, 512])
+def test_spmm_hub_pass_matches_the_oracle_and_keeps_its_bits(d, dtype):
+    say("spmm hub pass D=%d %s" % (d, dtype))
+    g, a = _hub_matrix(seed=31)
+    # split rows of more than 8 * seg_len entries take several parts; the longest rows all become hub rows
+    assert a.n_hub_rows == a.n_long_rows > 100 and g.degree_stats()["max_row_nnz"] > 8 * 16
+    assert a.hub_entries > g.nnz // 3
+    h32 = torch.randn(3000, d, generator=torch.Generator().manual_seed(d))
+    h = h32.to(dtype).to(DEV)
+    ref = oracle_spmm64(g, h.float().cpu())
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    y = ops.spmm(a, h)
+    assert rel_err(y.float().cpu(), ref) <= tol
+    assert torch.equal(ops.spmm(a, h), y)  # the order of every sum is fixed by the plan
+    assert torch.equal(ops.chunked_spmm(a, h, max_rows_per_chunk=700), y)  # row ranges run the same pass
+    a.set_hub(-1)
+    y_plain = ops.spmm(a, h)
+    a.set_hub(0)
+    assert rel_err(y_plain.float().cpu(), ref) <= tol
+    if dtype == torch.float32:
+        assert not torch.equal(y_plain, y)  # the pass was taken: hub rows are summed in another order
+        assert rel_err(y.cpu(), y_plain.cpu()) <= 2e-6
+    # the rows that are not hub rows are summed as without the pass
+    rows = torch.ones(3000, dtype=torch.bool)
+    long_rows = torch.nonzero((g.rowptr[1:] - g.rowptr[:-1]) > 16).reshape(-1)
+    rows[long_rows] = False
+    assert torch.equal(y.cpu()[rows], y_plain.cpu()[rows])
+
+
+def test_spmm_hub_pass_is_left_out_where_the_operand_does_not_suit_it():
+    say("spmm hub pass: widths and layouts it does not take")
+    g, a = _hub_matrix(seed=32)
+    for d in (47, 130 + 1):  # not a multiple of 4
+        h = torch.randn(3000, d, generator=torch.Generator().manual_seed(d)).to(DEV)
+        y = ops.spmm(a, h)
+        a.set_hub(-1)
+        assert torch.equal(ops.spmm(a, h), y)
+        a.set_hub(0)
+        assert rel_err(y.cpu(), oracle_spmm64(g, h.cpu())) <= FP32_TOL
+    # a view that starts 4 bytes into a wider matrix is not 16-byte aligned
+    wide = torch.randn(3000, 132, generator=torch.Generator().manual_seed(5)).to(DEV)
+    h = wide[:, 1:129]
+    y = ops.spmm(a, h)
+    a.set_hub(-1)
+    assert torch.equal(ops.spmm(a, h), y)
+    a.set_hub(0)
+    # a 16-byte aligned view of the same matrix is taken, and reads the view's columns only
+    h = wide[:, 4:132]
+    y = ops.spmm(a, h)
+    assert rel_err(y.cpu(), oracle_spmm64(g, h.cpu().contiguous())) <= FP32_TOL
+    a.set_hub(-1)
+    assert not torch.equal(ops.spmm(a, h), y)
+
+
+def test_spmm_hub_pass_on_transposes_few_columns_and_every_row_a_hub_row():
+    say("spmm hub pass: small and degenerate shapes")
+    # 40 rows of 300 entries over 5 columns... every row long, fewer columns than column ranges
+    gen = torch.Generator().manual_seed(3)
+    m, k = 40, 5
+    dense = torch.randn(m, k, generator=gen)
+    crow = torch.arange(0, m * k + 1, k, dtype=torch.int32)
+    col = torch.arange(k, dtype=torch.int32).repeat(m)
+    a = ops.CsrMatrix(crow.to(DEV), col.to(DEV), dense.reshape(-1).to(DEV), (m, k), 2)
+    a.build_hub()
+    assert a.n_hub_rows == m
+    h = torch.randn(k, 8, generator=gen)
+    y = ops.spmm(a, h.to(DEV)).cpu()
+    assert rel_err(y, (dense.double() @ h.double())) <= FP32_TOL
+    # the transpose of a power-law graph: columns and rows change roles, the hub rows are the popular columns
+    g = S.build_graph(3000, "chunglu", 40000, seed=33, device="cpu", gamma=2.1)
+    at = to_dev(g, transpose=True, seg_len=16)
+    at.build_hub()
+    h = torch.randn(3000, 128, generator=gen)
+    y = ops.spmm(at, h.to(DEV)).cpu()
+    assert rel_err(y, oracle_spmm64(g, h, transpose=True)) <= FP32_TOL
+    # one row far longer than a part (several slots), repeated columns allowed by CSR are not: columns are distinct here
+    k = 20000
+    crow = torch.tensor([0, k, k + 3], dtype=torch.int32)
+    col = torch.cat([torch.arange(k, dtype=torch.int32), torch.tensor([1, 7, 19999], dtype=torch.int32)])
+    val = torch.randn(k + 3, generator=gen)
+    a = ops.CsrMatrix(crow.to(DEV), col.to(DEV), val.to(DEV), (2, k), 64)
+    a.build_hub()
+    assert a.n_hub_rows == 1 and a.hub_entries == k
+    h = torch.randn(k, 64, generator=gen)
+    y = ops.spmm(a, h.to(DEV)).cpu()
+    ref = torch.stack([(val[:k, None].double() * h.double()).sum(0), (val[k:, None].double() * h[[1, 7, 19999]].double()).sum(0)])
+    assert rel_err(y, ref) <= FP32_TOL
+
+
 def test_spmm_staging_with_bf16_rows_and_dense_reuse():
     say("spmm: staging of bf16 rows and of 2,408-byte fp32 rows under heavy reuse")
     g = S.build_graph(2000, "uniform", 0, seed=11, device="cpu", exact_pairs=100000)  # about 100 entries per column of H
