@@ -75,6 +75,7 @@ SIGNATURES = {
 # include/plexus_hip_diag.h: measurement probes, not part of the path
 DIAG_SIGNATURES = {
     "plx_diag_random_gather_f32": (C.c_int, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_i64), _vp, _vp]),
+    "plx_diag_spmm_parts_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, C.c_size_t, C.c_int, _vp]),
 }
 
 PLX_GEMM_RELU = 1

@@ -634,7 +634,8 @@ size_t hub_workspace_bytes(const plx_spmm_plan *plan, int64_t D, int64_t elem)
 // it lies; same values in the same order, so the same result)
 template <typename T>
 int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const T *H, int64_t ldh,
-              int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream, bool may_stage = true)
+              int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream, bool may_stage = true,
+              int parts = 3)
 {
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
     PLX_REQUIRE(row_begin >= 0 && row_begin <= row_end && row_end <= plan->M, "spmm: row range [%lld, %lld) outside [0, %lld)",
@@ -707,7 +708,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     }
     float *hub_partial = reinterpret_cast<float *>(ws_base + seg_bytes);  // seg_bytes is a multiple of 16
     auto hub_pass = [&]() -> int {
-        if (!use_hub) return PLX_OK;
+        if (!use_hub || !(parts & 2)) return PLX_OK;
         return plx::hub::launch(plan->hub, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st);
     };
 
@@ -790,6 +791,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
 
     dim3 grid((unsigned)plx::ceil_div(tasks, 4), (unsigned)tiles, 1);
     int rc = -1;
+    if (!(parts & 1)) return hub_pass();  // measurement of the hub pass alone
     if (sliced) {  // one pass, summed in the order of the sliced product
         switch (vec) {
             case 1: rc = launch_chained<T, T, 1>(a, lpr, nacc, grid, st); break;
@@ -1080,6 +1082,14 @@ int plx_spmm_csr_f32_static(const plx_spmm_plan *plan, const float *val, const f
     // every partial row is written in full (columns < D) by its segment task before the reduction reads it, so nothing
     // of an earlier call has to be cleared
     return spmm_impl<float>(plan, 0, plan->M, val, H, ldh, D, Y, ldy, ptr, kStaticScratchBytes, stream, /*may_stage=*/false);
+}
+
+int plx_diag_spmm_parts_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y, int64_t ldy,
+                            void *workspace, size_t workspace_bytes, int parts, void *stream)
+{
+    PLX_REQUIRE(parts >= 1 && parts <= 3, "diag_spmm_parts: parts must be 1 (row kernel), 2 (hub pass) or 3 (both)");
+    PLX_REQUIRE(plan != nullptr, "diag_spmm_parts: plan is NULL");
+    return spmm_impl<float>(plan, 0, plan->M, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream, true, parts);
 }
 
 int plx_diag_random_gather_f32(const float *table, int64_t rows, int64_t ld, int64_t D, int64_t n_gathers, int64_t *gathers_done,

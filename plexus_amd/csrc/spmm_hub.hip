@@ -19,7 +19,10 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <functional>
 #include <numeric>
+#include <queue>
+#include <utility>
 #include <type_traits>
 #include <vector>
 
@@ -255,28 +258,65 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
     }
 }
 
-// Y[hub row] = sum over the row's slots (its parts, in order) and, per slot, over the ranges in range order
+// Y[hub row] = sum of the partial sums of the row's slots (its parts, in order) over the ranges (in range order).
+// A workgroup owns a hub row: 8 chains x 32 lanes, each lane a float4.  Chain c adds partial sums c, c + 8, ... of
+// the (slot, range) list in order; the 8 chain sums are then added in chain order, so the summation order is fixed.
 template <typename TOUT>
-__global__ void __launch_bounds__(128) spmm_hub_reduce_kernel(const HubArgs p, TOUT *__restrict__ Y, int64_t ldy)
+__global__ void __launch_bounds__(256) spmm_hub_reduce_kernel(const HubArgs p, TOUT *__restrict__ Y, int64_t ldy)
 {
+    __shared__ float4 part[8][32];
     const int q = blockIdx.x;
     const int row = p.rows[q];
     if (row < p.row_begin || row >= p.row_end) return;
-    const int s0 = p.row_slot_first[q], s1 = p.row_slot_first[q + 1];
-    for (int d = threadIdx.x; d < p.D; d += blockDim.x) {
-        float s = 0.f;
-        for (int i = s0; i < s1; ++i) {
-            const int slot = p.row_slots[i];
-#pragma unroll
-            for (int x = 0; x < kHubRanges; ++x) s += p.partial[((int64_t)x * kHubSlots + slot) * p.ldp + d];
+    const int s0 = p.row_slot_first[q], n = (p.row_slot_first[q + 1] - s0) * kHubRanges;
+    const int chain = threadIdx.x >> 5, l = threadIdx.x & 31;
+    for (int d0 = 0; d0 < p.D; d0 += kHubTile) {
+        const int d = d0 + l * 4;  // ldp is a multiple of kHubTile: the float4 at d lies inside the padded partial row
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        auto at = [&](int j) {
+            const int slot = p.row_slots[s0 + j / kHubRanges], x = j % kHubRanges;
+            return *reinterpret_cast<const float4 *>(p.partial + ((int64_t)x * kHubSlots + slot) * p.ldp + d);
+        };
+        auto add = [&](const float4 &t) {
+            acc.x += t.x;
+            acc.y += t.y;
+            acc.z += t.z;
+            acc.w += t.w;
+        };
+        int j = chain;
+        for (; j + 24 < n; j += 32) {  // four loads in flight, added in the order of the list
+            const float4 t0 = at(j), t1 = at(j + 8), t2 = at(j + 16), t3 = at(j + 24);
+            add(t0);
+            add(t1);
+            add(t2);
+            add(t3);
         }
-        if constexpr (sizeof(TOUT) == 4) {
-            Y[(int64_t)row * ldy + d] = s;
-        } else {
-            uint32_t u = __float_as_uint(s);
-            if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;
-            else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-            Y[(int64_t)row * ldy + d] = (uint16_t)u;
+        for (; j < n; j += 8) add(at(j));
+        __syncthreads();  // the chain sums of the tile before have been read
+        part[chain][l] = acc;
+        __syncthreads();
+        if (chain == 0) {
+            float4 s = part[0][l];
+#pragma unroll
+            for (int c = 1; c < 8; ++c) {
+                s.x += part[c][l].x;
+                s.y += part[c][l].y;
+                s.z += part[c][l].z;
+                s.w += part[c][l].w;
+            }
+            const float v[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (d + e >= p.D) break;
+                if constexpr (sizeof(TOUT) == 4) {
+                    Y[(int64_t)row * ldy + d + e] = v[e];
+                } else {
+                    uint32_t u = __float_as_uint(v[e]);
+                    if ((u & 0x7fffffffu) > 0x7f800000u) u = (u >> 16) | 0x40u;
+                    else u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+                    Y[(int64_t)row * ldy + d + e] = (uint16_t)u;
+                }
+            }
         }
     }
 }
@@ -415,7 +455,7 @@ int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st)
     dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, kHubTile), 1);
     spmm_hub_kernel<T><<<grid, kThreads, shm, st>>>(a);
     PLX_LAUNCH_CHECK("spmm_hub_kernel");
-    spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 128, 0, st>>>(a, static_cast<T *>(Y), ldy);
+    spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 256, 0, st>>>(a, static_cast<T *>(Y), ldy);
     PLX_LAUNCH_CHECK("spmm_hub_reduce_kernel");
     return PLX_OK;
 }
@@ -473,18 +513,32 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
         entries += l;
     }
     if (rows.empty() || entries < min_entries) return PLX_OK;
-    // the slots by size, dealt over the workgroups first, then over the wavefronts of a workgroup
+    // The slots go to the wavefronts largest first, each to the wavefront with the fewest entries so far that still has
+    // room: wavefronts with equal loads pass through the windows side by side, which is what keeps a window's rows of H
+    // in L2 while they are shared (a wavefront 5 % short of the others ends the pass four windows ahead of them).
     std::vector<int32_t> by_size(slots.size());
     std::iota(by_size.begin(), by_size.end(), 0);
     std::stable_sort(by_size.begin(), by_size.end(), [&](int32_t x, int32_t y) { return slots[(size_t)x].size > slots[(size_t)y].size; });
     std::vector<int32_t> hub_row((size_t)kHubSlots, -1), hub_part((size_t)kHubSlots, 1 << 16), row_slots(slots.size());
-    for (size_t k = 0; k < by_size.size(); ++k) {
-        const Slot &s = slots[(size_t)by_size[k]];
-        const int32_t id = (int32_t)((k % kHubGroups) * (kWaves * kHubRowsPerWave) + ((k / kHubGroups) % kWaves) * kHubRowsPerWave +
-                                     k / (kHubGroups * kWaves));
-        hub_row[(size_t)id] = s.row;
-        hub_part[(size_t)id] = s.part | (s.parts << 16);
-        row_slots[(size_t)row_slot_first[(size_t)s.q] + (size_t)s.part] = id;
+    {
+        constexpr int kBins = kHubGroups * kWaves;
+        using Bin = std::pair<int64_t, int32_t>;  // (entries, wavefront): the least loaded first, ties by number
+        std::priority_queue<Bin, std::vector<Bin>, std::greater<Bin>> bins;
+        // numbered so that consecutive wavefronts lie in different workgroups: few slots then spread over the chip
+        for (int32_t b = 0; b < kBins; ++b) bins.push(Bin{0, b});
+        std::vector<int32_t> held((size_t)kBins, 0);
+        for (size_t k = 0; k < by_size.size(); ++k) {
+            const Slot &sl = slots[(size_t)by_size[k]];
+            Bin bin = bins.top();
+            bins.pop();
+            const int32_t b = bin.second, group = b % kHubGroups, wave = b / kHubGroups;
+            const int32_t id = (group * kWaves + wave) * kHubRowsPerWave + held[(size_t)b];
+            hub_row[(size_t)id] = sl.row;
+            hub_part[(size_t)id] = sl.part | (sl.parts << 16);
+            row_slots[(size_t)row_slot_first[(size_t)sl.q] + (size_t)sl.part] = id;
+            bin.first += sl.size;
+            if (++held[(size_t)b] < kHubRowsPerWave) bins.push(bin);
+        }
     }
 
     const int32_t window = kHubWindow;
