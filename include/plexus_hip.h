@@ -134,7 +134,8 @@ int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
  * of a hub row.  plx_spmm_plan_create builds them by itself where it expects a gain: short rows on average (fewer
  * than 128 entries, the shapes that do not take column slices), 512-byte rows of H beyond 128 MB in total, an eighth
  * of the entries in hub rows.  plx_spmm_plan_build_hub builds them for any plan with split rows (synchronises
- * `stream`).  A product uses the pass when the tables exist, the mode allows it, the shape is not a sliced one, H
+ * `stream`).  A product uses the pass when the tables exist, the mode allows it, the shape is not a sliced one, a row
+ * of H holds at least 512 bytes in 128 columns (256 where a hub row has four or more entries per window on average), H
  * as passed spans less than 4 GiB and its base, row pitch and width are multiples of 4 elements; a row range runs the
  * whole pass if it holds a hub row.  The order of every sum is fixed by the plan: the same operands give the same bits
  * on every call and in every row range, but not the bits of a product without the pass (the two agree to fp32

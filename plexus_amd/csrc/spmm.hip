@@ -624,9 +624,17 @@ int64_t wanted_stage_ld(const plx_spmm_plan *plan, int64_t D, int64_t elem, uint
 
 // room for the partial sums of the hub pass, or 0 when this plan and width do not use it (column slices and the hub
 // pass answer different shapes of matrix; a product takes one or the other)
+// The pass saves memory traffic in proportion to the bytes of a row of H and costs instructions per entry and per change
+// of sum, so narrow rows do not repay it: measured on the 2.45 M-node power-law graph (7.4 entries per slot and window)
+// and on a 4.19 M-node R-MAT block (3 per slot and window), fp32: 512-byte rows 7.6 -> 6.0 and 4.1 -> 3.5 ms, 256-byte
+// rows 3.6 -> 3.1 and 2.3 -> 2.4 ms, 128-byte rows 2.3 -> 2.5 and 1.8 -> 2.1 ms; bf16 rows count by the 256 bytes that the
+// 128 columns of a tile hold (256 columns: 7.3 -> 6.7 and 4.2 -> 4.3 ms).  The rule looks at the plan and the width only,
+// so a whole product and its row ranges choose alike.
 size_t hub_workspace_bytes(const plx_spmm_plan *plan, int64_t D, int64_t elem)
 {
     if (plan->hub.block == nullptr || plan->hub_mode < 0 || sliced_plan(plan, D, elem)) return 0;
+    const int64_t tile_bytes = std::min<int64_t>(D, plx::hub::kHubTile) * elem;  // of a row of H, per load of the pass
+    if (tile_bytes < 256 || (tile_bytes < 512 && plan->hub.mean_run < 4.0)) return 0;
     return plx::hub::partial_bytes(D);
 }
 

@@ -30,6 +30,7 @@ struct HubPlan {
     int32_t n_slots = 0;   // slots in use
     int64_t entries = 0;   // entries of A in hub rows
     int64_t stored = 0;    // entries of the streams, padding included
+    double mean_run = 0;   // entries per (slot, window): how long a wavefront adds into one sum before it changes
     int32_t window = 0, n_windows = 0, windows_per_range = 0;
     void *block = nullptr;         // one device allocation behind every pointer below
     const int32_t *hub_row = nullptr;         // [kHubSlots] row of a slot, -1 for an empty slot

@@ -61,13 +61,23 @@ struct HubArgs {
 template <typename T, int VEC>
 __device__ __forceinline__ void load_vec(const T *p, float (&o)[VEC])
 {
-    static_assert(VEC == 4, "four elements per lane");
     if constexpr (sizeof(T) == 4) {
+        static_assert(VEC == 4, "16 bytes per lane");
         const float4 t = *reinterpret_cast<const float4 *>(p);
         o[0] = t.x;
         o[1] = t.y;
         o[2] = t.z;
         o[3] = t.w;
+    } else if constexpr (VEC == 8) {
+        const uint4 t = *reinterpret_cast<const uint4 *>(p);
+        o[0] = __uint_as_float(t.x << 16);
+        o[1] = __uint_as_float(t.x & 0xffff0000u);
+        o[2] = __uint_as_float(t.y << 16);
+        o[3] = __uint_as_float(t.y & 0xffff0000u);
+        o[4] = __uint_as_float(t.z << 16);
+        o[5] = __uint_as_float(t.z & 0xffff0000u);
+        o[6] = __uint_as_float(t.w << 16);
+        o[7] = __uint_as_float(t.w & 0xffff0000u);
     } else {
         const uint2 t = *reinterpret_cast<const uint2 *>(p);
         o[0] = __uint_as_float(t.x << 16);
@@ -82,26 +92,29 @@ __device__ __forceinline__ void load_vec(const T *p, float (&o)[VEC])
 // to whole batches of 64.  A batch moves through four stages, one per turn of the loop, so that no load is waited for
 // in the turn that issues it: positions and slots (coalesced) -> column and value of every entry (gathered) -> byte
 // offset of the row of H and value into LDS, run boundaries as a bit mask -> rows of H.  The vector memory pipeline
-// takes as long for a 64-lane load of 8 bytes per lane as for one of 16, so a row of H is read by half a wavefront,
-// 16 bytes per lane: lanes 0-31 go through entries 0-31 of the batch and lanes 32-63 through entries 32-63, U steps
-// at a time, the loads of one set of steps in flight while the set before is added up.  Every turn issues the same
+// takes as long for a 64-lane load of 4 or 8 bytes per lane as for one of 16, so a row of H (a tile of LPR * VEC
+// columns of it) is read by LPR lanes, 16 bytes per lane where the rows allow it, and the 64 / LPR lane groups go
+// through different entries: group g through entries g * LPR ... of the batch, one per step, U steps at a time, the
+// loads of one set of steps in flight while the set before is added up.  Every turn issues the same
 // loads whatever it finds (past the end of the stream they repeat its last batch), so the counter of outstanding
 // loads the hardware waits on has a fixed meaning.
-template <typename T>
+template <typename T, int VEC, int LPR>
 __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    constexpr int VEC = kHubVec;
-    constexpr int TW = kHubTile;  // columns of H covered by a wavefront
-    constexpr int U = PLX_HUB_U;  // steps (two entries each) per set of loads
-    constexpr int kHalf = kWave / 2;
-    static_assert(kHalf == 4 * U, "the 32 steps of a batch are four sets");
+    constexpr int TW = LPR * VEC;   // columns of H covered by a wavefront
+    constexpr int G = kWave / LPR;  // lane groups: group g goes through entries g * STEPS ... of a batch, one per step
+    constexpr int STEPS = kWave / G;
+    constexpr int U = PLX_HUB_U;    // steps (G entries each) per set of loads
+    constexpr int SETS = STEPS / U;
+    static_assert(SETS == 2 || SETS == 4, "the steps of a batch are two or four sets");
+    static_assert(VEC == 4 || VEC == 8, "a lane reads 4 or 8 elements");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    const int half = lane >> 5;
+    const int grp = lane / LPR;
     const int range = blockIdx.x % kHubRanges;  // workgroups go to the XCDs in turn
     const int group = blockIdx.x / kHubRanges;
-    const int dl = (lane & (kHalf - 1)) * VEC;  // this lane's columns inside the tile
+    const int dl = (lane % LPR) * VEC;  // this lane's columns inside the tile
     const int d0 = blockIdx.y * TW + dl;
     // a lane whose columns lie past the readable width gathers the first columns instead; its sums are never stored
     const bool ok = d0 + VEC <= p.d_read;
@@ -138,20 +151,18 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
             y.run = x.run;
             return y;
         };
-        int carry_lo = -1, carry_hi = -1;  // slots of entries 31 and 63 of the batch before: where the two halves stand
+        int carry = -1;  // slot of the last entry this lane's group had in the batch before: where the group stands
         auto ready = [&](const Read &y, int k, int slot) {
             Ready z;
             uint2 *dst = ring + slot * kWave;
             dst[lane] = make_uint2((uint32_t)y.c * row_bytes, __float_as_uint(y.v));
             int before = __shfl_up(y.run, 1, kWave);
-            if (lane == 0) before = carry_lo;
-            if (lane == kHalf) before = carry_hi;
+            if (lane % STEPS == 0) before = carry;
             z.left = min(max(total - k * kWave, 0), kWave);
             z.starts = __ballot(y.run != before && lane < z.left);
-            carry_lo = __builtin_amdgcn_readlane(y.run, kHalf - 1);
-            carry_hi = __builtin_amdgcn_readlane(y.run, kWave - 1);
+            carry = __shfl(y.run, grp * STEPS + STEPS - 1, kWave);
             z.run = y.run;
-            z.mine = dst + half * kHalf;
+            z.mine = dst + grp * STEPS;
             plx::wave_lds_fence();
             return z;
         };
@@ -159,58 +170,61 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
         auto fetch = [&](const Ready &z, int g, Rows &r) {
 #pragma unroll
             for (int u = 0; u < U; u += 2) {
-                const uint4 e = *reinterpret_cast<const uint4 *>(z.mine + g * U + u);  // two entries of this half
+                const uint4 e = *reinterpret_cast<const uint4 *>(z.mine + g * U + u);  // two entries of this group
                 r.v[u] = __uint_as_float(e.y);
                 r.v[u + 1] = __uint_as_float(e.w);
                 load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.x + lane_off)), r.h[u]);
                 load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.z + lane_off)), r.h[u + 1]);
             }
         };
-        int cur = -1;  // the slot this half is summing
+        int cur = -1;  // the slot this group is summing
         float sum[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) sum[k] = 0.f;
         // Products are summed in registers while the slot stays the same and added to the slot's sum in LDS when it
-        // changes; the two halves may hold the same slot, so they add to LDS one after the other.
+        // changes; several groups may hold the same slot, so they add to LDS one after the other.
         auto flush = [&](int run) {
             if (cur >= 0) {
-                float4 t = *reinterpret_cast<float4 *>(acc + cur * TW + dl);
-                t.x += sum[0];
-                t.y += sum[1];
-                t.z += sum[2];
-                t.w += sum[3];
-                *reinterpret_cast<float4 *>(acc + cur * TW + dl) = t;
+#pragma unroll
+                for (int k = 0; k < VEC; k += 4) {
+                    float4 t = *reinterpret_cast<float4 *>(acc + cur * TW + dl + k);
+                    t.x += sum[k];
+                    t.y += sum[k + 1];
+                    t.z += sum[k + 2];
+                    t.w += sum[k + 3];
+                    *reinterpret_cast<float4 *>(acc + cur * TW + dl + k) = t;
+                }
             }
 #pragma unroll
             for (int k = 0; k < VEC; ++k) sum[k] = 0.f;
             cur = run;
         };
-        auto consume = [&](const Ready &z, int g, const Rows &r, auto checked) {
+        uint64_t every_group = 0;  // bit g * STEPS for every group g
+#pragma unroll
+        for (int g = 0; g < G; ++g) every_group |= 1ull << (g * STEPS);
+        auto consume = [&](const Ready &z, int s, const Rows &r, auto checked) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int i = g * U + u;
-                const bool lo = (z.starts >> i) & 1, hi = (z.starts >> (kHalf + i)) & 1;
-                if (lo | hi) {
-                    if (lo) {
-                        const int run = __builtin_amdgcn_readlane(z.run, i);
-                        if (half == 0) flush(run);
-                        plx::wave_lds_fence();
-                    }
-                    if (hi) {
-                        const int run = __builtin_amdgcn_readlane(z.run, kHalf + i);
-                        if (half == 1) flush(run);
-                        plx::wave_lds_fence();
+                const int i = s * U + u;
+                if ((z.starts >> i) & every_group) {
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        if ((z.starts >> (g * STEPS + i)) & 1) {
+                            const int run = __builtin_amdgcn_readlane(z.run, g * STEPS + i);
+                            if (grp == g) flush(run);
+                            plx::wave_lds_fence();
+                        }
                     }
                 }
-                if (!decltype(checked)::value || half * kHalf + i < z.left) {
+                if (!decltype(checked)::value || grp * STEPS + i < z.left) {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) sum[k] = fmaf(r.v[u], r.h[u][k], sum[k]);
                 }
             }
         };
-        auto add_up = [&](const Ready &z, int g, const Rows &r) {
-            if (z.left == kWave) consume(z, g, r, std::false_type{});
-            else consume(z, g, r, std::true_type{});
+        auto add_up = [&](const Ready &z, int s, const Rows &r) {
+            if (z.left == kWave) consume(z, s, r, std::false_type{});
+            else consume(z, s, r, std::true_type{});
         };
 
         Rows ra, rb;
@@ -225,14 +239,21 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
             const Ready after = ready(rd, k + 2, s_free);
             rd = read(li);
             li = list(k + 4);
-            fetch(now, 1, rb);
-            add_up(now, 0, ra);
-            fetch(now, 2, ra);
-            add_up(now, 1, rb);
-            fetch(now, 3, rb);
-            add_up(now, 2, ra);
-            fetch(next, 0, ra);
-            add_up(now, 3, rb);
+            if constexpr (SETS == 4) {
+                fetch(now, 1, rb);
+                add_up(now, 0, ra);
+                fetch(now, 2, ra);
+                add_up(now, 1, rb);
+                fetch(now, 3, rb);
+                add_up(now, 2, ra);
+                fetch(next, 0, ra);
+                add_up(now, 3, rb);
+            } else {
+                fetch(now, 1, rb);
+                add_up(now, 0, ra);
+                fetch(next, 0, ra);
+                add_up(now, 1, rb);
+            }
             now = next;
             next = after;
             const int t = s_now;
@@ -240,14 +261,15 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
             s_next = s_free;
             s_free = t;
         }
-        if (half == 0) flush(-1);
-        plx::wave_lds_fence();
-        if (half == 1) flush(-1);
-        plx::wave_lds_fence();
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (grp == g) flush(-1);
+            plx::wave_lds_fence();
+        }
     }
 
     // the sums of this range: P[range][slot][ldp]
-    if (half == 0 && ok) {
+    if (grp == 0 && ok) {
         for (int r = 0; r < kHubRowsPerWave; ++r) {
             if (p.hub_row[slot0 + r] < 0) continue;
             float *dst = p.partial + ((int64_t)range * kHubSlots + slot0 + r) * p.ldp + blockIdx.y * TW + dl;
@@ -445,15 +467,15 @@ struct DeviceBlock {  // freed on every way out
     }
 };
 
-size_t lds_bytes() { return ((size_t)kWaves * kHubRowsPerWave * kHubTile) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2); }
-
-template <typename T>
+template <typename T, int VEC, int LPR>
 int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st)
 {
-    const size_t shm = lds_bytes();
-    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_hub_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm));
-    dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, kHubTile), 1);
-    spmm_hub_kernel<T><<<grid, kThreads, shm, st>>>(a);
+    constexpr int TW = LPR * VEC;
+    const size_t shm = ((size_t)kWaves * kHubRowsPerWave * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2);
+    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)shm));
+    dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, TW), 1);
+    spmm_hub_kernel<T, VEC, LPR><<<grid, kThreads, shm, st>>>(a);
     PLX_LAUNCH_CHECK("spmm_hub_kernel");
     spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 256, 0, st>>>(a, static_cast<T *>(Y), ldy);
     PLX_LAUNCH_CHECK("spmm_hub_reduce_kernel");
@@ -610,6 +632,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     out.n_rows = (int32_t)n_rows;
     out.n_slots = (int32_t)n_slots;
     out.entries = entries;
+    out.mean_run = (double)entries / ((double)n_slots * (double)n_windows);
     out.stored = stored;
     out.window = window;
     out.n_windows = n_windows;
@@ -655,8 +678,11 @@ int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *
     a.row_begin = (int32_t)row_begin;
     a.row_end = (int32_t)row_end;
     a.partial = partial;
-    a.ldp = ceil_div(D, kHubTile) * kHubTile;
-    return bf16 ? launch_t<uint16_t>(a, Y, ldy, st) : launch_t<float>(a, Y, ldy, st);
+    a.ldp = ceil_div(D, kHubTile) * kHubTile;  // every kernel's tile divides kHubTile
+    // fp32 rows of at most 256 bytes are read by a quarter of a wavefront, four entries per load instruction
+    // (bf16 rows read 16 bytes per lane by a quarter of a wavefront were measured too: no faster than 8 bytes by a half)
+    if (!bf16) return D <= 64 ? launch_t<float, 4, 16>(a, Y, ldy, st) : launch_t<float, 4, 32>(a, Y, ldy, st);
+    return launch_t<uint16_t, 4, 32>(a, Y, ldy, st);
 }
 
 }  // namespace hub
