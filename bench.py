@@ -49,6 +49,8 @@ def measured_spmm_traffic(n, nnz, d):
         return None, None
     source = {"profile": SPMM_TRAFFIC_PROFILE, "commit": commit.group(1) if commit else None,
               "kernel": kernel.group(1).strip() if kernel else None}
+    hub = re.search(r"^\s*hub_traffic_bytes_per_launch\[%d,%d,%d\]\s*=\s*([0-9.eE+]+)" % (n, nnz, d), text, flags=re.M)
+    source["hub_pass_traffic"] = float(hub.group(1)) if hub else None
     return float(m.group(1)), source
 
 
@@ -459,6 +461,8 @@ def main():
                                 "alg_bytes": rows_bytes, "alg_GBps": rows_bytes / rows_ms / 1e6},
                  "hub_pass": {"kernel": "spmm_hub_kernel", "ms": hub_ms, "entries": hub_nnz, "rows": hub_rows,
                               "alg_bytes": hub_bytes, "alg_GBps": hub_bytes / hub_ms / 1e6}}
+        src = measured_spmm_traffic(n, nnz, d_main)[1]
+        parts["hub_pass"]["traffic"] = src["hub_pass_traffic"] if src else None
         print("# spmm D=%d in parts: row kernel %.3f ms (%.1f %% of the entries), hub pass %.3f ms (%d rows, %.1f %% of the entries)"
               % (d_main, rows_ms, 100.0 * (nnz - hub_nnz) / nnz, hub_ms, hub_rows, 100.0 * hub_nnz / nnz), file=sys.stderr, flush=True)
         del h, out
