@@ -21,6 +21,9 @@ constexpr int kHubTile = 32 * kHubVec;
 constexpr int kHubSlots = kHubGroups * kWaves * kHubRowsPerWave;  // 9,216 slots: a hub row takes one per part
 constexpr int kHubStreams = kHubRanges * kHubGroups * kWaves;     // one per wavefront of the pass
 constexpr int kHubWindow = 4096;     // columns per window: 2 MB of 512-byte rows, half of an XCD's L2
+constexpr int kHubPace = 1;          // windows a wavefront may run ahead of the slowest of its workgroup (measured, hub pass of the
+                                     // 2.45 M-node graph: none 1.36 ms and 6.1 GB fetched, 0 / 1 / 2 / 3: 1.35 / 1.27 / 1.30 / 1.31 ms, 1: 3.9 GB)
+constexpr int kHubMaxPolls = 4096;   // of a wavefront waiting for the others, then it goes on regardless
 constexpr int kHubPartFactor = 8;    // a hub row is cut into parts of at most kHubPartFactor * seg_len entries
 constexpr int64_t kHubMaxBytes = 1ll << 32;  // rows of H are addressed with 32-bit byte offsets
 
@@ -41,6 +44,7 @@ struct HubPlan {
     const int32_t *stream_total = nullptr;    // [kHubStreams] entries of the stream (stored padded to whole batches of 64)
     const int32_t *stream_pos = nullptr;      // [stored] position of an entry in the CSR arrays
     const uint8_t *stream_run = nullptr;      // [stored] its slot among the wavefront's kHubRowsPerWave
+    const int32_t *stream_mark = nullptr;     // [kHubStreams][windows_per_range] batch of the stream in which a window begins
     const uint8_t *long_is_hub = nullptr;     // [n_long] flags over the plan's split rows
     const uint8_t *seg_is_hub = nullptr;      // [n_seg] flags over their segments
     std::vector<int32_t> h_rows_sorted;       // hub rows in ascending order (host), to intersect with a row range

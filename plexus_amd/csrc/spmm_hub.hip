@@ -49,6 +49,9 @@ struct HubArgs {
     const int32_t *stream_total;
     const int32_t *stream_pos;
     const uint8_t *stream_run;
+    const int32_t *stream_mark;  // [streams][windows_per_range] batch in which a window of the range begins
+    int32_t windows_per_range;
+    int32_t pace;                // windows a wavefront may be ahead of the slowest of its workgroup (< 0: no pacing)
     int32_t n_rows;
     const int32_t *rows;
     const int32_t *row_slot_first;
@@ -123,6 +126,10 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
     float *acc = lds + (size_t)wave * kHubRowsPerWave * TW;  // [kHubRowsPerWave][TW], this wavefront's sums
     uint2 *ring = reinterpret_cast<uint2 *>(lds + (size_t)kWaves * kHubRowsPerWave * TW) + wave * 3 * kWave;  // [3][64] (offset, value)
     for (int i = lane; i < kHubRowsPerWave * TW; i += kWave) acc[i] = 0.f;
+    // window each wavefront of the workgroup is in (pacing, below)
+    int *progress = reinterpret_cast<int *>(reinterpret_cast<uint2 *>(lds + (size_t)kWaves * kHubRowsPerWave * TW) + kWaves * 3 * kWave);
+    if (lane == 0) progress[wave] = 0;
+    __syncthreads();
 
     const int slot0 = (group * kWaves + wave) * kHubRowsPerWave;
     const int stream = (range * kHubGroups + group) * kWaves + wave;
@@ -235,7 +242,31 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
         Read rd = read(l2);
         Listed li = list(3);
         fetch(now, 0, ra);
+        // Pacing: the rows of H of a window stay in L2 only while the wavefronts that share them are in the same few
+        // windows.  Left alone they drift apart by the random walk of their entry counts; here a wavefront that enters a
+        // window waits until the slowest wavefront of its workgroup is at most `pace` windows behind.  The wait reads
+        // LDS only, ends when the others move on (they never wait for a wavefront ahead of them, and a wavefront that has
+        // finished counts as far ahead), and is cut off after a fixed number of polls whatever happens.
+        const int32_t *marks = p.stream_mark + (int64_t)stream * p.windows_per_range;
+        int w_next = 1;
+        int mark_next = p.pace >= 0 && w_next < p.windows_per_range ? marks[w_next] : 0x7fffffff;
         for (int k = 0; k < nb; ++k) {
+            if (k >= mark_next) {
+                while (w_next < p.windows_per_range && k >= mark_next) {
+                    ++w_next;
+                    mark_next = w_next < p.windows_per_range ? marks[w_next] : 0x7fffffff;
+                }
+                const int here = w_next - 1;
+                if (lane == 0) __hip_atomic_store(&progress[wave], here, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                for (int polls = 0; polls < kHubMaxPolls; ++polls) {
+                    int slowest = 0x7fffffff;
+#pragma unroll
+                    for (int x = 0; x < kWaves; ++x)
+                        slowest = min(slowest, __hip_atomic_load(&progress[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+                    if (slowest >= here - p.pace) break;
+                    __builtin_amdgcn_s_sleep(8);
+                }
+            }
             const Ready after = ready(rd, k + 2, s_free);
             rd = read(li);
             li = list(k + 4);
@@ -267,6 +298,8 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
             plx::wave_lds_fence();
         }
     }
+
+    if (lane == 0) __hip_atomic_store(&progress[wave], 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // done: nobody waits for this wavefront
 
     // the sums of this range: P[range][slot][ldp]
     if (grp == 0 && ok) {
@@ -354,6 +387,7 @@ struct BuildArgs {
     int32_t *stream_total;        // count
     int32_t *stream_pos;          // fill
     uint8_t *stream_run;          // fill
+    int32_t *stream_mark;         // fill
 };
 
 // One wavefront per stream.  Lane l follows slot l of the wavefront through the windows of the range: the entries of
@@ -399,6 +433,7 @@ __global__ void __launch_bounds__(64) hub_streams_kernel(const BuildArgs b)
         if constexpr (!FILL) {
             length += n;
         } else {
+            if (lane == 0) b.stream_mark[(int64_t)stream * b.windows_per_range + (w - w_begin)] = (int32_t)(length / kWave);
             int incl = n;
 #pragma unroll
             for (int o = 1; o < kWave; o <<= 1) {
@@ -428,6 +463,7 @@ __global__ void __launch_bounds__(64) hub_streams_kernel(const BuildArgs b)
         for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
         if (lane == 0) b.stream_total[stream] = (int32_t)sum;
     } else {
+        for (int w = w_end - w_begin + lane; w < b.windows_per_range; w += kWave) b.stream_mark[(int64_t)stream * b.windows_per_range + w] = 0x7fffffff;
         // padding up to a whole batch: a valid position (entry 0 of the matrix), a slot number no wavefront has
         const int64_t padded = (length + kWave - 1) / kWave * kWave;
         for (int64_t f = length + lane; f < padded; f += kWave) {
@@ -471,7 +507,7 @@ template <typename T, int VEC, int LPR>
 int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st)
 {
     constexpr int TW = LPR * VEC;
-    const size_t shm = ((size_t)kWaves * kHubRowsPerWave * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2);
+    const size_t shm = ((size_t)kWaves * kHubRowsPerWave * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2) + kWaves * sizeof(int);
     PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       (int)shm));
     dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, TW), 1);
@@ -573,7 +609,8 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     const size_t o_hub_row = 0, o_hub_part = o_hub_row + up16(sizeof(int32_t) * kHubSlots), o_rows = o_hub_part + up16(sizeof(int32_t) * kHubSlots),
                  o_rsf = o_rows + up16(sizeof(int32_t) * n_rows), o_rs = o_rsf + up16(sizeof(int32_t) * (n_rows + 1)),
                  o_first = o_rs + up16(sizeof(int32_t) * n_slots), o_total = o_first + up16(sizeof(int64_t) * kHubStreams),
-                 o_lflag = o_total + up16(sizeof(int32_t) * kHubStreams), o_sflag = o_lflag + up16((size_t)n_long),
+                 o_mark = o_total + up16(sizeof(int32_t) * kHubStreams), o_lflag = o_mark + up16(sizeof(int32_t) * (size_t)kHubStreams * (size_t)wpr),
+                 o_sflag = o_lflag + up16((size_t)n_long),
                  small_bytes = o_sflag + up16((size_t)n_seg);
     DeviceBlock small;
     PLX_HIP_CHECK(hipMalloc(&small.p, small_bytes));
@@ -622,6 +659,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     b.stream_total = nullptr;
     b.stream_pos = reinterpret_cast<int32_t *>(bb + o_pos);
     b.stream_run = reinterpret_cast<uint8_t *>(bb + o_run);
+    b.stream_mark = reinterpret_cast<int32_t *>(bb + o_mark);
     hub_streams_kernel<true><<<kHubStreams, 64, 0, st>>>(b);
     PLX_LAUNCH_CHECK("hub_streams_kernel (fill)");
     hub_flags_kernel<<<(unsigned)n_rows, 64, 0, st>>>((int32_t)n_long, long_rows, seg_first, reinterpret_cast<const int32_t *>(bb + o_rows),
@@ -647,6 +685,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     out.stream_total = reinterpret_cast<const int32_t *>(bb + o_total);
     out.stream_pos = reinterpret_cast<const int32_t *>(bb + o_pos);
     out.stream_run = reinterpret_cast<const uint8_t *>(bb + o_run);
+    out.stream_mark = reinterpret_cast<const int32_t *>(bb + o_mark);
     out.long_is_hub = reinterpret_cast<const uint8_t *>(bb + o_lflag);
     out.seg_is_hub = reinterpret_cast<const uint8_t *>(bb + o_sflag);
     out.h_rows_sorted = rows;
@@ -671,6 +710,9 @@ int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *
     a.stream_total = hp.stream_total;
     a.stream_pos = hp.stream_pos;
     a.stream_run = hp.stream_run;
+    a.stream_mark = hp.stream_mark;
+    a.windows_per_range = hp.windows_per_range;
+    a.pace = kHubPace;
     a.n_rows = hp.n_rows;
     a.rows = hp.rows;
     a.row_slot_first = hp.row_slot_first;
