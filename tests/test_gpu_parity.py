@@ -1164,6 +1164,36 @@ def test_spmm_hub_pass_matches_the_oracle_and_keeps_its_bits(d, dtype):
     assert torch.equal(y.cpu()[rows], y_plain.cpu()[rows])
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_spmm_hub_pass_on_random_shapes(seed):
+    """Rectangular matrices with a few very long rows, every width class and both element types, against the fp64 oracle."""
+    say("spmm hub pass, random shape %d" % seed)
+    gen = torch.Generator().manual_seed(100 + seed)
+    m = int(torch.randint(50, 4000, (1,), generator=gen))
+    k = int(torch.randint(9, 30000, (1,), generator=gen))
+    seg_len = [2, 8, 64, 256][seed % 4]
+    # row lengths: mostly short, some far beyond a part (8 * seg_len), one covering every column
+    lens = torch.randint(0, 6, (m,), generator=gen)
+    long_rows = torch.randperm(m, generator=gen)[: max(3, m // 20)]
+    lens[long_rows] = torch.randint(seg_len + 1, max(seg_len + 2, min(k, 40 * seg_len)), (long_rows.numel(),), generator=gen)
+    lens[long_rows[0]] = k
+    lens = lens.clamp(max=k)
+    cols = [torch.randperm(k, generator=gen)[: int(n)].sort().values for n in lens]
+    rowptr = torch.zeros(m + 1, dtype=torch.int64)
+    rowptr[1:] = torch.cumsum(lens, 0)
+    col = torch.cat(cols).to(torch.int32)
+    val = torch.randn(col.numel(), generator=gen)
+    a = ops.CsrMatrix(rowptr.to(torch.int32).to(DEV), col.to(DEV), val.to(DEV), (m, k), seg_len)
+    a.build_hub()
+    assert a.n_hub_rows > 0
+    for d, dtype in ((128, torch.float32), (64, torch.float32), (388, torch.float32), (256, torch.bfloat16), (132, torch.bfloat16)):
+        h = torch.randn(k, d, generator=gen).to(dtype)
+        ref = oracle_c.csr_spmm(rowptr.to(torch.int32).numpy(), col.numpy(), val.numpy(), h.float().numpy())
+        y = ops.spmm(a, h.to(DEV))
+        assert rel_err(y.float().cpu(), ref) <= (FP32_TOL if dtype == torch.float32 else BF16_TOL), (m, k, seg_len, d, dtype)
+        assert torch.equal(ops.chunked_spmm(a, h.to(DEV), max_rows_per_chunk=max(1, m // 3)), y)
+
+
 def test_spmm_hub_pass_is_left_out_where_the_operand_does_not_suit_it():
     say("spmm hub pass: widths and layouts it does not take")
     g, a = _hub_matrix(seed=32)

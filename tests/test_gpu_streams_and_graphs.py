@@ -28,13 +28,17 @@ def to_dev(g, transpose=False, seg_len=0):
 
 
 @pytest.mark.filterwarnings("ignore:The AccumulateGrad node")  # the warm-up runs on a side stream on purpose
-@pytest.mark.parametrize("association", ["reference", "auto"])
-def test_forward_loss_backward_replay_from_a_hip_graph(association):
-    say("HIP graph capture of forward + loss + backward, association=%s" % association)
-    n, dims, classes = 3000, [40, 32, 7], 7
+@pytest.mark.parametrize("association,hub", [("reference", False), ("auto", False), ("reference", True)])
+def test_forward_loss_backward_replay_from_a_hip_graph(association, hub):
+    say("HIP graph capture of forward + loss + backward, association=%s, hub pass=%s" % (association, hub))
+    n, dims, classes = 3000, ([128, 64, 7] if hub else [40, 32, 7]), 7
     g = S.build_graph(n, "chunglu", 40000, seed=5, device="cpu", gamma=2.1)
     shards = [(to_dev(g, seg_len=64), to_dev(g, True, seg_len=64))]  # split rows: the workspace path is recorded too
     assert shards[0][0].n_long_rows > 0
+    if hub:  # the longest rows go through the hub pass (its kernels, its LDS size attribute and its workspace are recorded too)
+        for a in shards[0]:
+            a.build_hub()
+            assert a.n_hub_rows > 0
     ws = S.glorot_weights(dims, seed=3)
     model = Net(2, dims[0], dims[1], dims[2], weights=ws, fuse_relu=True, association=association)
     params = list(model.parameters())
