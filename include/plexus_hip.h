@@ -128,7 +128,7 @@ int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host
 int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
 /* The hub pass.  On a power-law graph a third of the entries sit in a few thousand rows; gathered row by row they miss
  * the cache like every other row.  A plan may carry tables that let those rows ("hub rows": the longest of the split
- * rows, cut into at most 9,216 parts of at most 8 * seg_len entries) walk the columns together, window after window of
+ * rows, cut into at most 9,216 parts of at most 16 * seg_len entries) walk the columns together, window after window of
  * 4,096 columns, one eighth of the columns per XCD, so that a row of H fetched for one of them is found in that XCD's
  * L2 by the others (2.45 M nodes, 126 M entries, 128 fp32 columns: 7.3 -> 5.7 ms).  The tables cost 5 bytes per entry
  * of a hub row.  plx_spmm_plan_create builds them by itself where it expects a gain: short rows on average (fewer

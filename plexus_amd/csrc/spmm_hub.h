@@ -24,7 +24,8 @@ constexpr int kHubWindow = 4096;     // columns per window: 2 MB of 512-byte row
 constexpr int kHubPace = 1;          // windows a wavefront may run ahead of the slowest of its workgroup (measured, hub pass of the
                                      // 2.45 M-node graph: none 1.36 ms and 6.1 GB fetched, 0 / 1 / 2 / 3: 1.35 / 1.27 / 1.30 / 1.31 ms, 1: 3.9 GB)
 constexpr int kHubMaxPolls = 4096;   // of a wavefront waiting for the others, then it goes on regardless
-constexpr int kHubPartFactor = 8;    // a hub row is cut into parts of at most kHubPartFactor * seg_len entries
+constexpr int kHubPartFactor = 16;   // a hub row is cut into parts of at most kHubPartFactor * seg_len entries (8 / 16 / 32 / 64 on the
+                                     // 2.45 M-node graph: 6,530 / 8,170 / 8,820 / 9,074 hub rows, product 5.73 / 5.69 / 5.67 / 5.68 ms)
 constexpr int64_t kHubMaxBytes = 1ll << 32;  // rows of H are addressed with 32-bit byte offsets
 
 // Device tables of a plan's hub pass.  A slot is a part of a hub row; the slots are dealt over the wavefronts by size.

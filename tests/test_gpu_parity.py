@@ -1136,8 +1136,8 @@ def _hub_matrix(seed, n=3000, pairs=40000, seg_len=16):
 def test_spmm_hub_pass_matches_the_oracle_and_keeps_its_bits(d, dtype):
     say("spmm hub pass D=%d %s" % (d, dtype))
     g, a = _hub_matrix(seed=31)
-    # split rows of more than 8 * seg_len entries take several parts; the longest rows all become hub rows
-    assert a.n_hub_rows == a.n_long_rows > 100 and g.degree_stats()["max_row_nnz"] > 8 * 16
+    # split rows of more than 16 * seg_len entries take several parts; the longest rows all become hub rows
+    assert a.n_hub_rows == a.n_long_rows > 100 and g.degree_stats()["max_row_nnz"] > 16 * 16
     assert a.hub_entries > g.nnz // 3
     h32 = torch.randn(3000, d, generator=torch.Generator().manual_seed(d))
     h = h32.to(dtype).to(DEV)
@@ -1172,7 +1172,7 @@ def test_spmm_hub_pass_on_random_shapes(seed):
     m = int(torch.randint(50, 4000, (1,), generator=gen))
     k = int(torch.randint(9, 30000, (1,), generator=gen))
     seg_len = [2, 8, 64, 256][seed % 4]
-    # row lengths: mostly short, some far beyond a part (8 * seg_len), one covering every column
+    # row lengths: mostly short, some far beyond a part (16 * seg_len), one covering every column
     lens = torch.randint(0, 6, (m,), generator=gen)
     long_rows = torch.randperm(m, generator=gen)[: max(3, m // 20)]
     lens[long_rows] = torch.randint(seg_len + 1, max(seg_len + 2, min(k, 40 * seg_len)), (long_rows.numel(),), generator=gen)
