@@ -21,6 +21,7 @@ constexpr int kHubTile = 32 * kHubVec;
 constexpr int kHubSlots = kHubGroups * kWaves * kHubRowsPerWave;  // 9,216 slots: a hub row takes one per part
 constexpr int kHubStreams = kHubRanges * kHubGroups * kWaves;     // one per wavefront of the pass
 constexpr int kHubWindow = 4096;     // columns per window: 2 MB of 512-byte rows, half of an XCD's L2
+constexpr int kHubMaxWindows = 4096;  // windows per range a plan may have
 constexpr int kHubPace = 1;          // windows a wavefront may run ahead of the slowest of its workgroup (measured, hub pass of the
                                      // 2.45 M-node graph: none 1.36 ms and 6.1 GB fetched, 0 / 1 / 2 / 3: 1.35 / 1.27 / 1.30 / 1.31 ms, 1: 3.9 GB)
 constexpr int kHubMaxPolls = 4096;   // of a wavefront waiting for the others, then it goes on regardless

@@ -602,6 +602,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     const int32_t window = kHubWindow;
     const int32_t wpr = (int32_t)ceil_div(ceil_div(K, kHubRanges), window);
     const int32_t n_windows = wpr * kHubRanges;
+    if (wpr > kHubMaxWindows) return PLX_OK;  // beyond 134 M columns the per-window tables outgrow their use: no hub pass
 
     // the small tables and the stream lengths
     const size_t n_rows = rows.size(), n_slots = slots.size();
