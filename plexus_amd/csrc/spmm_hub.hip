@@ -10,7 +10,8 @@
 // A hub row is cut into parts of bounded length ("slots": part s of S takes the s-th S-th of the row's entries inside
 // every window), and the slots are dealt over the wavefronts by size.  A workgroup keeps the sums of its slots for its
 // range in LDS for the whole pass; a wavefront owns kHubRowsPerWave of them, so no two wavefronts touch the same sum
-// and nothing needs an atomic or a barrier.  The entries of a slot inside a window are a contiguous run of the CSR
+// and no sum needs an atomic or a barrier (all that wavefronts tell each other is the window they are in, so that
+// none runs far ahead of the rows of H the others still share: "pacing" in the kernel).  The entries of a slot inside a window are a contiguous run of the CSR
 // arrays (columns are sorted within a row); the plan writes out, for every wavefront, the runs of its slots window
 // after window as one stream of positions.  The partial sums of the kHubRanges ranges of a slot go to memory and a
 // second kernel adds them, slot by slot and range by range, into the row of Y: the order of every sum is fixed by
