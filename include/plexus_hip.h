@@ -213,6 +213,21 @@ int plx_gemm_nn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64
 int plx_gemm_nt_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                           int64_t ldc, const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The ReLU mask as one bit per element.  plx_gemm_nn_f32_split_bits is plx_gemm_nn_f32_split that also writes the sign
+ * bits of C: bit c % 32 of word sign_bits[row * ldw + c / 32] is set when C[row][c] > 0 (ldw >= ceil(N / 32) words; bits
+ * of columns past N are 0).  plx_gemm_nt_f32_split_bits is plx_gemm_nt_f32_split that reads the mask of A in that form
+ * (`mask_bits`, ldw >= ceil(K / 32)) where its kernel can -- weights of at most 128 x 128, A read with 128-bit loads --
+ * and the fp32 `mask`, which must say the same, elsewhere and in the guarded fp32 launch: GRAD_AGG = (GRAD_OUT ⊙ mask) . W^T
+ * of a hidden layer then reads 1/32 of the mask's bytes (2,449,029 x 128: 0.76 -> 0.55 ms).  Same results bit for bit.
+ * plx_sign_bits_f32 writes the bits of any matrix.   examples/train.py:77-78 (F.relu between the layers) */
+int plx_gemm_nn_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                               int64_t ldc, unsigned flags, uint32_t *sign_bits, int64_t ldw, void *workspace, size_t workspace_bytes,
+                               void *stream);
+int plx_gemm_nt_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                               int64_t ldc, const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, void *workspace,
+                               size_t workspace_bytes, void *stream);
+int plx_sign_bits_f32(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *sign_bits, int64_t ldw, void *stream);
+
 /* C[K x N] = A[M x K]^T . (B ⊙ [mask > 0])[M x N]   GRAD_W = AGG^T . GRAD_OUT   plexus/gcn_conv.py:237-239
  * The reduction over M is split over workgroups; partial tiles go to `workspace` and are summed
  * in a fixed order. */

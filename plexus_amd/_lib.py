@@ -51,6 +51,9 @@ SIGNATURES = {
     "plx_gemm_f32_split_workspace_bytes": (_sz, [_i64, _i64]),
     "plx_gemm_nn_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _vp, _sz, _vp]),
     "plx_gemm_nt_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_gemm_nn_f32_split_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, C.c_uint, _vp, _i64, _vp, _sz, _vp]),
+    "plx_gemm_nt_f32_split_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_sign_bits_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),

@@ -52,6 +52,10 @@ struct SplitArgs {
     int64_t rows_per_split;
     float *ws;
     int64_t ws_ld, ws_slab;
+    // sign bits: bit c % 32 of word [row * ldw + c / 32] says that element (row, c) is positive
+    uint32_t *relu_bits;        // written beside C (resident NT kernel), or NULL
+    const uint32_t *mask_bits;  // the mask of A in that form (resident NT kernel, 128-bit loads of A), or NULL
+    int64_t ldw;
 };
 
 // x = p0 + p1 + p2 exactly (bf16 pieces, round to nearest even each); pieces of 2 values packed per word.  Holds for
@@ -349,9 +353,12 @@ constexpr int kRBS = kRMaxK + 8;      // stride of the resident B planes (272 by
 constexpr int kRAPlane = 32 * kRAS;   // bf16 elements of one private plane
 constexpr size_t kRLdsBytes = ((size_t)3 * kRMaxN * kRBS + (size_t)kRWaves * 3 * kRAPlane) * sizeof(uint16_t);
 
-template <int TN, bool MASKED>
+// MASK: 0 none, 1 fp32 values beside A (mask > 0 keeps the element), 2 one bit per element
+template <int TN, int MASK>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel(const SplitArgs g)
 {
+    constexpr bool MASKED = MASK == 1;      // the fp32 mask travels in registers beside its chunk
+    constexpr bool BITS = MASK == 2;        // the bit mask of a panel row is four words, loaded once per panel
     constexpr int kSteps = kRMaxK / kRCK;   // chunk positions of a panel (positions past K are skipped)
     constexpr int kRing = MASKED ? 4 : 8;   // register slots = how many positions ahead a chunk is requested
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
@@ -390,6 +397,12 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     int f_kc = 0;
     const int64_t lda16 = 16 * g.lda, ldm16 = 16 * g.ldmask;
     float4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
+    // Bit mask: a 64-lane load takes the memory pipeline as long for 4 bytes per lane as for 16, so the bits are not
+    // fetched chunk by chunk; the 128 bits of rows r and r + 16 of a panel come with its first chunk and stay in registers.
+    static_assert(!BITS || kRing == kSteps, "the chunks in flight are those of exactly one panel ahead");
+    u32x4 pb_cur[2], pb_next[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p] = u32x4{~0u, ~0u, ~0u, ~0u};
     auto fetch = [&](float4(&dst)[2], float4(&mdst)[2]) __attribute__((always_inline)) {
         if (f_kc < n_kc && f_panel < n_panels) {
             const int64_t row = f_panel * 32 + r;
@@ -397,6 +410,13 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             const int rows_left = (int)min(g.M - row, (int64_t)32);  // rows row + 16 p with 16 p < rows_left exist
             const float *pa = g.A + row * g.lda + k;
             const float *pm = MASKED ? g.mask + row * g.ldmask + k : nullptr;
+            if constexpr (BITS) {
+                if (f_kc == 0) {
+#pragma unroll
+                    for (int p = 0; p < 2; ++p)
+                        if (16 * p < rows_left) pb_next[p] = *reinterpret_cast<const u32x4 *>(g.mask_bits + (row + 16 * p) * g.ldw);
+                }
+            }
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f), m = make_float4(1.f, 1.f, 1.f, 1.f);
@@ -453,6 +473,11 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                     const float4 m = mcur[p];
                     v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
                 }
+                if constexpr (BITS) {
+                    // chunk kc holds contraction elements 16 kc ...: bits 16 (kc % 2) + 4 kq ... of word kc / 2
+                    const uint32_t mb = pb_cur[p][kc >> 1] >> (16 * (kc & 1) + 4 * kq);
+                    v = make_float4((mb & 1u) ? v.x : 0.f, (mb & 2u) ? v.y : 0.f, (mb & 4u) ? v.z : 0.f, (mb & 8u) ? v.w : 0.f);
+                }
                 care |= needs_care(v);
                 uint32_t lo0, lo1, lo2, hi0, hi1, hi2;
                 split2(v.x, v.y, lo0, lo1, lo2);
@@ -485,6 +510,10 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
 #pragma unroll
     for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0]);
     for (int64_t panel = first; panel < n_panels; panel += stride) {
+        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
+#pragma unroll
+            for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
+        }
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
         // the panel is complete: register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
@@ -494,36 +523,72 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
             const bool col_ok = li + t * 32 < N;
+            uint32_t word = 0;  // lane li < 16 of half h collects the sign bits of row r0 + d(li), columns 32 t ... 32 t + 31
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int d = 8 * (v / 4) + (v % 4);
                 float x = acc[t][v];
                 if (relu) x = fmaxf(x, 0.f);
                 if (col_ok && d < rows_left) pc[(int64_t)d * g.ldc + t * 32] = x;
+                if (g.relu_bits != nullptr) {  // one vote of the wavefront gives the words of two rows
+                    const uint64_t votes = __ballot(col_ok && x > 0.f);
+                    if (li == v) word = h ? (uint32_t)(votes >> 32) : (uint32_t)votes;
+                }
                 acc[t][v] = 0.f;
+            }
+            if (g.relu_bits != nullptr && li < 16) {
+                const int d = 8 * (li / 4) + (li % 4);
+                if (d < rows_left) g.relu_bits[(r0 + d) * g.ldw + t] = word;
             }
         }
     }
 }
 
-template <int TN, bool MASKED>
+template <int TN, int MASK>
 int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
 {
     // more than 64 KB of dynamic LDS has to be allowed per kernel and device (a host-side setting, cheap to repeat)
-    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASKED>),
+    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRLdsBytes));
-    gemm_split_nt_resident_kernel<TN, MASKED><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    gemm_split_nt_resident_kernel<TN, MASK><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
     return PLX_OK;
 }
 
-template <bool MASKED>
+template <int MASK>
 int launch_resident_tn(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
 {
     switch (tn) {
-        case 1: return launch_resident<1, MASKED>(g, blocks, st);
-        case 2: return launch_resident<2, MASKED>(g, blocks, st);
-        default: return launch_resident<4, MASKED>(g, blocks, st);
+        case 1: return launch_resident<1, MASK>(g, blocks, st);
+        case 2: return launch_resident<2, MASK>(g, blocks, st);
+        default: return launch_resident<4, MASK>(g, blocks, st);
     }
+}
+
+// sign bits of a matrix: word [row * ldw + w] = bits of columns 32 w ... 32 w + 31 (columns past N: 0).  Runs only if
+// *run_if is set (run_if == NULL: always): the bits a product wrote beside C are wrong once the guarded fp32 launch has
+// redone C.
+__global__ void __launch_bounds__(256) sign_bits_kernel(int64_t M, int64_t N, const float *__restrict__ X, int64_t ldx,
+                                                        uint32_t *__restrict__ bits, int64_t ldw, const unsigned *__restrict__ run_if)
+{
+    if (run_if != nullptr && *run_if == 0u) return;
+    const int64_t words = (N + 31) / 32;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < M * words; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = i / words, w = i % words;
+        const float *x = X + row * ldx + w * 32;
+        const int n = (int)min((int64_t)32, N - w * 32);
+        uint32_t word = 0;
+        for (int c = 0; c < n; ++c) word |= (x[c] > 0.f ? 1u : 0u) << c;
+        bits[row * ldw + w] = word;
+    }
+}
+
+int launch_sign_bits(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *bits, int64_t ldw, const unsigned *run_if, hipStream_t st)
+{
+    const int64_t items = M * ((N + 31) / 32);
+    if (items == 0) return PLX_OK;
+    sign_bits_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(items, 256), 8192), 256, 0, st>>>(M, N, X, ldx, bits, ldw, run_if);
+    PLX_LAUNCH_CHECK("sign_bits_kernel");
+    return PLX_OK;
 }
 
 int pick_tn(int64_t n) { return n <= 32 ? 1 : (n <= 64 ? 2 : 4); }
@@ -546,12 +611,15 @@ int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
 // C = epilogue((A*mask) . X^T) with X (N x K) = B^T (transpose_b) or B
 int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
             int transpose_b, float *C, int64_t ldc, const float *mask, int64_t ldmask, unsigned flags, void *workspace,
-            size_t workspace_bytes, void *stream)
+            size_t workspace_bytes, void *stream, uint32_t *relu_bits = nullptr, const uint32_t *mask_bits = nullptr, int64_t ldw = 0)
 {
     PLX_REQUIRE(M >= 0 && N >= 0 && K > 0 && N < (1ll << 30) && K < (1ll << 30), "%s: bad dimension", who);
     if (M == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(C != nullptr && A != nullptr && B != nullptr, "%s: NULL operand", who);
     PLX_REQUIRE(lda >= K && ldc >= N && (mask == nullptr || ldmask >= K), "%s: leading dimension too small", who);
+    PLX_REQUIRE(relu_bits == nullptr || ldw >= (N + 31) / 32, "%s: pitch of the sign bits smaller than ceil(N / 32) words", who);
+    PLX_REQUIRE(mask_bits == nullptr || (mask != nullptr && ldw >= (K + 31) / 32),
+                "%s: a bit mask comes with the fp32 mask it stands for and a pitch of at least ceil(K / 32) words", who);
     const int tn = pick_tn(N);
     const int64_t Np = round_up(N, 32 * tn), Kp = round_up(std::max<int64_t>(K, 1), kBK);
     const bool vec = aligned16(A, lda) && aligned16(mask, ldmask) && K % 4 == 0;
@@ -573,18 +641,27 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     // Inf / NaN / values next to FLT_MAX in either operand: the split product is then meaningless and the fp32 MFMA
     // kernel redoes it.  That
     // launch is always enqueued and returns at once unless the flag word is set.
-    auto redo = [&]() {
-        if (transpose_b)
-            return plx::gemm_nn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, flags, flag_words, 1, stream);
+    auto redo = [&]() -> int {
+        if (transpose_b) {
+            const int rc = plx::gemm_nn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, flags, flag_words, 1, stream);
+            if (rc != PLX_OK || relu_bits == nullptr) return rc;
+            return launch_sign_bits(M, N, C, ldc, relu_bits, ldw, flag_words, st);  // of the C that launch wrote, if it ran
+        }
         return plx::gemm_nt_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, flag_words, 1, stream);
     };
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags; g.a_vec = vec;
     g.nonfinite = flag_words;
+    g.ldw = ldw;
     if (resident) {
         const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
-        const int rc = mask != nullptr ? launch_resident_tn<true>(g, tn, blocks, st) : launch_resident_tn<false>(g, tn, blocks, st);
+        g.relu_bits = relu_bits;
+        // the bit mask is read with the 128-bit loads of A; other layouts take the fp32 mask
+        const bool bits = mask_bits != nullptr && vec && ldw % 4 == 0 && reinterpret_cast<uintptr_t>(mask_bits) % 16 == 0;
+        g.mask_bits = bits ? mask_bits : nullptr;
+        const int rc = bits ? launch_resident_tn<2>(g, tn, blocks, st)
+                            : (mask != nullptr ? launch_resident_tn<1>(g, tn, blocks, st) : launch_resident_tn<0>(g, tn, blocks, st));
         if (rc != PLX_OK) return rc;
         PLX_LAUNCH_CHECK("gemm_split_nt_resident_kernel");
         return redo();
@@ -596,6 +673,10 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
         if (mask != nullptr) launch_nt<true, 2>(g, tn, blocks, st); else launch_nt<false, 2>(g, tn, blocks, st);
     }
     PLX_LAUNCH_CHECK("gemm_split_nt_kernel");
+    if (relu_bits != nullptr) {  // this kernel does not write them: a pass over C does
+        const int rc = launch_sign_bits(M, N, C, ldc, relu_bits, ldw, nullptr, st);
+        if (rc != PLX_OK) return rc;
+    }
     return redo();
 }
 
@@ -622,6 +703,34 @@ int plx_gemm_nt_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64
 {
     PLX_REQUIRE(ldb >= K, "gemm_nt_split: leading dimension too small");
     return nt_form("gemm_nt_split", M, N, K, A, lda, B, ldb, 0, C, ldc, mask, ldmask, 0u, workspace, workspace_bytes, stream);
+}
+
+int plx_gemm_nn_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                               int64_t ldc, unsigned flags, uint32_t *sign_bits, int64_t ldw, void *workspace, size_t workspace_bytes,
+                               void *stream)
+{
+    PLX_REQUIRE(ldb >= N, "gemm_nn_split_bits: leading dimension too small");
+    PLX_REQUIRE(sign_bits != nullptr, "gemm_nn_split_bits: NULL sign bits");
+    return nt_form("gemm_nn_split_bits", M, N, K, A, lda, B, ldb, 1, C, ldc, nullptr, 0, flags, workspace, workspace_bytes, stream,
+                   sign_bits, nullptr, ldw);
+}
+
+int plx_gemm_nt_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                               int64_t ldc, const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, void *workspace,
+                               size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(ldb >= K, "gemm_nt_split_bits: leading dimension too small");
+    PLX_REQUIRE(mask_bits != nullptr, "gemm_nt_split_bits: NULL bit mask");
+    return nt_form("gemm_nt_split_bits", M, N, K, A, lda, B, ldb, 0, C, ldc, mask, ldmask, 0u, workspace, workspace_bytes, stream,
+                   nullptr, mask_bits, ldw);
+}
+
+int plx_sign_bits_f32(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *sign_bits, int64_t ldw, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && ldx >= N && ldw >= (N + 31) / 32, "sign_bits: bad dimension or pitch");
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(X != nullptr && sign_bits != nullptr, "sign_bits: NULL operand");
+    return launch_sign_bits(M, N, X, ldx, sign_bits, ldw, nullptr, plx::as_stream(stream));
 }
 
 }  // extern "C"

@@ -86,12 +86,15 @@ class GCNConvFunction(torch.autograd.Function):
         if bf16:
             OUT = ops.gemm_nt_bf16(AGG, ops.cast_bf16(W, transpose=True), relu=fuse_relu, dropout_p=dropout_p,
                                    seed=dropout_seed, offset=dropout_offset)
+        elif fuse_relu:
+            # the ReLU mask also as one bit per element, written by the product itself: GRAD_AGG reads it in place of OUT
+            OUT, BITS = ops.gemm_nn(AGG, W, relu=True, want_bits=True)
         else:
-            OUT = ops.gemm_nn(AGG, W, relu=fuse_relu)
+            OUT = ops.gemm_nn(AGG, W)
         timers.stop("OUT = AGG * W")
 
         # the reference saves AGG, weight and the transposed adjacency (plexus/gcn_conv.py:194)
-        ctx.save_for_backward(AGG, weight, OUT if fuse_relu else None)
+        ctx.save_for_backward(AGG, weight, OUT if fuse_relu else None, BITS if fuse_relu and not bf16 else None)
         ctx.adj_t = At
         ctx.local_weight_shape = tuple(local_weight_shape)
         ctx.x_shape = x.shape
@@ -191,7 +194,7 @@ class GCNConvFunction(torch.autograd.Function):
             return GCNConvFunction._backward_transform_first(ctx, grad_output)
         timers = get_timers()
         timers.start("gcn conv bwd")
-        agg, weight, out = ctx.saved_tensors
+        agg, weight, out, bits = ctx.saved_tensors
         W = weight.detach().reshape(ctx.local_weight_shape)
         mask = out if ctx.fuse_relu else None
         grad_output = grad_output.contiguous()
@@ -212,7 +215,7 @@ class GCNConvFunction(torch.autograd.Function):
             if ctx.bf16:
                 grad_agg = ops.gemm_nt_bf16(grad_output, ops.cast_bf16(W), mask=mask, alpha=ctx.grad_scale)
             else:
-                grad_agg = ops.gemm_nt(grad_output, W, mask=mask)
+                grad_agg = ops.gemm_nt(grad_output, W, mask=mask, mask_bits=bits)
             timers.stop("GRAD_AGG = GRAD_OUT * W.T")
 
             timers.start("GRAD_H = A.T * GRAD_AGG")

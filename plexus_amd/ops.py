@@ -360,8 +360,26 @@ def _split_ws(n: int, k: int, device):
     return _aligned_workspace(need, device), need
 
 
-def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix."""
+def _new_bits(m: int, n: int, device) -> torch.Tensor:
+    """int32 [m x ceil(n / 32)] with rows of a multiple of four words (the products read a row's bits with one 128-bit load)."""
+    words = (n + 31) // 32
+    return torch.empty((m, (words + 3) // 4 * 4), dtype=torch.int32, device=device)[:, :words]
+
+
+def sign_bits(x: torch.Tensor) -> torch.Tensor:
+    """One bit per element of an fp32 matrix: bit c % 32 of word [row, c // 32] is set when x[row, c] > 0 (int32 words)."""
+    _need_gpu(x)
+    _need_fp32("sign_bits", x=x)
+    x = _rowmajor(x)
+    m, n = x.shape
+    bits = _new_bits(m, n, x.device)
+    check(_lib.load().plx_sign_bits_f32(m, n, x.data_ptr(), _ld(x), bits.data_ptr(), _ld(bits), _stream()), "plx_sign_bits_f32")
+    return bits
+
+
+def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None, want_bits: bool = False):
+    """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix.  With ``want_bits`` the result is
+    (C, sign bits of C as by ``sign_bits``): the ReLU mask of the layer in the form ``gemm_nt(mask_bits=)`` reads."""
     _need_gpu(a, b, out)
     _need_fp32("gemm_nn", a=a, b=b)
     a, b = _rowmajor(a), _rowmajor(b)
@@ -377,6 +395,15 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
             raise ValueError("gemm_nn: out must be fp32 [%d x %d] with contiguous rows" % (m, n))
     if _split_ok(n, k, a):
         ws, need = _split_ws(n, k, a.device)
+        if want_bits:
+            bits = _new_bits(m, n, a.device)
+            check(
+                _lib.load().plx_gemm_nn_f32_split_bits(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                                       PLX_GEMM_RELU if relu else 0, bits.data_ptr(), _ld(bits), ws.data_ptr(),
+                                                       need, _stream()),
+                "plx_gemm_nn_f32_split_bits",
+            )
+            return c, bits
         check(
             _lib.load().plx_gemm_nn_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
                                               PLX_GEMM_RELU if relu else 0, ws.data_ptr(), need, _stream()),
@@ -388,11 +415,13 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
                                     PLX_GEMM_RELU if relu else 0, _stream()),
         "plx_gemm_nn_f32",
     )
-    return c
+    return (c, sign_bits(c)) if want_bits else c
 
 
-def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """C = (A * [mask > 0]).B^T with B stored [N x K]."""
+def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None,
+            mask_bits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = (A * [mask > 0]).B^T with B stored [N x K].  ``mask_bits`` (``sign_bits(mask)``, or the second result of
+    ``gemm_nn(want_bits=True)``) lets the product read the mask as one bit per element where its kernel can."""
     _need_gpu(a, b, mask)
     _need_fp32("gemm_nt", a=a, b=b, mask=mask)
     a, b = _rowmajor(a), _rowmajor(b)
@@ -405,8 +434,20 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
         if mask.shape != a.shape:
             raise ValueError("gemm_nt: mask shape differs from A")
     c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    if mask_bits is not None:
+        if mask is None or mask_bits.dtype != torch.int32 or mask_bits.dim() != 2 or mask_bits.shape[0] != m or \
+                mask_bits.shape[1] < (k + 31) // 32 or mask_bits.stride(1) != 1:
+            raise ValueError("gemm_nt: mask_bits must be int32 [%d x >= %d] beside the fp32 mask" % (m, (k + 31) // 32))
     if _split_ok(n, k, a, mask):
         ws, need = _split_ws(n, k, a.device)
+        if mask_bits is not None:
+            check(
+                _lib.load().plx_gemm_nt_f32_split_bits(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                                       mask.data_ptr(), _ld(mask), mask_bits.data_ptr(), _ld(mask_bits),
+                                                       ws.data_ptr(), need, _stream()),
+                "plx_gemm_nt_f32_split_bits",
+            )
+            return c
         check(
             _lib.load().plx_gemm_nt_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
                                               mask.data_ptr() if mask is not None else None,

@@ -402,6 +402,57 @@ def test_gemm_nt_and_mask(m, n, k, fp32_gemm_path):
     assert rel_err(cm, ref) <= FP32_TOL
 
 
+def _pack_bits(x):
+    """Reference of the sign bits: bit c % 32 of int32 word [row, c // 32] is x[row, c] > 0."""
+    m, n = x.shape
+    words = (n + 31) // 32
+    pos = torch.zeros(m, words * 32, dtype=torch.int64)
+    pos[:, :n] = (x > 0).to(torch.int64)
+    w = (pos.reshape(m, words, 32) << torch.arange(32, dtype=torch.int64)).sum(-1)
+    return torch.where(w >= 2**31, w - 2**32, w).to(torch.int32)
+
+
+@pytest.mark.parametrize("m,n,k", [(3000, 128, 100), (1001, 128, 128), (777, 47, 128), (2050, 100, 64), (500, 200, 150), (33, 7, 5)])
+def test_relu_mask_as_sign_bits(m, n, k, fp32_gemm_path):
+    say("sign bits of a product and a bit mask into the next, M=%d N=%d K=%d (%s)" % (m, n, k, fp32_gemm_path))
+    gen = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=gen).to(DEV)
+    w = torch.randn(k, n, generator=gen).to(DEV) * 0.1
+    # forward: the product writes the bits of its own result (fused in the kernel for weights up to 128 x 128)
+    out, bits = ops.gemm_nn(a, w, relu=True, want_bits=True)
+    assert torch.equal(out, ops.gemm_nn(a, w, relu=True))
+    assert bits.dtype == torch.int32 and tuple(bits.shape) == (m, (n + 31) // 32)
+    assert torch.equal(bits.cpu(), _pack_bits(out.cpu()))
+    assert torch.equal(ops.sign_bits(out), bits)
+    assert 0.3 < (out > 0).float().mean().item() < 0.7  # a real mask, not all ones
+    # backward: GRAD_AGG = (G * mask) . W^T with the mask as bits gives the bits of the fp32 mask
+    gout = torch.randn(m, n, generator=gen).to(DEV)
+    want = ops.gemm_nt(gout, w, mask=out)
+    got = ops.gemm_nt(gout, w, mask=out, mask_bits=bits)
+    assert torch.equal(got, want)
+    ref = (gout.cpu().double() * (out.cpu() > 0)) @ w.cpu().double().T
+    assert rel_err(got.cpu(), ref) <= FP32_TOL
+    # a view with a row pitch that 128-bit loads cannot take: the fp32 mask is read instead, same result
+    wide = torch.zeros(m, n + 3, device=DEV)
+    wide[:, 1:n + 1] = gout
+    view = wide[:, 1:n + 1]
+    assert torch.equal(ops.gemm_nt(view, w, mask=out, mask_bits=bits), ops.gemm_nt(view, w, mask=out))
+    with pytest.raises(ValueError):
+        ops.gemm_nt(gout, w, mask_bits=bits)  # the bits stand for a mask that must be given too
+
+
+def test_sign_bits_follow_the_product_the_guarded_launch_redoes():
+    say("sign bits when an operand holds Inf (the fp32 kernel redoes the product)")
+    gen = torch.Generator().manual_seed(9)
+    a = torch.randn(700, 128, generator=gen)
+    a[5, 3] = float("inf")
+    a[9, 7] = float("nan")
+    w = torch.randn(128, 128, generator=gen) * 0.1
+    out, bits = ops.gemm_nn(a.to(DEV), w.to(DEV), relu=True, want_bits=True)
+    assert torch.isinf(out[5]).any() or torch.isnan(out[5]).any()
+    assert torch.equal(bits.cpu(), _pack_bits(out.cpu()))
+
+
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(70000, 128, 100), (40000, 47, 128)])
 def test_gemm_tn_and_mask(m, n, k):
     say("gemm_tn %dx%dx%d" % (m, n, k))
