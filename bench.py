@@ -286,9 +286,14 @@ def bench_dense_kernels(args, dev):
             w = torch.randn(k, n, device=dev) * 0.1
             wt = w.t().contiguous()
             act = torch.relu(S.normal_features(m, n, dev, seed=20 + li))
-            rec("OUT = AGG.W %dx%d%s" % (k, n, "" if last else " +ReLU"), lambda: ops.gemm_nn(a, w, relu=not last), e * m * (k + n), 2.0 * m * k * n)
-            rec("GRAD_AGG = (G*mask).W^T %dx%d" % (n, k), lambda: ops.gemm_nt(g, w, mask=None if last else act),
-                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            # a hidden layer's product also writes the sign bits of its result, and GRAD_AGG reads the mask in that form
+            bits = None if last else ops.sign_bits(act)
+            rec("OUT = AGG.W %dx%d%s" % (k, n, "" if last else " +ReLU +sign bits"),
+                (lambda: ops.gemm_nn(a, w)) if last else (lambda: ops.gemm_nn(a, w, relu=True, want_bits=True)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
+            rec("GRAD_AGG = (G*mask).W^T %dx%d%s" % (n, k, "" if last else " (bit mask)"),
+                (lambda: ops.gemm_nt(g, w)) if last else (lambda: ops.gemm_nt(g, w, mask=act, mask_bits=bits)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
             rec("GRAD_W = AGG^T.(G*mask) %dx%d" % (k, n), lambda: ops.gemm_tn(a, g, mask=None if last else act),
                 e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
             del wt
