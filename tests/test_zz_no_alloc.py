@@ -62,3 +62,26 @@ def test_static_scratch_spmm_refuses_what_does_not_fit():
     assert b"static" in lib.plx_last_error()
     with pytest.raises(_lib.PlexusHipError, match="workspace"):
         _lib.check(rc, "plx_spmm_csr_f32_static")
+
+
+def test_static_scratch_spmm_on_a_plan_with_a_hub_pass():
+    """The static entry point never takes the hub pass: bit for bit the product with the pass switched off, and within
+    fp32 rounding of the product that takes it."""
+    lib = _lib.load()
+    print("[case] static-scratch spmm on a plan with hub tables", flush=True)
+    g = S.build_graph(3000, "chunglu", 40000, seed=7, device="cpu", gamma=2.1)
+    a = ops.CsrMatrix(g.rowptr.to(DEV), g.col.to(DEV), g.val.to(DEV), g.shape, 16)
+    a.build_hub()
+    assert a.n_hub_rows > 0
+    d = 128
+    h = torch.randn(3000, d, generator=torch.Generator().manual_seed(8)).to(DEV)
+    y_hub = ops.spmm(a, h)
+    a.set_hub(-1)
+    y_plain = ops.spmm(a, h)
+    a.set_hub(0)
+    assert not torch.equal(y_hub, y_plain)
+    y = torch.full((3000, d), float("nan"), device=DEV)
+    _lib.check(lib.plx_spmm_csr_f32_static(a._plan, a.val.data_ptr(), h.data_ptr(), d, d, y.data_ptr(), d,
+                                           torch.cuda.current_stream().cuda_stream), "plx_spmm_csr_f32_static")
+    assert torch.equal(y, y_plain)
+    assert rel_err(y.cpu(), y_hub.cpu()) <= 2e-6
