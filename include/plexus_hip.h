@@ -164,9 +164,10 @@ int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t 
                           void *stream);
 /* The whole-matrix fp32 product for callers that CANNOT ALLOCATE device memory or bring a workspace (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
- * Same kernels and the same bits as plx_spmm_csr_f32, but the partial sums of the split rows live in a static device
- * array of PLX_SPMM_STATIC_SCRATCH_BYTES (32 MiB, held by every GPU the library runs on until the process ends) and
- * H is never copied into line-aligned rows.  The call allocates nothing; the array's device address is looked up on
+ * The row kernel of plx_spmm_csr_f32 with the same bits, but the partial sums of the split rows live in a static device
+ * array of PLX_SPMM_STATIC_SCRATCH_BYTES (32 MiB, held by every GPU the library runs on until the process ends),
+ * H is never copied into line-aligned rows and the hub pass is never taken (its partial sums would not fit): on a plan
+ * with hub tables the result is that of plx_spmm_csr_f32 with the pass switched off, bit for bit.  The call allocates nothing; the array's device address is looked up on
  * the first call on each device (make that call outside a capture).  A plan whose split rows need more than the
  * array holds -- segments x ceil(D / 4) x 16 bytes -- is refused with PLX_ERR_WORKSPACE.  All calls on one GPU share
  * the array: calls that may overlap there (different streams or host threads) race, so order them. */
