@@ -12,9 +12,11 @@
  *     stream-ordered and asynchronous, they never synchronise the device unless stated;
  *   - the return value is 0 on success or a negative plx_status; nothing throws;
  *     plx_last_error() gives a thread-local message for the last failure;
- *   - apart from plx_spmm_plan_create (which owns a few small device tables until
- *     plx_spmm_plan_destroy, and a 4-byte counter during the call) no call allocates: scratch comes from the caller, sized by the
- *     matching *_workspace_bytes query;
+ *   - two calls allocate device memory (hipMalloc, outside any caller's allocator), both of them plan construction and
+ *     both released by plx_spmm_plan_destroy: plx_spmm_plan_create (the tables of the split rows, a few counters during
+ *     the call, and -- where it builds them by itself -- the tables of the hub pass) and plx_spmm_plan_build_hub (the
+ *     tables of the hub pass: 5 bytes per entry of a hub row, reported by plx_spmm_plan_info(plan, 8)).  No other call
+ *     allocates: scratch comes from the caller, sized by the matching *_workspace_bytes query;
  *   - results are deterministic: no atomics, fixed summation order for given inputs and plan.
  */
 #ifndef PLEXUS_HIP_H
@@ -38,7 +40,9 @@ typedef enum plx_status {
 
 /* epilogue / prologue flags of the GEMM entry points */
 #define PLX_GEMM_RELU 1u    /* C = max(C, 0) (examples/train.py:77-78 fused into the producer) */
-#define PLX_GEMM_DROPOUT 2u /* after the ReLU: zero with probability p, scale the rest by 1 / (1 - p) */
+#define PLX_GEMM_DROPOUT 2u /* after the ReLU: zero with probability p, scale the rest by 1 / (1 - p).  Understood by the
+                             * entry points that take (p, seed, offset): plx_gemm_nt_bf16, plx_gemm_nn_f32_split_dropout;
+                             * the others refuse it (PLX_ERR_UNSUPPORTED / PLX_ERR_INVALID) rather than ignore it */
 
 int plx_version(void);
 const char *plx_error_string(int status);
@@ -140,16 +144,23 @@ int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
  * whole pass if it holds a hub row.  The order of every sum is fixed by the plan: the same operands give the same bits
  * on every call and in every row range, but not the bits of a product without the pass (the two agree to fp32
  * rounding).  plx_spmm_csr_f32_static never uses it.
+ * The tables are cut out of the rows by bisection, so the columns of every split row must ascend (what to_sparse_csr()
+ * gives, plexus/utils/dataloader.py:367; the other products take the columns of a row in any order): on a matrix where
+ * they do not, plx_spmm_plan_build_hub returns PLX_ERR_UNSUPPORTED and plx_spmm_plan_create leaves the tables out.
  * mode 0: use the pass where possible (the default), -1: never. */
 int plx_spmm_plan_build_hub(plx_spmm_plan *plan, void *stream);
 int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode);
-/* bytes of scratch an SpMM of width D needs: fp32 partial sums of the split rows, plus -- when rows of D fp32
+/* bytes of scratch an fp32 SpMM of width D needs (plx_spmm_workspace_bytes_bf16: a bf16 one -- the hub pass, the column
+ * slices and the copy below go by the bytes of a row, so the two types differ, and a product given less than its own
+ * query asks for returns PLX_ERR_WORKSPACE): fp32 partial sums of the split rows, the partial sums
+ * of the hub pass where the plan has one and the width takes it, plus -- when rows of D fp32
  * elements laid end to end straddle more 128-byte lines than they have to and every row of H is gathered often
  * enough to repay a copy -- room for a copy of H in rows that start on lines, which whole-matrix products then
  * gather from (0.2 ms of copying against 3 ms saved at K = 232,965, D = 602, 492 gathers per row).  0 if neither
  * applies; for a sliced shape (above) whose contiguous rows do not start on 128-byte lines, room for that copy as well.
  * The result does not depend on whether the copy is used. */
 size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D);
+size_t plx_spmm_workspace_bytes_bf16(const plx_spmm_plan *plan, int64_t D);
 
 /* fp32 values, fp32 H and Y. */
 int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H, int64_t ldh, int64_t D, float *Y,
@@ -162,6 +173,15 @@ int plx_spmm_csr_f32(const plx_spmm_plan *plan, const float *val, const float *H
 int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const float *H,
                           int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
                           void *stream);
+/* A product computed chunk by chunk in stream order, as the blocked aggregation of plexus/gcn_conv.py:67-128 does: the calls
+ * share plan, val, H, D and workspace and differ in their row range; `first_chunk` != 0 on the first of them.  Same rows,
+ * same bits as plx_spmm_csr_rows_f32, but what the chunks have in common is computed once: where the plan has a hub
+ * pass, the first chunk runs it for every hub row and leaves its partial sums in the workspace, and the later chunks
+ * only add up the hub rows of their range (plx_spmm_csr_rows_f32 runs the whole pass in every range that holds a hub
+ * row: three times on a 2.45 M-row matrix in chunks of a million rows).  A later chunk must therefore follow the first
+ * in stream order and find the workspace as the first left it; chunks after the first may still overlap each other. */
+int plx_spmm_csr_chunk_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, int first_chunk, const float *val, const float *H,
+                           int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream);
 /* The whole-matrix fp32 product for callers that CANNOT ALLOCATE device memory or bring a workspace (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * The row kernel of plx_spmm_csr_f32 with the same bits, but the partial sums of the split rows live in a static device
@@ -182,6 +202,10 @@ int plx_spmm_csr_bf16(const plx_spmm_plan *plan, const float *val, const uint16_
 int plx_spmm_csr_rows_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const uint16_t *H,
                            int64_t ldh, int64_t D, uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
                            void *stream);
+/* chunk of a bf16 product computed chunk by chunk, as plx_spmm_csr_chunk_f32 */
+int plx_spmm_csr_chunk_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, int first_chunk, const float *val,
+                            const uint16_t *H, int64_t ldh, int64_t D, uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                            void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Dense products of the layer (all replace tuned_matmul -> torch.mm, plexus/utils/matmul_tuning.py:94-95)
@@ -228,6 +252,27 @@ int plx_gemm_nt_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, 
                                int64_t ldc, const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, void *workspace,
                                size_t workspace_bytes, void *stream);
 int plx_sign_bits_f32(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *sign_bits, int64_t ldw, void *stream);
+
+/* Dropout for fp32 storage, fused after the ReLU of the forward product (examples/train.py:77-78 is where a model puts it;
+ * the reference's Net has none, this follows plx_gemm_nt_bf16).  The mask is the one defined there: element e (row-major
+ * linear index row * N + col) is kept iff 16-bit lane e % 8 of Philox-4x32-10(counter = (e / 8, offset), key = seed) is
+ * >= round(p * 65536), and a kept element is scaled by 1 / (1 - p) -- a host regenerates it from (seed, offset, p).
+ *   plx_gemm_nn_f32_split_dropout: plx_gemm_nn_f32_split_bits with PLX_GEMM_DROPOUT honoured: C = dropout(relu(A . B))
+ *     and, if sign_bits is not NULL, the bits of that C (zero where the ReLU or the dropout zeroed it: the mask the
+ *     backward products need).  For weights of at most 128 x 128 and N a multiple of 8 the product's kernel applies the
+ *     mask to its accumulators (one call of the generator per 8 elements); other shapes take a pass over C.
+ *   plx_gemm_nt_f32_split_scaled: plx_gemm_nt_f32_split_bits (mask_bits may be NULL) times alpha, the 1 / (1 - p) of the
+ *     backward pass: GRAD_AGG = alpha * (GRAD_OUT (.) mask) . W^T; alpha multiplies the weight before it is split, so
+ *     alpha = 1 gives the bits of the unscaled entry point and a power of two scales them exactly.
+ *   plx_dropout_f32: the same mask applied in place to any fp32 matrix (after plx_gemm_nn_f32 for operands the split
+ *     products do not take). */
+int plx_gemm_nn_f32_split_dropout(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                                  int64_t ldc, unsigned flags, float dropout_p, uint64_t seed, uint64_t offset, uint32_t *sign_bits,
+                                  int64_t ldw, void *workspace, size_t workspace_bytes, void *stream);
+int plx_gemm_nt_f32_split_scaled(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                                 int64_t ldc, const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, float alpha,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+int plx_dropout_f32(int64_t M, int64_t N, float *X, int64_t ldx, float dropout_p, uint64_t seed, uint64_t offset, void *stream);
 
 /* C[K x N] = A[M x K]^T . (B ⊙ [mask > 0])[M x N]   GRAD_W = AGG^T . GRAD_OUT   plexus/gcn_conv.py:237-239
  * The reduction over M is split over workgroups; partial tiles go to `workspace` and are summed

@@ -362,11 +362,15 @@ class OracleNet:
     (flat, as the reference keeps them) and the input features are the trained tensors.
     """
 
-    def __init__(self, weights: Sequence[torch.Tensor], dims: Sequence[int]):
+    def __init__(self, weights: Sequence[torch.Tensor], dims: Sequence[int], dropout_p: float = 0.0, seed: int = 0):
         self.weights = [w.clone() for w in weights]
         self.dims = list(dims)
+        # dropout after every ReLU (not in the reference's Net; the counter-based mask of dropout_keep_mask below)
+        self.p = dropout_p
+        self.seed = seed
 
-    def forward(self, x, adj_shards):
+    def forward(self, x, adj_shards, offsets=None):
+        """``offsets[i]``: dropout offset of layer i for this pass (needed when dropout_p > 0)."""
         saved = []
         h = x
         n_layers = len(self.weights)
@@ -376,9 +380,13 @@ class OracleNet:
             wshape = (self.dims[i], self.dims[i + 1])
             out, agg = gcn_conv_forward(h, a, w, fshape, wshape)
             pre = out
+            keep = None
             if i != n_layers - 1:
                 out = F.relu(out)  # train.py:77-78
-            saved.append((agg, a_t, wshape, pre))
+                if self.p > 0.0:
+                    keep = torch.from_numpy(dropout_keep_mask(out.numel(), self.seed, offsets[i], self.p).reshape(out.shape)).to(out.dtype)
+                    out = out * keep / (1.0 - self.p)
+            saved.append((agg, a_t, wshape, pre, keep))
             h = out
         self._saved = saved
         return h
@@ -391,10 +399,12 @@ class OracleNet:
         grads_w = [None] * len(self.weights)
         n_layers = len(self.weights)
         for i in reversed(range(n_layers)):
-            agg, a_t, wshape, pre = self._saved[i]
+            agg, a_t, wshape, pre, keep = self._saved[i]
             if i != n_layers - 1:
                 mask = (pre > 0) if masks is None or masks[i] is None else masks[i]
                 g = g * mask.to(g.dtype)
+                if keep is not None:
+                    g = g * keep / (1.0 - self.p)
             g, grads_w[i] = gcn_conv_backward(g, agg, self.weights[i], a_t, wshape, flatten_grad_x=(i == 0))
         return g, grads_w
 

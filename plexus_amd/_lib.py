@@ -41,8 +41,11 @@ SIGNATURES = {
     "plx_spmm_plan_build_hub": (C.c_int, [_vp, _vp]),
     "plx_spmm_plan_set_hub": (C.c_int, [_vp, C.c_int]),
     "plx_spmm_workspace_bytes": (_sz, [_vp, _i64]),
+    "plx_spmm_workspace_bytes_bf16": (_sz, [_vp, _i64]),
     "plx_spmm_csr_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_spmm_csr_rows_f32": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_spmm_csr_chunk_f32": (C.c_int, [_vp, _i64, _i64, C.c_int, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "plx_spmm_csr_chunk_bf16": (C.c_int, [_vp, _i64, _i64, C.c_int, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_spmm_static_scratch_bytes": (_sz, []),
     "plx_spmm_csr_f32_static": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp]),
     "plx_spmm_csr_bf16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _sz, _vp]),
@@ -54,6 +57,11 @@ SIGNATURES = {
     "plx_gemm_nn_f32_split_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, C.c_uint, _vp, _i64, _vp, _sz, _vp]),
     "plx_gemm_nt_f32_split_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_sign_bits_f32": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "plx_gemm_nn_f32_split_dropout": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _u32, _f32, C.c_uint64, C.c_uint64,
+                                                _vp, _i64, _vp, _sz, _vp]),
+    "plx_gemm_nt_f32_split_scaled": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz,
+                                               _vp]),
+    "plx_dropout_f32": (C.c_int, [_i64, _i64, _vp, _i64, _f32, C.c_uint64, C.c_uint64, _vp]),
     "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -36,7 +37,7 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                    int64_t ldc, unsigned flags, const unsigned *run_if, int n_run_if, void *stream);
 int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
-                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream);
+                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream, float alpha = 1.f);
 
 #if defined(__HIPCC__)
 // Orders the LDS accesses of one wavefront for the compiler: lanes that exchange data through a tile private to their
@@ -72,3 +73,21 @@ __device__ __forceinline__ void wave_lds_fence()
     do {                                                        \
         if (!(cond)) return plx::fail(PLX_ERR_INVALID, __VA_ARGS__); \
     } while (0)
+
+namespace plx {
+
+// A kernel that takes more than 64 KB of dynamic LDS has to be allowed to, per kernel and device.  The setting is a
+// runtime call, so a launcher makes it once per (kernel instantiation, device) and remembers it in `done`, one bit per
+// device ordinal (ordinals past 63 make the call every time); later launches only ask which device is current.
+inline int allow_dynamic_lds(const void *kernel, size_t bytes, std::atomic<uint64_t> &done)
+{
+    int dev = 0;
+    PLX_HIP_CHECK(hipGetDevice(&dev));
+    const uint64_t bit = (dev >= 0 && dev < 64) ? (1ull << dev) : 0ull;
+    if (bit != 0 && (done.load(std::memory_order_acquire) & bit) != 0) return PLX_OK;
+    PLX_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    if (bit != 0) done.fetch_or(bit, std::memory_order_release);
+    return PLX_OK;
+}
+
+}  // namespace plx

@@ -50,6 +50,7 @@ struct GemmArgs {
     float *ws;             // TN only: partial tiles [split][Kpad][Npad]
     int64_t ws_ld, ws_slab;
     unsigned flags;
+    float alpha;           // NN / NT: C = epilogue(alpha * product)
     int a_vec, b_vec, m_vec;  // 1 when 128-bit global loads of that operand are legal
     // when set, the launch does nothing unless one of these n_run_if device words (a few at most) is non-zero: the
     // fp32 redo of a split product whose operands turned out to hold Inf / NaN
@@ -321,6 +322,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
             const int64_t r = row0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
             if (r < nrows) {
                 float x = acc[t][v];
+                if constexpr (MODE != kTN) x *= g.alpha;
                 if (relu) x = fmaxf(x, 0.f);
                 out[r * ldo + c] = x;
             }
@@ -548,6 +550,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
 #pragma unroll
                 for (int t = 0; t < TN; ++t) {
                     float x = acc[t][4 * v4 + vv];
+                    if constexpr (MODE != kTN) x *= g.alpha;
                     if (relu) x = fmaxf(x, 0.f);
                     if (t * 32 < cols_left) q[t * 32] = x;
                 }
@@ -656,7 +659,7 @@ int gemm_nn_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
     PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_nn: leading dimension too small");
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
-    g.M = M; g.N = N; g.K = K; g.flags = flags;
+    g.M = M; g.N = N; g.K = K; g.flags = flags; g.alpha = 1.f;
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb);
     g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
@@ -667,7 +670,7 @@ int gemm_nn_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
 }
 
 int gemm_nt_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
-                 int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream)
+                 int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream, float alpha = 1.f)
 {
     int rc = check_common("gemm_nt", M, N, K, A, B, C);
     if (rc != PLX_OK) return rc < 0 ? rc : PLX_OK;
@@ -675,7 +678,7 @@ int gemm_nt_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
     PLX_REQUIRE(mask == nullptr || ldmask >= K, "gemm_nt: mask leading dimension too small");
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
-    g.M = M; g.N = N; g.K = K;
+    g.M = M; g.N = N; g.K = K; g.alpha = alpha;
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
     g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
@@ -695,9 +698,9 @@ int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
     return gemm_nn_impl(M, N, K, A, lda, B, ldb, C, ldc, flags, run_if, n_run_if, stream);
 }
 int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
-                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream)
+                   int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream, float alpha)
 {
-    return gemm_nt_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, run_if, n_run_if, stream);
+    return gemm_nt_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, run_if, n_run_if, stream, alpha);
 }
 }  // namespace plx
 
@@ -706,6 +709,8 @@ extern "C" {
 int plx_gemm_nn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
                     float *C, int64_t ldc, unsigned flags, void *stream)
 {
+    if (flags & PLX_GEMM_DROPOUT)  // this entry point carries no p / seed / offset
+        return plx::fail(PLX_ERR_UNSUPPORTED, "gemm_nn: PLX_GEMM_DROPOUT needs plx_gemm_nn_f32_split_dropout, or plx_dropout_f32 after this product");
     return gemm_nn_impl(M, N, K, A, lda, B, ldb, C, ldc, flags, nullptr, 0, stream);
 }
 
@@ -742,7 +747,7 @@ int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
 
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
-    g.M = M; g.N = N; g.K = K;
+    g.M = M; g.N = N; g.K = K; g.alpha = 1.f;
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
     // every split covers a multiple of the 32-row chunk so that chunk boundaries do not depend on the split
     g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;

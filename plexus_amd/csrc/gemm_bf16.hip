@@ -425,9 +425,9 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 template <int TN, bool MASKED>
 int launch_nt_resident(const Bf16Args &g, unsigned blocks, hipStream_t st)
 {
-    // more than 64 KB of dynamic LDS has to be allowed per kernel and device (a host-side setting, cheap to repeat)
-    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRLdsBytes));
+    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED>), kRLdsBytes, allowed);
+    if (rc != PLX_OK) return rc;
     gemm_bf16_nt_resident_kernel<TN, MASKED><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
     return PLX_OK;
 }

@@ -10,15 +10,14 @@
 //             Bp = the three bf16 planes of the small operand, made once per call by split_planes_kernel:
 //               forward   OUT      = AGG . W         Bp = planes of W^T   (+ ReLU)
 //               backward  GRAD_AGG = GRAD_OUT . W^T  Bp = planes of W     (+ ReLU mask on GRAD_OUT)
-//   TN form   C[K x N] = A[M x K]^T . (B*mask)[M x N]                GRAD_W = AGG^T . GRAD_OUT, both operands
-//             split on the fly, tiles transposed on their way into LDS, M split over workgroups with a
-//             fixed-order reduction of the partial tiles.
+//             (GRAD_W = AGG^T . GRAD_OUT, the reduction over the rows, runs on the fp32 MFMA: gemm.hip)
 //
 // The large operand is read as fp32 with 128-bit loads, split in registers and stored to LDS as three bf16
 // planes; an MFMA lane then reads its 8 consecutive contraction elements of a plane with one 128-bit LDS load.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 
 #include "bf16.h"
@@ -46,12 +45,10 @@ struct SplitArgs {
     unsigned flags;
     unsigned *nonfinite;  // device word raised when an operand holds a value the split cannot carry
     int a_vec;  // A (and mask) 16-byte aligned, leading dimensions and K multiples of 4: 128-bit loads
-    // TN form
-    const float *B;
-    int64_t ldb;
-    int64_t rows_per_split;
-    float *ws;
-    int64_t ws_ld, ws_slab;
+    // dropout after the ReLU (resident NT kernel): element e = row * N + col is kept iff 16-bit lane e % 8 of
+    // Philox-4x32-10(counter = (e / 8, offset), key = seed) is >= thresh16, and then scaled by keep_scale
+    uint32_t thresh16, seed_lo, seed_hi, off_lo, off_hi;
+    float keep_scale;
     // sign bits: bit c % 32 of word [row * ldw + c / 32] says that element (row, c) is positive
     uint32_t *relu_bits;        // written beside C (resident NT kernel), or NULL
     const uint32_t *mask_bits;  // the mask of A in that form (resident NT kernel, 128-bit loads of A), or NULL
@@ -81,18 +78,18 @@ __device__ __forceinline__ int needs_care(const float4 &v) { return needs_care(v
 // all of them show as Inf / NaN first pieces).
 constexpr size_t kFlagBytes = 256;
 
-// the three bf16 planes of a small fp32 matrix, optionally transposed: P[p][n][k] = piece p of X(n, k) with
+// the three bf16 planes of a small fp32 matrix, optionally transposed: P[p][n][k] = piece p of alpha * X(n, k) with
 // X(n, k) = B[k][n] (transpose) or B[n][k]; zero outside N x K.  Also clears the flag word.
 __global__ void __launch_bounds__(256) split_planes_kernel(const float *__restrict__ B, int64_t ldb, int transpose, int64_t N,
                                                            int64_t K, int64_t Np, int64_t Kp, uint16_t *__restrict__ P,
-                                                           unsigned *__restrict__ flag)
+                                                           unsigned *__restrict__ flag, float alpha)
 {
     const int64_t total = Np * Kp;
     if (blockIdx.x == 0 && threadIdx.x == 0) *flag = 0u;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t n = i / Kp, k = i % Kp;
         float x = 0.f;
-        if (n < N && k < K) x = transpose ? B[k * ldb + n] : B[n * ldb + k];
+        if (n < N && k < K) x = (transpose ? B[k * ldb + n] : B[n * ldb + k]) * alpha;  // alpha = 1 leaves the bits alone
         uint32_t p0, p1, p2;
         split2(x, 0.f, p0, p1, p2);
         P[i] = (uint16_t)p0;
@@ -354,7 +351,8 @@ constexpr int kRAPlane = 32 * kRAS;   // bf16 elements of one private plane
 constexpr size_t kRLdsBytes = ((size_t)3 * kRMaxN * kRBS + (size_t)kRWaves * 3 * kRAPlane) * sizeof(uint16_t);
 
 // MASK: 0 none, 1 fp32 values beside A (mask > 0 keeps the element), 2 one bit per element
-template <int TN, int MASK>
+// DROP: dropout after the ReLU, for N a multiple of 8 (a call of the generator then covers 8 columns of one row)
+template <int TN, int MASK, bool DROP = false>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel(const SplitArgs g)
 {
     constexpr bool MASKED = MASK == 1;      // the fp32 mask travels in registers beside its chunk
@@ -520,15 +518,44 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
         const int64_t r0 = panel * 32 + 4 * h;
         float *pc = g.C + r0 * g.ldc + li;
         const int rows_left = (int)min(g.M - r0, (int64_t)32);
+        // Dropout: one call of the generator gives the 16-bit lanes of 8 consecutive columns of a row, and an accumulator
+        // register holds one column of a row, so the keep bits go through LDS: lane (row li, half h) makes the bits of
+        // columns 32 t + 16 h ... + 15 of its row for every tile t (two calls each), stored as halves of the 32-bit word
+        // [t][row] in the private tile (idle between the last product of a panel and the first chunk of the next); a
+        // lane then reads the words of its four consecutive rows with one 128-bit load per four registers.
+        uint32_t *const keep_words = reinterpret_cast<uint32_t *>(apriv);  // [TN][32]
+        if constexpr (DROP) {
+            const uint64_t row = (uint64_t)(panel * 32 + li);
+            const uint64_t q_row = row * (uint64_t)(N >> 3);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                uint32_t bits = 0;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint64_t q = q_row + (uint64_t)(4 * t + 2 * h + j);
+                    const plx::Philox4 rnd = plx::philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), g.off_lo, g.off_hi, g.seed_lo, g.seed_hi);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) bits |= (plx::dropout_lane16(rnd, e) >= g.thresh16 ? 1u : 0u) << (8 * j + e);
+                }
+                reinterpret_cast<uint16_t *>(keep_words)[(t * 32 + li) * 2 + h] = (uint16_t)bits;
+            }
+            plx::wave_lds_fence();
+        }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
             const bool col_ok = li + t * 32 < N;
             uint32_t word = 0;  // lane li < 16 of half h collects the sign bits of row r0 + d(li), columns 32 t ... 32 t + 31
+            u32x4 keep4[4];
+            if constexpr (DROP) {
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) keep4[v4] = *reinterpret_cast<const u32x4 *>(keep_words + t * 32 + 8 * v4 + 4 * h);
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int d = 8 * (v / 4) + (v % 4);
                 float x = acc[t][v];
                 if (relu) x = fmaxf(x, 0.f);
+                if constexpr (DROP) x = ((keep4[v / 4][v % 4] >> li) & 1u) ? x * g.keep_scale : 0.f;
                 if (col_ok && d < rows_left) pc[(int64_t)d * g.ldc + t * 32] = x;
                 if (g.relu_bits != nullptr) {  // one vote of the wavefront gives the words of two rows
                     const uint64_t votes = __ballot(col_ok && x > 0.f);
@@ -538,30 +565,84 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             }
             if (g.relu_bits != nullptr && li < 16) {
                 const int d = 8 * (li / 4) + (li % 4);
-                if (d < rows_left) g.relu_bits[(r0 + d) * g.ldw + t] = word;
+                // a row holds ceil(N / 32) words: tiles that lie past N altogether (N <= 96 under four tiles) have none
+                if (d < rows_left && t * 32 < N) g.relu_bits[(r0 + d) * g.ldw + t] = word;
+            }
+        }
+        if constexpr (DROP) plx::wave_lds_fence();  // the next panel's first chunk overwrites the keep bits
+    }
+}
+
+template <int TN, int MASK, bool DROP = false>
+int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
+{
+    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK, DROP>), kRLdsBytes, allowed);
+    if (rc != PLX_OK) return rc;
+    gemm_split_nt_resident_kernel<TN, MASK, DROP><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    return PLX_OK;
+}
+
+template <int MASK, bool DROP = false>
+int launch_resident_tn(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
+{
+    switch (tn) {
+        case 1: return launch_resident<1, MASK, DROP>(g, blocks, st);
+        case 2: return launch_resident<2, MASK, DROP>(g, blocks, st);
+        default: return launch_resident<4, MASK, DROP>(g, blocks, st);
+    }
+}
+
+// Dropout of a matrix in place, for the products whose kernel does not apply it (weights beyond 128 x 128, widths that
+// are not multiples of 8, the fp32 MFMA kernels): thread i takes call i of the generator, i.e. elements 8 i ... 8 i + 7
+// of the row-major numbering e = row * N + col.  Runs only if *run_if is set (run_if == NULL: always).
+struct DropArgs {
+    uint32_t thresh16, seed_lo, seed_hi, off_lo, off_hi;
+    float keep_scale;
+};
+
+__global__ void __launch_bounds__(256) dropout_f32_kernel(int64_t M, int64_t N, float *__restrict__ X, int64_t ldx, const DropArgs a,
+                                                          const unsigned *__restrict__ run_if)
+{
+    if (run_if != nullptr && *run_if == 0u) return;
+    const uint64_t total = (uint64_t)M * (uint64_t)N;
+    const uint64_t calls = (total + 7) / 8;
+    for (uint64_t q = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; q < calls; q += (uint64_t)gridDim.x * blockDim.x) {
+        const plx::Philox4 rnd = plx::philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
+        uint64_t e = q * 8;
+        uint64_t r = e / (uint64_t)N, c = e % (uint64_t)N;
+#pragma unroll
+        for (int i = 0; i < 8; ++i, ++e) {
+            if (e >= total) break;
+            float *px = X + (int64_t)r * ldx + (int64_t)c;
+            *px = plx::dropout_lane16(rnd, i) >= a.thresh16 ? *px * a.keep_scale : 0.f;
+            if (++c == (uint64_t)N) {
+                c = 0;
+                ++r;
             }
         }
     }
 }
 
-template <int TN, int MASK>
-int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
+int launch_dropout(int64_t M, int64_t N, float *X, int64_t ldx, const DropArgs &a, const unsigned *run_if, hipStream_t st)
 {
-    // more than 64 KB of dynamic LDS has to be allowed per kernel and device (a host-side setting, cheap to repeat)
-    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRLdsBytes));
-    gemm_split_nt_resident_kernel<TN, MASK><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    const int64_t calls = (M * N + 7) / 8;
+    if (calls == 0) return PLX_OK;
+    dropout_f32_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(calls, 256), 1 << 20), 256, 0, st>>>(M, N, X, ldx, a, run_if);
+    PLX_LAUNCH_CHECK("dropout_f32_kernel");
     return PLX_OK;
 }
 
-template <int MASK>
-int launch_resident_tn(const SplitArgs &g, int tn, unsigned blocks, hipStream_t st)
+int drop_args(const char *who, float p, uint64_t seed, uint64_t offset, DropArgs &a)
 {
-    switch (tn) {
-        case 1: return launch_resident<1, MASK>(g, blocks, st);
-        case 2: return launch_resident<2, MASK>(g, blocks, st);
-        default: return launch_resident<4, MASK>(g, blocks, st);
-    }
+    PLX_REQUIRE(p >= 0.f && p < 1.f, "%s: dropout p=%g outside [0, 1)", who, (double)p);
+    a.thresh16 = (uint32_t)std::min<long long>(65535, llroundf(p * 65536.f));
+    a.keep_scale = 1.f / (1.f - p);
+    a.seed_lo = (uint32_t)seed;
+    a.seed_hi = (uint32_t)(seed >> 32);
+    a.off_lo = (uint32_t)offset;
+    a.off_hi = (uint32_t)(offset >> 32);
+    return PLX_OK;
 }
 
 // sign bits of a matrix: word [row * ldw + w] = bits of columns 32 w ... 32 w + 31 (columns past N: 0).  Runs only if
@@ -609,10 +690,15 @@ bool aligned8(const void *p, int64_t ld) { return p == nullptr || (reinterpret_c
 int64_t round_up(int64_t x, int64_t q) { return (x + q - 1) / q * q; }
 
 // C = epilogue((A*mask) . X^T) with X (N x K) = B^T (transpose_b) or B
+// `drop` (forward only): dropout after the ReLU; `alpha` (backward only): the product is scaled by it, through the
+// planes of the small operand
 int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
             int transpose_b, float *C, int64_t ldc, const float *mask, int64_t ldmask, unsigned flags, void *workspace,
-            size_t workspace_bytes, void *stream, uint32_t *relu_bits = nullptr, const uint32_t *mask_bits = nullptr, int64_t ldw = 0)
+            size_t workspace_bytes, void *stream, uint32_t *relu_bits = nullptr, const uint32_t *mask_bits = nullptr, int64_t ldw = 0,
+            const DropArgs *drop = nullptr, float alpha = 1.f)
 {
+    if (drop == nullptr && (flags & PLX_GEMM_DROPOUT) != 0)  // this entry point carries no p / seed / offset
+        return plx::fail(PLX_ERR_UNSUPPORTED, "%s: PLX_GEMM_DROPOUT needs plx_gemm_nn_f32_split_dropout", who);
     PLX_REQUIRE(M >= 0 && N >= 0 && K > 0 && N < (1ll << 30) && K < (1ll << 30), "%s: bad dimension", who);
     if (M == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(C != nullptr && A != nullptr && B != nullptr, "%s: NULL operand", who);
@@ -635,25 +721,48 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     hipStream_t st = plx::as_stream(stream);
     uint16_t *planes = static_cast<uint16_t *>(workspace);
     unsigned *flag_words = reinterpret_cast<unsigned *>(static_cast<char *>(workspace) + plane_bytes);
+    PLX_REQUIRE(M < (1ll << 40), "%s: too many rows", who);
     split_planes_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(Np * Kp, 256), 4096), 256, 0, st>>>(B, ldb, transpose_b, N, K, Np,
-                                                                                                    Kp, planes, flag_words);
+                                                                                                    Kp, planes, flag_words, alpha);
     PLX_LAUNCH_CHECK("split_planes_kernel");
+    const unsigned mm_flags = flags & ~PLX_GEMM_DROPOUT;  // what the fp32 MFMA launch understands
     // Inf / NaN / values next to FLT_MAX in either operand: the split product is then meaningless and the fp32 MFMA
     // kernel redoes it.  That
     // launch is always enqueued and returns at once unless the flag word is set.
     auto redo = [&]() -> int {
         if (transpose_b) {
-            const int rc = plx::gemm_nn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, flags, flag_words, 1, stream);
+            int rc = plx::gemm_nn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mm_flags, flag_words, 1, stream);
+            if (rc == PLX_OK && drop != nullptr) rc = launch_dropout(M, N, C, ldc, *drop, flag_words, st);
             if (rc != PLX_OK || relu_bits == nullptr) return rc;
             return launch_sign_bits(M, N, C, ldc, relu_bits, ldw, flag_words, st);  // of the C that launch wrote, if it ran
         }
-        return plx::gemm_nt_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, flag_words, 1, stream);
+        return plx::gemm_nt_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, flag_words, 1, stream, alpha);
+    };
+    // dropout that the product's kernel does not apply: a pass over C, and the sign bits after it
+    auto drop_after = [&]() -> int {
+        int rc = launch_dropout(M, N, C, ldc, *drop, nullptr, st);
+        if (rc == PLX_OK && relu_bits != nullptr) rc = launch_sign_bits(M, N, C, ldc, relu_bits, ldw, nullptr, st);
+        return rc;
     };
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
-    g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = flags; g.a_vec = vec;
+    g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = mm_flags; g.a_vec = vec;
     g.nonfinite = flag_words;
     g.ldw = ldw;
+    if (drop != nullptr) {
+        g.thresh16 = drop->thresh16; g.keep_scale = drop->keep_scale;
+        g.seed_lo = drop->seed_lo; g.seed_hi = drop->seed_hi; g.off_lo = drop->off_lo; g.off_hi = drop->off_hi;
+    }
+    if (resident && drop != nullptr) {
+        const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
+        const bool fused = N % 8 == 0;
+        g.relu_bits = fused ? relu_bits : nullptr;
+        int rc = fused ? launch_resident_tn<0, true>(g, tn, blocks, st) : launch_resident_tn<0>(g, tn, blocks, st);
+        if (rc != PLX_OK) return rc;
+        PLX_LAUNCH_CHECK("gemm_split_nt_resident_kernel");
+        if (!fused && (rc = drop_after()) != PLX_OK) return rc;
+        return redo();
+    }
     if (resident) {
         const unsigned blocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
         g.relu_bits = relu_bits;
@@ -673,7 +782,10 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
         if (mask != nullptr) launch_nt<true, 2>(g, tn, blocks, st); else launch_nt<false, 2>(g, tn, blocks, st);
     }
     PLX_LAUNCH_CHECK("gemm_split_nt_kernel");
-    if (relu_bits != nullptr) {  // this kernel does not write them: a pass over C does
+    if (drop != nullptr) {
+        const int rc = drop_after();
+        if (rc != PLX_OK) return rc;
+    } else if (relu_bits != nullptr) {  // this kernel does not write them: a pass over C does
         const int rc = launch_sign_bits(M, N, C, ldc, relu_bits, ldw, nullptr, st);
         if (rc != PLX_OK) return rc;
     }
@@ -723,6 +835,39 @@ int plx_gemm_nt_f32_split_bits(int64_t M, int64_t N, int64_t K, const float *A, 
     PLX_REQUIRE(mask_bits != nullptr, "gemm_nt_split_bits: NULL bit mask");
     return nt_form("gemm_nt_split_bits", M, N, K, A, lda, B, ldb, 0, C, ldc, mask, ldmask, 0u, workspace, workspace_bytes, stream,
                    nullptr, mask_bits, ldw);
+}
+
+int plx_gemm_nn_f32_split_dropout(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                                  int64_t ldc, unsigned flags, float dropout_p, uint64_t seed, uint64_t offset, uint32_t *sign_bits,
+                                  int64_t ldw, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(ldb >= N, "gemm_nn_split_dropout: leading dimension too small");
+    DropArgs d{};
+    const int rc = drop_args("gemm_nn_split_dropout", dropout_p, seed, offset, d);
+    if (rc != PLX_OK) return rc;
+    const bool drop = (flags & PLX_GEMM_DROPOUT) != 0 && dropout_p > 0.f;
+    return nt_form("gemm_nn_split_dropout", M, N, K, A, lda, B, ldb, 1, C, ldc, nullptr, 0, drop ? flags : (flags & ~PLX_GEMM_DROPOUT),
+                   workspace, workspace_bytes, stream, sign_bits, nullptr, ldw, drop ? &d : nullptr);
+}
+
+int plx_gemm_nt_f32_split_scaled(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
+                                 int64_t ldc, const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, float alpha,
+                                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    PLX_REQUIRE(ldb >= K, "gemm_nt_split_scaled: leading dimension too small");
+    return nt_form("gemm_nt_split_scaled", M, N, K, A, lda, B, ldb, 0, C, ldc, mask, ldmask, 0u, workspace, workspace_bytes, stream,
+                   nullptr, mask_bits, ldw, nullptr, alpha);
+}
+
+int plx_dropout_f32(int64_t M, int64_t N, float *X, int64_t ldx, float dropout_p, uint64_t seed, uint64_t offset, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && ldx >= N && M < (1ll << 40) && N < (1ll << 30), "dropout: bad dimension or pitch");
+    if (M == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(X != nullptr, "dropout: NULL operand");
+    DropArgs d{};
+    const int rc = drop_args("dropout", dropout_p, seed, offset, d);
+    if (rc != PLX_OK) return rc;
+    return launch_dropout(M, N, X, ldx, d, nullptr, plx::as_stream(stream));
 }
 
 int plx_sign_bits_f32(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *sign_bits, int64_t ldw, void *stream)

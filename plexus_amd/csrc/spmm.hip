@@ -638,13 +638,28 @@ size_t hub_workspace_bytes(const plx_spmm_plan *plan, int64_t D, int64_t elem)
     return plx::hub::partial_bytes(D);
 }
 
+// scratch of a product of width D whose elements take `elem` bytes: partial rows of the split rows, partial sums of the
+// hub pass, and room for a line-aligned copy of H where contiguous rows of that type would want one
+size_t workspace_need(const plx_spmm_plan *plan, int64_t D, int64_t elem)
+{
+    if (!plan || D <= 0) return 0;
+    const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
+    const int64_t ld_st = wanted_stage_ld(plan, D, elem, 0, D);
+    const size_t hub_bytes = hub_workspace_bytes(plan, D, elem);
+    if (ld_st == 0) return seg_bytes + hub_bytes;
+    return (size_t)kLine + (size_t)plan->K * (size_t)ld_st * (size_t)elem + seg_bytes + hub_bytes;
+}
+
 // `may_stage` = false: the workspace holds the partial rows of the split rows and nothing else (H is gathered where
 // it lies; same values in the same order, so the same result)
 template <typename T>
 int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, const float *val, const T *H, int64_t ldh,
               int64_t D, T *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream, bool may_stage = true,
-              int parts = 3)
+              int parts = 3, int hub_stage = 0)
 {
+    // hub_stage, for a product computed range by range with one workspace: 0 = this call stands alone (a range that holds
+    // a hub row runs the whole pass); 1 = first range of a sequence: the pass runs now, for every hub row, and leaves its
+    // partial sums in the workspace; 2 = a later range: the partial sums are there, only this range's hub rows are added up
     PLX_REQUIRE(plan != nullptr, "spmm: plan is NULL");
     PLX_REQUIRE(row_begin >= 0 && row_begin <= row_end && row_end <= plan->M, "spmm: row range [%lld, %lld) outside [0, %lld)",
                 (long long)row_begin, (long long)row_end, (long long)plan->M);
@@ -653,9 +668,11 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     PLX_REQUIRE((val || plan->nnz == 0) && H && Y, "spmm: NULL operand (val=%p H=%p Y=%p)", (const void *)val, (const void *)H, (void *)Y);
     PLX_REQUIRE(ldh >= D && ldy >= D, "spmm: leading dimension smaller than D (ldh=%lld ldy=%lld D=%lld)",
                 (long long)ldh, (long long)ldy, (long long)D);
+    // sized for this element type: the hub pass and the column slices go by the bytes of a row, so a bf16 product may
+    // need room that the fp32 product of the same width does not (each type has its size query)
     const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
     const size_t hub_bytes = may_stage ? hub_workspace_bytes(plan, D, sizeof(T)) : 0;
-    const size_t need = may_stage ? plx_spmm_workspace_bytes(plan, D) : seg_bytes;
+    const size_t need = may_stage ? workspace_need(plan, D, sizeof(T)) : seg_bytes;
     if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return plx::fail(PLX_ERR_WORKSPACE, "spmm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     PLX_REQUIRE(need == 0 || (reinterpret_cast<uintptr_t>(workspace) % 16) == 0, "spmm: workspace not 16-byte aligned");
@@ -701,13 +718,13 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     // (4-element vectors at 32-bit byte offsets).  The choice looks at the operand as the caller passed it, so a whole
     // product and a row range of it choose alike, and a row range runs the whole pass when it holds a hub row: the sums
     // of a hub row are then the same bits whatever range it is computed in and wherever H is gathered from.
-    bool use_hub = false;
+    bool use_hub = false, hub_in_range = false;
     const T *hub_h = H0;
     int64_t hub_ldh = ldh0;
     if (hub_bytes > 0) {
         const auto &hr = plan->hub.h_rows_sorted;
-        const bool any = std::lower_bound(hr.begin(), hr.end(), (int32_t)row_begin) != std::lower_bound(hr.begin(), hr.end(), (int32_t)row_end);
-        use_hub = any && D % 4 == 0 && ldh0 % 4 == 0 && reinterpret_cast<uintptr_t>(H0) % (4 * sizeof(T)) == 0 &&
+        hub_in_range = std::lower_bound(hr.begin(), hr.end(), (int32_t)row_begin) != std::lower_bound(hr.begin(), hr.end(), (int32_t)row_end);
+        use_hub = (hub_in_range || hub_stage == 1) && D % 4 == 0 && ldh0 % 4 == 0 && reinterpret_cast<uintptr_t>(H0) % (4 * sizeof(T)) == 0 &&
                   plan->K * ldh0 * kElem < plx::hub::kHubMaxBytes;
         if (h_is_staged && plan->K * ldh * kElem < plx::hub::kHubMaxBytes) {
             hub_h = H;
@@ -715,9 +732,13 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
         }
     }
     float *hub_partial = reinterpret_cast<float *>(ws_base + seg_bytes);  // seg_bytes is a multiple of 16
+    if (use_hub && (ws_base == nullptr || (size_t)(ws_base - static_cast<char *>(workspace)) + seg_bytes + hub_bytes > workspace_bytes))
+        return plx::fail(PLX_ERR_WORKSPACE, "spmm: the partial sums of the hub pass need %zu bytes behind the %zu of the split rows, %zu given",
+                         hub_bytes, seg_bytes, workspace_bytes);
     auto hub_pass = [&]() -> int {
         if (!use_hub || !(parts & 2)) return PLX_OK;
-        return plx::hub::launch(plan->hub, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st);
+        return plx::hub::launch(plan->hub, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st,
+                                /*run_pass=*/hub_stage != 2, /*run_reduce=*/hub_in_range);
     };
 
     SpmmArgs a;
@@ -972,7 +993,8 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
     // rows: 7.3 ms without, 5.7 ms with.
     if (t.n_long > 0 && M > 0 && nnz / M < 128 && K * 512 >= (128ll << 20)) {
         const int hrc = build_hub(p, nnz / 8, st);
-        if (hrc != PLX_OK && hrc != PLX_ERR_NOMEM) {  // no room for the tables: the plan works without them
+        // no room for the tables, or rows whose columns do not ascend: the plan works without them
+        if (hrc != PLX_OK && hrc != PLX_ERR_NOMEM && hrc != PLX_ERR_UNSUPPORTED) {
             plx_spmm_plan_destroy(p);
             return hrc;
         }
@@ -1038,17 +1060,10 @@ int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host
     return PLX_OK;
 }
 
-size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D)
-{
-    if (!plan || D <= 0) return 0;
-    const size_t seg_bytes = (size_t)plan->n_seg * (size_t)ws_ld(D) * sizeof(float);
-    // room for the line-aligned copy of H, decided for contiguous fp32 rows (an operand laid out otherwise is staged
-    // only if it fits what the caller brought)
-    const int64_t ld_st = wanted_stage_ld(plan, D, 4, 0, D);
-    const size_t hub_bytes = hub_workspace_bytes(plan, D, 4);
-    if (ld_st == 0) return seg_bytes + hub_bytes;
-    return (size_t)kLine + (size_t)plan->K * (size_t)ld_st * sizeof(float) + seg_bytes + hub_bytes;
-}
+// The room for the line-aligned copy of H is decided for contiguous rows of the element type (an operand laid out
+// otherwise is staged only if it fits what the caller brought).
+size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D) { return workspace_need(plan, D, 4); }
+size_t plx_spmm_workspace_bytes_bf16(const plx_spmm_plan *plan, int64_t D) { return workspace_need(plan, D, 2); }
 
 int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode)
 {
@@ -1069,6 +1084,12 @@ int plx_spmm_csr_rows_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t 
                           void *stream)
 {
     return spmm_impl<float>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+int plx_spmm_csr_chunk_f32(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, int first_chunk, const float *val, const float *H,
+                           int64_t ldh, int64_t D, float *Y, int64_t ldy, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_impl<float>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream, true, 3, first_chunk ? 1 : 2);
 }
 
 size_t plx_spmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
@@ -1138,6 +1159,13 @@ int plx_spmm_csr_rows_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t
                            void *stream)
 {
     return spmm_impl<uint16_t>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream);
+}
+
+int plx_spmm_csr_chunk_bf16(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, int first_chunk, const float *val,
+                            const uint16_t *H, int64_t ldh, int64_t D, uint16_t *Y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                            void *stream)
+{
+    return spmm_impl<uint16_t>(plan, row_begin, row_end, val, H, ldh, D, Y, ldy, workspace, workspace_bytes, stream, true, 3, first_chunk ? 1 : 2);
 }
 
 }  // extern "C"

@@ -66,9 +66,12 @@ size_t partial_bytes(int64_t D);
 
 // One pass: Y[r] for the hub rows r in [row_begin, row_end).  `d_read` = columns of a row of H that may be read (a
 // multiple of kHubVec: D itself, or D rounded up where the row pitch covers it).  Rows of H: K * ldh * sizeof(T) <
-// kHubMaxBytes, 16-byte aligned (fp32) or 8-byte aligned (bf16) base and pitch.
+// kHubMaxBytes, 16-byte aligned (fp32) or 8-byte aligned (bf16) base and pitch.  `run_pass`: compute the partial sums of
+// every hub row into `partial` (false: they are there from an earlier call with the same operands); `run_reduce`: add
+// up the hub rows of the range.
 int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *H, int64_t ldh, int64_t D, int64_t d_read, bool bf16,
-           int64_t row_begin, int64_t row_end, void *Y, int64_t ldy, float *partial, hipStream_t st);
+           int64_t row_begin, int64_t row_end, void *Y, int64_t ldy, float *partial, hipStream_t st, bool run_pass = true,
+           bool run_reduce = true);
 
 }  // namespace hub
 }  // namespace plx

@@ -496,6 +496,23 @@ __global__ void __launch_bounds__(256) row_lengths_kernel(int64_t n, const int32
     if (i < n) len[i] = rowptr[rows[i] + 1] - rowptr[rows[i]];
 }
 
+// The streams are cut out of a row by bisection over its columns, so the columns of a hub row must ascend (equal
+// neighbours are harmless).  One workgroup per split row; *unsorted receives the number of rows that do not comply.
+__global__ void __launch_bounds__(256) rows_ascend_kernel(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
+                                                          const int32_t *__restrict__ rows, int32_t *__restrict__ unsorted)
+{
+    __shared__ int bad;
+    if (threadIdx.x == 0) bad = 0;
+    __syncthreads();
+    const int32_t r = rows[blockIdx.x];
+    const int32_t a = rowptr[r], b = rowptr[r + 1];
+    int mine = 0;
+    for (int32_t i = a + 1 + (int32_t)threadIdx.x; i < b; i += (int32_t)blockDim.x) mine |= col[i] < col[i - 1] ? 1 : 0;
+    if (mine) bad = 1;  // every writer stores the same value
+    __syncthreads();
+    if (threadIdx.x == 0 && bad) atomicAdd(unsorted, 1);
+}
+
 struct DeviceBlock {  // freed on every way out
     void *p = nullptr;
     ~DeviceBlock()
@@ -505,17 +522,22 @@ struct DeviceBlock {  // freed on every way out
 };
 
 template <typename T, int VEC, int LPR>
-int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st)
+int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st, bool run_pass, bool run_reduce)
 {
     constexpr int TW = LPR * VEC;
     const size_t shm = ((size_t)kWaves * kHubRowsPerWave * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2) + kWaves * sizeof(int);
-    PLX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)shm));
+    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR>), shm, allowed);
+    if (rc != PLX_OK) return rc;
     dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, TW), 1);
-    spmm_hub_kernel<T, VEC, LPR><<<grid, kThreads, shm, st>>>(a);
-    PLX_LAUNCH_CHECK("spmm_hub_kernel");
-    spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 256, 0, st>>>(a, static_cast<T *>(Y), ldy);
-    PLX_LAUNCH_CHECK("spmm_hub_reduce_kernel");
+    if (run_pass) {
+        spmm_hub_kernel<T, VEC, LPR><<<grid, kThreads, shm, st>>>(a);
+        PLX_LAUNCH_CHECK("spmm_hub_kernel");
+    }
+    if (run_reduce) {
+        spmm_hub_reduce_kernel<T><<<(unsigned)a.n_rows, 256, 0, st>>>(a, static_cast<T *>(Y), ldy);
+        PLX_LAUNCH_CHECK("spmm_hub_reduce_kernel");
+    }
     return PLX_OK;
 }
 
@@ -540,16 +562,24 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     out = HubPlan();
     if (n_long <= 0 || K <= 0 || nnz <= 0) return PLX_OK;
 
-    // lengths of the split rows, to the host
-    std::vector<int32_t> len((size_t)n_long);
+    // lengths of the split rows, and whether their columns ascend, to the host
+    std::vector<int32_t> len((size_t)n_long + 1);
     {
         DeviceBlock d_len;
-        PLX_HIP_CHECK(hipMalloc(&d_len.p, sizeof(int32_t) * (size_t)n_long));
-        row_lengths_kernel<<<(unsigned)ceil_div(n_long, 256), 256, 0, st>>>(n_long, rowptr, long_rows, static_cast<int32_t *>(d_len.p));
+        PLX_HIP_CHECK(hipMalloc(&d_len.p, sizeof(int32_t) * ((size_t)n_long + 1)));
+        int32_t *d = static_cast<int32_t *>(d_len.p);
+        PLX_HIP_CHECK(hipMemsetAsync(d + n_long, 0, sizeof(int32_t), st));
+        row_lengths_kernel<<<(unsigned)ceil_div(n_long, 256), 256, 0, st>>>(n_long, rowptr, long_rows, d);
         PLX_LAUNCH_CHECK("row_lengths_kernel");
-        PLX_HIP_CHECK(hipMemcpyAsync(len.data(), d_len.p, sizeof(int32_t) * (size_t)n_long, hipMemcpyDeviceToHost, st));
+        rows_ascend_kernel<<<(unsigned)n_long, 256, 0, st>>>(rowptr, col, long_rows, d + n_long);
+        PLX_LAUNCH_CHECK("rows_ascend_kernel");
+        PLX_HIP_CHECK(hipMemcpyAsync(len.data(), d_len.p, sizeof(int32_t) * ((size_t)n_long + 1), hipMemcpyDeviceToHost, st));
         PLX_HIP_CHECK(hipStreamSynchronize(st));
     }
+    if (len[(size_t)n_long] != 0)
+        return plx::fail(PLX_ERR_UNSUPPORTED, "hub plan: the columns of %d of the %lld split rows do not ascend; the hub pass needs them sorted "
+                         "within each row (the products without it do not)", len[(size_t)n_long], (long long)n_long);
+    len.pop_back();
     // longest first (ties: lower row first); a row takes ceil(len / part_len) slots, rows are taken while slots last
     std::vector<int32_t> order((size_t)n_long);
     std::iota(order.begin(), order.end(), 0);
@@ -696,7 +726,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
 }
 
 int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *H, int64_t ldh, int64_t D, int64_t d_read, bool bf16,
-           int64_t row_begin, int64_t row_end, void *Y, int64_t ldy, float *partial, hipStream_t st)
+           int64_t row_begin, int64_t row_end, void *Y, int64_t ldy, float *partial, hipStream_t st, bool run_pass, bool run_reduce)
 {
     PLX_REQUIRE(hp.block != nullptr && partial != nullptr, "hub pass: no tables or no room for the partial sums");
     PLX_REQUIRE(d_read % kHubVec == 0 && d_read <= ldh, "hub pass: readable width %lld", (long long)d_read);
@@ -725,8 +755,8 @@ int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *
     a.ldp = ceil_div(D, kHubTile) * kHubTile;  // every kernel's tile divides kHubTile
     // fp32 rows of at most 256 bytes are read by a quarter of a wavefront, four entries per load instruction
     // (bf16 rows read 16 bytes per lane by a quarter of a wavefront were measured too: no faster than 8 bytes by a half)
-    if (!bf16) return D <= 64 ? launch_t<float, 4, 16>(a, Y, ldy, st) : launch_t<float, 4, 32>(a, Y, ldy, st);
-    return launch_t<uint16_t, 4, 32>(a, Y, ldy, st);
+    if (!bf16) return D <= 64 ? launch_t<float, 4, 16>(a, Y, ldy, st, run_pass, run_reduce) : launch_t<float, 4, 32>(a, Y, ldy, st, run_pass, run_reduce);
+    return launch_t<uint16_t, 4, 32>(a, Y, ldy, st, run_pass, run_reduce);
 }
 
 }  // namespace hub

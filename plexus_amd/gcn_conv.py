@@ -67,8 +67,8 @@ class GCNConvFunction(torch.autograd.Function):
         A = ops.as_csr(edge_index)
         At = ops.as_csr(edge_index_t)
         bf16 = x.dtype == torch.bfloat16
-        if dropout_p > 0.0 and not (bf16 and fuse_relu):
-            raise ValueError("fused dropout needs bf16 storage and fuse_relu=True")
+        if dropout_p > 0.0 and not fuse_relu:
+            raise ValueError("fused dropout follows the fused ReLU: it needs fuse_relu=True")
 
         # layer-0 features arrive flat (plexus/gcn_conv.py:176-180)
         H = x.detach().reshape(local_features_shape)
@@ -87,8 +87,9 @@ class GCNConvFunction(torch.autograd.Function):
             OUT = ops.gemm_nt_bf16(AGG, ops.cast_bf16(W, transpose=True), relu=fuse_relu, dropout_p=dropout_p,
                                    seed=dropout_seed, offset=dropout_offset)
         elif fuse_relu:
-            # the ReLU mask also as one bit per element, written by the product itself: GRAD_AGG reads it in place of OUT
-            OUT, BITS = ops.gemm_nn(AGG, W, relu=True, want_bits=True)
+            # the mask (ReLU, and dropout where it applies) also as one bit per element, written by the product itself:
+            # GRAD_AGG reads it in place of OUT
+            OUT, BITS = ops.gemm_nn(AGG, W, relu=True, want_bits=True, dropout_p=dropout_p, seed=dropout_seed, offset=dropout_offset)
         else:
             OUT = ops.gemm_nn(AGG, W)
         timers.stop("OUT = AGG * W")
@@ -205,7 +206,7 @@ class GCNConvFunction(torch.autograd.Function):
             if ctx.bf16:
                 grad_weight = ops.gemm_tn_bf16(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
             else:
-                grad_weight = ops.gemm_tn(agg, grad_output, mask=mask)
+                grad_weight = ops.gemm_tn(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
             grad_weight = grad_weight.reshape(weight.shape)
             timers.stop("GRAD_W = AGG.T * GRAD_OUT")
 
@@ -215,7 +216,7 @@ class GCNConvFunction(torch.autograd.Function):
             if ctx.bf16:
                 grad_agg = ops.gemm_nt_bf16(grad_output, ops.cast_bf16(W), mask=mask, alpha=ctx.grad_scale)
             else:
-                grad_agg = ops.gemm_nt(grad_output, W, mask=mask, mask_bits=bits)
+                grad_agg = ops.gemm_nt(grad_output, W, mask=mask, mask_bits=bits, alpha=ctx.grad_scale)
             timers.stop("GRAD_AGG = GRAD_OUT * W.T")
 
             timers.start("GRAD_H = A.T * GRAD_AGG")
@@ -236,7 +237,7 @@ class GCNConv(torch.nn.Module):
     generator, so that a seed reproduces the same weights on any device -- or taken from ``weight``.
 
     Additions: ``association`` selects the order of the two products (see above; the default is the
-    reference's); ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (bf16 storage only) drops
+    reference's); ``fuse_relu`` folds the model's ReLU into the layer; ``dropout`` (with ``fuse_relu``) drops
     activations after the ReLU in training mode with a counter-based generator keyed by ``dropout_seed``;
     every training forward uses a fresh offset (``layer_num + 64 * call count``), which is a host-side
     counter: a recorded HIP graph replays the mask it was recorded with.  The storage type follows the

@@ -137,6 +137,11 @@ class CsrMatrix:
     def hub_entries(self) -> int:
         return int(_lib.load().plx_spmm_plan_info(self._plan, 7))
 
+    @property
+    def hub_table_bytes(self) -> int:
+        """Device memory the plan holds for the hub pass (the streams: 5 bytes per stored entry), 0 without one."""
+        return max(0, int(_lib.load().plx_spmm_plan_info(self._plan, 8)))
+
     def build_hub(self) -> None:
         """Builds the tables of the hub pass whatever the library's size rule says (it builds them by itself for large
         power-law matrices): the longest rows then walk the columns together, sharing the rows of H through L2."""
@@ -149,8 +154,10 @@ class CsrMatrix:
         check(_lib.load().plx_spmm_plan_set_hub(self._plan, int(mode)), "plx_spmm_plan_set_hub")
         self._ws = None
 
-    def _workspace(self, d: int):
-        need = int(_lib.load().plx_spmm_workspace_bytes(self._plan, d))
+    def _workspace(self, d: int, dtype=torch.float32):
+        lib = _lib.load()
+        query = lib.plx_spmm_workspace_bytes_bf16 if dtype == torch.bfloat16 else lib.plx_spmm_workspace_bytes
+        need = int(query(self._plan, d))
         if need == 0:
             return None, 0
         if self._ws is None or self._ws.numel() < need:
@@ -293,7 +300,7 @@ def spmm(a, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor
     d = h.shape[1]
     if out is None:
         out = torch.empty((m, d), dtype=h.dtype, device=h.device)
-    ws, ws_bytes = a._workspace(d)
+    ws, ws_bytes = a._workspace(d, h.dtype)
     lib = _lib.load()
     fn = {torch.float32: lib.plx_spmm_csr_f32, torch.bfloat16: lib.plx_spmm_csr_bf16}.get(h.dtype)
     if fn is None:
@@ -311,14 +318,14 @@ def spmm(a, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor
 def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk=None) -> torch.Tensor:
     """Row-chunked Y = A.H with the reference's chunk boundaries (plexus/gcn_conv.py:77-91).
 
-    Each chunk is one launch writing its rows of the full output; ``on_chunk(i, (start, end), y)`` is called after
-    chunk i has been enqueued (the place where the reference starts the chunk's all-reduce, gcn_conv.py:103-110).
-    The rows are bit-identical to the un-chunked product."""
+    Each chunk is one launch writing its rows of the full output (the hub pass of a plan that has one runs with the first
+    chunk, for all of them); ``on_chunk(i, (start, end), y)`` is called after chunk i has been enqueued (the place where
+    the reference starts the chunk's all-reduce, gcn_conv.py:103-110).  The rows are bit-identical to the un-chunked product."""
     a = as_csr(a)
     _need_gpu(h)
     h = _rowmajor(h)
     lib = _lib.load()
-    fn = {torch.float32: lib.plx_spmm_csr_rows_f32, torch.bfloat16: lib.plx_spmm_csr_rows_bf16}.get(h.dtype)
+    fn = {torch.float32: lib.plx_spmm_csr_chunk_f32, torch.bfloat16: lib.plx_spmm_csr_chunk_bf16}.get(h.dtype)
     if fn is None:
         raise TypeError("chunked_spmm: unsupported dtype %s" % h.dtype)
     m, k = a.shape
@@ -326,16 +333,16 @@ def chunked_spmm(a, h: torch.Tensor, max_rows_per_chunk: int = 1000000, on_chunk
         raise ValueError("chunked_spmm: A is %dx%d but H has %d rows" % (m, k, h.shape[0]))
     d = h.shape[1]
     y = torch.empty((m, d), dtype=h.dtype, device=h.device)
-    ws, ws_bytes = a._workspace(d)
+    ws, ws_bytes = a._workspace(d, h.dtype)
     num_chunks = max(1, (m + max_rows_per_chunk - 1) // max_rows_per_chunk)
     rows_per_chunk = m // num_chunks
     for i in range(num_chunks):
         start = i * rows_per_chunk
         end = m if i == num_chunks - 1 else (i + 1) * rows_per_chunk
         check(
-            fn(a._plan, start, end, a.val.data_ptr(), h.data_ptr(), _ld(h), d, y.data_ptr(), _ld(y),
+            fn(a._plan, start, end, int(i == 0), a.val.data_ptr(), h.data_ptr(), _ld(h), d, y.data_ptr(), _ld(y),
                ws.data_ptr() if ws is not None else None, ws_bytes, _stream()),
-            "plx_spmm_csr_rows",
+            "plx_spmm_csr_chunk",
         )
         if on_chunk is not None:
             on_chunk(i, (start, end), y)
@@ -377,9 +384,23 @@ def sign_bits(x: torch.Tensor) -> torch.Tensor:
     return bits
 
 
-def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None, want_bits: bool = False):
-    """C = A.B, optionally max(C, 0); ``out`` may be a column slice of a wider matrix.  With ``want_bits`` the result is
-    (C, sign bits of C as by ``sign_bits``): the ReLU mask of the layer in the form ``gemm_nt(mask_bits=)`` reads."""
+def dropout_(x: torch.Tensor, p: float, seed: int = 0, offset: int = 0) -> torch.Tensor:
+    """In-place dropout of an fp32 matrix with the counter-based mask of the fused products (kept elements scaled by
+    1 / (1 - p)); the form the products use for operands their kernels do not take."""
+    _need_gpu(x)
+    _need_fp32("dropout_", x=x)
+    if x.dim() != 2 or (x.shape[1] > 1 and x.stride(1) != 1):
+        raise ValueError("dropout_: a 2-D tensor with contiguous rows is expected")
+    check(_lib.load().plx_dropout_f32(x.shape[0], x.shape[1], x.data_ptr(), _ld(x), float(p), int(seed), int(offset), _stream()),
+          "plx_dropout_f32")
+    return x
+
+
+def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[torch.Tensor] = None, want_bits: bool = False,
+            dropout_p: float = 0.0, seed: int = 0, offset: int = 0):
+    """C = A.B, optionally max(C, 0), optionally dropout after that (the mask of ``gemm_nt_bf16``); ``out`` may be a column
+    slice of a wider matrix.  With ``want_bits`` the result is (C, sign bits of C as by ``sign_bits``): the mask of the
+    layer (ReLU and dropout) in the form ``gemm_nt(mask_bits=)`` reads."""
     _need_gpu(a, b, out)
     _need_fp32("gemm_nn", a=a, b=b)
     a, b = _rowmajor(a), _rowmajor(b)
@@ -393,6 +414,25 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
         c = out
         if tuple(c.shape) != (m, n) or c.dtype != torch.float32 or (n > 1 and c.stride(1) != 1):
             raise ValueError("gemm_nn: out must be fp32 [%d x %d] with contiguous rows" % (m, n))
+    if dropout_p > 0.0:
+        bits = _new_bits(m, n, a.device) if want_bits else None
+        if _split_ok(n, k, a):
+            ws, need = _split_ws(n, k, a.device)
+            check(
+                _lib.load().plx_gemm_nn_f32_split_dropout(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                                          (PLX_GEMM_RELU if relu else 0) | PLX_GEMM_DROPOUT, float(dropout_p), int(seed),
+                                                          int(offset), bits.data_ptr() if want_bits else None,
+                                                          _ld(bits) if want_bits else 0, ws.data_ptr(), need, _stream()),
+                "plx_gemm_nn_f32_split_dropout",
+            )
+            return (c, bits) if want_bits else c
+        check(
+            _lib.load().plx_gemm_nn_f32(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                        PLX_GEMM_RELU if relu else 0, _stream()),
+            "plx_gemm_nn_f32",
+        )
+        dropout_(c, dropout_p, seed, offset)
+        return (c, sign_bits(c)) if want_bits else c
     if _split_ok(n, k, a):
         ws, need = _split_ws(n, k, a.device)
         if want_bits:
@@ -418,9 +458,13 @@ def gemm_nn(a: torch.Tensor, b: torch.Tensor, relu: bool = False, out: Optional[
     return (c, sign_bits(c)) if want_bits else c
 
 
+def _device_scalar(value: float, device) -> torch.Tensor:
+    return torch.full((1,), float(value), dtype=torch.float32, device=device)
+
+
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None,
-            mask_bits: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """C = (A * [mask > 0]).B^T with B stored [N x K].  ``mask_bits`` (``sign_bits(mask)``, or the second result of
+            mask_bits: Optional[torch.Tensor] = None, alpha: float = 1.0) -> torch.Tensor:
+    """C = alpha * (A * [mask > 0]).B^T with B stored [N x K].  ``mask_bits`` (``sign_bits(mask)``, or the second result of
     ``gemm_nn(want_bits=True)``) lets the product read the mask as one bit per element where its kernel can."""
     _need_gpu(a, b, mask)
     _need_fp32("gemm_nt", a=a, b=b, mask=mask)
@@ -438,6 +482,18 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
         if mask is None or mask_bits.dtype != torch.int32 or mask_bits.dim() != 2 or mask_bits.shape[0] != m or \
                 mask_bits.shape[1] < (k + 31) // 32 or mask_bits.stride(1) != 1:
             raise ValueError("gemm_nt: mask_bits must be int32 [%d x >= %d] beside the fp32 mask" % (m, (k + 31) // 32))
+    if _split_ok(n, k, a, mask) and alpha != 1.0:
+        ws, need = _split_ws(n, k, a.device)
+        check(
+            _lib.load().plx_gemm_nt_f32_split_scaled(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                                     mask.data_ptr() if mask is not None else None,
+                                                     _ld(mask) if mask is not None else 0,
+                                                     mask_bits.data_ptr() if mask_bits is not None else None,
+                                                     _ld(mask_bits) if mask_bits is not None else 0, float(alpha),
+                                                     ws.data_ptr(), need, _stream()),
+            "plx_gemm_nt_f32_split_scaled",
+        )
+        return c
     if _split_ok(n, k, a, mask):
         ws, need = _split_ws(n, k, a.device)
         if mask_bits is not None:
@@ -461,11 +517,11 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
                                     _ld(mask) if mask is not None else 0, _stream()),
         "plx_gemm_nt_f32",
     )
-    return c
+    return c if alpha == 1.0 else scale_by_scalar(c, _device_scalar(alpha, c.device))  # operands the split kernels do not take
 
 
-def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """C[K x N] = A[M x K]^T.(B * [mask > 0])[M x N]."""
+def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0) -> torch.Tensor:
+    """C[K x N] = alpha * A[M x K]^T.(B * [mask > 0])[M x N]."""
     _need_gpu(a, b, mask)
     _need_fp32("gemm_tn", a=a, b=b, mask=mask)
     a, b = _rowmajor(a), _rowmajor(b)
@@ -487,7 +543,7 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
                             ws.data_ptr() if ws is not None else None, need, _stream()),
         "plx_gemm_tn_f32",
     )
-    return c
+    return c if alpha == 1.0 else scale_by_scalar(c, _device_scalar(alpha, c.device))  # K x N elements: a weight's worth
 
 
 def cast_bf16(x: torch.Tensor, transpose: bool = False) -> torch.Tensor:

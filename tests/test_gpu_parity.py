@@ -441,6 +441,32 @@ def test_relu_mask_as_sign_bits(m, n, k, fp32_gemm_path):
         ops.gemm_nt(gout, w, mask_bits=bits)  # the bits stand for a mask that must be given too
 
 
+@pytest.mark.parametrize("n", [70, 96, 33, 128])
+def test_sign_bits_through_the_raw_entry_point_with_the_smallest_pitch(n):
+    """N in 65..96 runs four column tiles but a row holds three words: with a pitch of exactly ceil(N / 32) words the
+    fourth tile must not write (it would land on the next row's first word, and past the buffer after the last row)."""
+    say("sign bits with ldw = ceil(N / 32), N=%d" % n)
+    from plexus_amd import _lib
+
+    lib = _lib.load()
+    m, k = 1000 + 7, 64
+    words = (n + 31) // 32
+    gen = torch.Generator().manual_seed(n)
+    a = torch.randn(m, k, generator=gen).to(DEV)
+    w = (torch.randn(k, n, generator=gen) * 0.1).to(DEV)
+    c = torch.empty(m, n, device=DEV)
+    guard = 0x5A5A5A5A
+    bits = torch.full((m * words + 8,), guard, dtype=torch.int32, device=DEV)  # rows packed back to back, guard words behind
+    need = int(lib.plx_gemm_f32_split_workspace_bytes(n, k))
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    _lib.check(lib.plx_gemm_nn_f32_split_bits(m, n, k, a.data_ptr(), k, w.data_ptr(), n, c.data_ptr(), n, _lib.PLX_GEMM_RELU,
+                                              bits.data_ptr(), words, ws.data_ptr(), need, torch.cuda.current_stream().cuda_stream),
+               "plx_gemm_nn_f32_split_bits")
+    assert torch.equal(bits[: m * words].reshape(m, words).cpu(), _pack_bits(c.cpu()))
+    assert (bits[m * words:] == guard).all()
+    assert 0.3 < (c > 0).float().mean().item() < 0.7
+
+
 def test_sign_bits_follow_the_product_the_guarded_launch_redoes():
     say("sign bits when an operand holds Inf (the fp32 kernel redoes the product)")
     gen = torch.Generator().manual_seed(9)
@@ -1243,6 +1269,41 @@ def test_spmm_hub_pass_on_random_shapes(seed):
         y = ops.spmm(a, h.to(DEV))
         assert rel_err(y.float().cpu(), ref) <= (FP32_TOL if dtype == torch.float32 else BF16_TOL), (m, k, seg_len, d, dtype)
         assert torch.equal(ops.chunked_spmm(a, h.to(DEV), max_rows_per_chunk=max(1, m // 3)), y)
+
+
+def test_spmm_workspace_covers_the_hub_pass_of_either_storage_type():
+    """With column slicing forced on, 128 fp32 columns (512-byte rows) are sliced and take no hub pass, while 128 bf16
+    columns (256-byte rows) are not sliced and do: each storage type has its size query, and each product checks what it
+    was given against its own."""
+    say("spmm: slicing forced on + hub tables, D=128 in fp32 and bf16")
+    from plexus_amd import _lib
+
+    lib = _lib.load()
+    g, a = _hub_matrix(seed=34)
+    a.set_slicing(1)
+    d = 128
+    seg_bytes = a.n_segments * d * 4
+    partial = 8 * 9216 * 128 * 4  # ranges x slots x columns of the partial sums of a pass
+    need = int(lib.plx_spmm_workspace_bytes_bf16(a._plan, d))
+    assert need >= seg_bytes + partial > int(lib.plx_spmm_workspace_bytes(a._plan, d))  # the fp32 product takes slices, no pass
+    h32 = torch.randn(3000, d, generator=torch.Generator().manual_seed(7))
+    ref = oracle_spmm64(g, h32.to(torch.bfloat16).float())
+    # behind the workspace lies a tensor that must come back untouched
+    arena = torch.zeros(need + (1 << 20), dtype=torch.uint8, device=DEV)
+    arena[need:] = 0xA5
+    hb = h32.to(torch.bfloat16).to(DEV)
+    y = torch.empty(3000, d, dtype=torch.bfloat16, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.plx_spmm_csr_bf16(a._plan, a.val.data_ptr(), hb.data_ptr(), d, d, y.data_ptr(), d, arena.data_ptr(), need, st), "plx_spmm_csr_bf16")
+    assert rel_err(y.float().cpu(), ref) <= BF16_TOL
+    assert (arena[need:] == 0xA5).all()
+    assert torch.equal(ops.spmm(a, hb), y)  # through the front end, which sizes its workspace with the same query
+    # a workspace that holds the partial rows of the split rows only is refused, not overrun
+    rc = lib.plx_spmm_csr_bf16(a._plan, a.val.data_ptr(), hb.data_ptr(), d, d, y.data_ptr(), d, arena.data_ptr(), seg_bytes, st)
+    assert rc == _lib.PLX_ERR_WORKSPACE
+    # the fp32 product of the same width runs in column slices and agrees with the oracle too
+    yf = ops.spmm(a, h32.to(DEV))
+    assert rel_err(yf.cpu(), oracle_spmm64(g, h32)) <= FP32_TOL
 
 
 def test_spmm_hub_pass_is_left_out_where_the_operand_does_not_suit_it():

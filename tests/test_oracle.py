@@ -439,7 +439,7 @@ def test_bf16_oracle_equals_fp32_oracle_when_rounding_is_the_identity():
         out_ref = ref.forward(x, [(a, a_t)])
         gx_ref, gw_ref = ref.backward(g_logits)
         # precondition: everything the bf16 path stores survives the rounding unchanged
-        for agg, _, _, pre in ref._saved:
+        for agg, _, _, pre, _ in ref._saved:
             assert torch.equal(po.rb(agg), agg) and torch.equal(po.rb(pre), pre)
         assert torch.equal(po.rb(gx_ref), gx_ref) and (ref._saved[0][3] > 0).any() and (ref._saved[0][3] < 0).any()
         net = po.OracleNetBf16(ws, dims, dropout_p=0.0)
@@ -571,3 +571,42 @@ def test_bf16_epoch_loop_matches_autograd_training():
     for u_, v_ in zip(wf, wt):
         assert torch.allclose(u_, v_.detach(), rtol=0, atol=1e-12)
     assert losses[0] != losses[1]
+
+
+@pytest.mark.parametrize("p", [0.5, 0.25])
+def test_fp32_oracle_with_dropout_backward_equals_autograd_over_its_forward(p):
+    """OracleNet with dropout after the ReLU: the hand backward == torch.autograd over the plain-operator forward with the
+    keep masks as constant factors (fp64).  Fails if 1/(1-p) is missing or doubled in grad_w or in the gradient handed to
+    the aggregation, if dropped units keep a gradient, or if the last layer is dropped too."""
+    n, dims, seed = 70, [9, 7, 6, 4], 5
+    a = small_graph(n=n, pairs=350, seed=21).double()
+    a_t = a.transpose(0, 1).to_sparse_csr()
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(n * dims[0], generator=gen, dtype=torch.float64)
+    ws = [torch.randn(dims[i] * dims[i + 1], generator=gen, dtype=torch.float64) for i in range(3)]
+    g_logits = torch.randn(n, dims[-1], generator=gen, dtype=torch.float64)
+    offsets = [11, 12, 13]
+    keeps = [torch.from_numpy(po.dropout_keep_mask(n * dims[i + 1], seed, offsets[i], p).reshape(n, dims[i + 1])).double()
+             for i in range(2)]
+    net = po.OracleNet(ws, dims, dropout_p=p, seed=seed)
+    out = net.forward(x, [(a, a_t)], offsets=offsets)
+    gx, gw = net.backward(g_logits)
+
+    xs = x.clone().requires_grad_()
+    wt = [w.clone().requires_grad_() for w in ws]
+    h = xs
+    for i, w in enumerate(wt):
+        h = torch.mm(torch.sparse.mm(a, h.reshape(n, dims[i])), w.reshape(dims[i], dims[i + 1]))
+        if i != 2:
+            h = F.dropout(F.relu(h), 0.0) * keeps[i] / (1.0 - p)
+    assert torch.allclose(out, h.detach(), rtol=1e-14, atol=0)
+    grads = torch.autograd.grad(h, [xs] + wt, g_logits)
+    scale = lambda t: t.abs().max()
+    assert (gx.reshape(-1) - grads[0]).abs().max() <= 1e-13 * scale(grads[0])
+    for u, v in zip(gw, grads[1:]):
+        assert (u - v).abs().max() <= 1e-13 * scale(v) and scale(v) > 0
+    assert abs(float(keeps[0].mean()) - (1.0 - p)) < 0.12  # the mask drops about p of the units
+    assert (net._saved[0][3][keeps[0] == 0] != 0).any()  # ... units that were alive before it
+    # without dropout the class is what it was: same numbers as a net built without the arguments
+    plain, plain0 = po.OracleNet(ws, dims), po.OracleNet(ws, dims, dropout_p=0.0, seed=3)
+    assert torch.equal(plain.forward(x, [(a, a_t)]), plain0.forward(x, [(a, a_t)], offsets=offsets))
