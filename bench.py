@@ -117,6 +117,7 @@ def spmm_record(a, d, dtype, iters, seed=None):
            "gather_GBps": (nnz * 8 + (m + 1) * 4 + nnz * d * elem + m * d * elem) / ms / 1e6,
            "t_roof_ms": max(b / (HBM_PEAK_GBPS * 1e6), flops / (FP32_VECTOR_TFLOPS * 1e9)),
            "roofline_frac": b / ms / 1e6 / HBM_PEAK_GBPS}
+    rec["t_roof_frac"] = rec["t_roof_ms"] / ms  # against max(bytes / HBM peak, flops / fp32 vector peak): differs from roofline_frac at D = 602
     note("spmm %d x %d, nnz %d, D=%d %s: %.3f ms, %.1f GB/s algorithmic (%.2f %% of HBM peak), %.1f GFLOP/s"
          % (m, k, nnz, d, "bf16" if elem == 2 else "fp32", ms, rec["alg_GBps"], 100 * rec["roofline_frac"], rec["GFLOPs"]))
     return rec, h

@@ -117,7 +117,7 @@ int plx_spmm_plan_create(plx_spmm_plan **plan, int64_t M, int64_t K, int64_t nnz
                          const int32_t *col, int32_t seg_len, void *stream);
 int plx_spmm_plan_destroy(plx_spmm_plan *plan);
 /* what == 0: rows, 1: cols, 2: nnz, 3: long rows, 4: segments, 5: seg_len, 6: hub rows, 7: entries in hub rows,
- * 8: bytes of the hub pass's tables */
+ * 8: bytes of the hub pass's tables (both layouts), 9 / 10: hub rows / entries in hub rows of the wide layout */
 int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what);
 /* Copies the plan's tables to host arrays (any of them may be NULL): long rows [long rows], seg_first [long rows + 1],
  * seg_begin / seg_end [segments] -- the layout of plx_spmm_segments_host.  For inspection and tests; synchronous. */
@@ -150,6 +150,16 @@ int plx_spmm_plan_set_slicing(plx_spmm_plan *plan, int mode);
  * mode 0: use the pass where possible (the default), -1: never. */
 int plx_spmm_plan_build_hub(plx_spmm_plan *plan, void *stream);
 int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode);
+/* A second set of tables for bf16 products whose rows of H hold 512 bytes or more (256 columns: the bf16 counterpart of
+ * 128 fp32 columns).  The regular tables give every wavefront 36 sums of 128 columns, so such a product runs them once
+ * per 128-column tile, reading every stream, column index and value again and loading 8 bytes per lane; in this layout
+ * a wavefront owns 18 sums of 256 columns (the same LDS), a hub row is cut into parts of 32 * seg_len entries, and half a
+ * wavefront reads a whole 512-byte row with 16 bytes per lane (2.45 M nodes, 126 M entries, 256 bf16 columns).  Never built by
+ * plx_spmm_plan_create, which does not know the storage type; costs another 5 bytes per entry of a hub row; same
+ * requirements and return values as plx_spmm_plan_build_hub; used when it exists, the mode allows the pass, the width is a
+ * multiple of 8 and H is 16-byte aligned with a pitch that is a multiple of 8 (other operands take the regular tables
+ * by the rule above). */
+int plx_spmm_plan_build_hub_wide(plx_spmm_plan *plan, void *stream);
 /* bytes of scratch an fp32 SpMM of width D needs (plx_spmm_workspace_bytes_bf16: a bf16 one -- the hub pass, the column
  * slices and the copy below go by the bytes of a row, so the two types differ, and a product given less than its own
  * query asks for returns PLX_ERR_WORKSPACE): fp32 partial sums of the split rows, the partial sums

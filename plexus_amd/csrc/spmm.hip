@@ -539,6 +539,7 @@ struct plx_spmm_plan {
     std::vector<int32_t> h_long_rows, h_seg_first;  // host copies, to cut row ranges out of the plan
     int slicing = 0;  // 0: column slices of H where the cost model says so, 1: whenever rows exceed a slice, -1: never
     plx::hub::HubPlan hub;  // tables of the hub pass (empty: no hub pass)
+    plx::hub::HubPlan hub_wide;  // the same in the wide layout, for bf16 rows of 512 bytes and more (empty: those take `hub`)
     int hub_mode = 0;       // 0: hub pass where the tables exist and the operands allow it, -1: never
 };
 
@@ -630,12 +631,31 @@ int64_t wanted_stage_ld(const plx_spmm_plan *plan, int64_t D, int64_t elem, uint
 // rows 3.6 -> 3.1 and 2.3 -> 2.4 ms, 128-byte rows 2.3 -> 2.5 and 1.8 -> 2.1 ms; bf16 rows count by the 256 bytes that the
 // 128 columns of a tile hold (256 columns: 7.3 -> 6.7 and 4.2 -> 4.3 ms).  The rule looks at the plan and the width only,
 // so a whole product and its row ranges choose alike.
+// which tables a product of this width and element size takes: the wide layout for bf16 rows of 512 bytes and more
+// where the plan has it (the operand must also allow 16-byte loads: wide_ok), else the regular one by the rule above
+enum HubChoice { kHubNone = 0, kHubRegular = 1, kHubWide = 2 };
+
+bool hub_regular_pays(const plx_spmm_plan *plan, int64_t D, int64_t elem)
+{
+    if (plan->hub.block == nullptr) return false;
+    const int64_t tile_bytes = std::min<int64_t>(D, plx::hub::kHubTile) * elem;  // of a row of H, per load of the pass
+    return !(tile_bytes < 256 || (tile_bytes < 512 && plan->hub.mean_run < 4.0));
+}
+
+HubChoice hub_choice(const plx_spmm_plan *plan, int64_t D, int64_t elem, bool wide_ok)
+{
+    if (plan->hub_mode < 0 || sliced_plan(plan, D, elem)) return kHubNone;
+    if (elem == 2 && D * elem >= 512 && plan->hub_wide.block != nullptr && wide_ok) return kHubWide;
+    return hub_regular_pays(plan, D, elem) ? kHubRegular : kHubNone;
+}
+
+// sized for whichever tables the operand may turn out to allow
 size_t hub_workspace_bytes(const plx_spmm_plan *plan, int64_t D, int64_t elem)
 {
-    if (plan->hub.block == nullptr || plan->hub_mode < 0 || sliced_plan(plan, D, elem)) return 0;
-    const int64_t tile_bytes = std::min<int64_t>(D, plx::hub::kHubTile) * elem;  // of a row of H, per load of the pass
-    if (tile_bytes < 256 || (tile_bytes < 512 && plan->hub.mean_run < 4.0)) return 0;
-    return plx::hub::partial_bytes(D);
+    size_t bytes = 0;
+    if (hub_choice(plan, D, elem, true) == kHubWide) bytes = plx::hub::partial_bytes(D, true);
+    if (hub_choice(plan, D, elem, false) == kHubRegular) bytes = std::max(bytes, plx::hub::partial_bytes(D, false));
+    return bytes;
 }
 
 // scratch of a product of width D whose elements take `elem` bytes: partial rows of the split rows, partial sums of the
@@ -721,11 +741,19 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
     bool use_hub = false, hub_in_range = false;
     const T *hub_h = H0;
     int64_t hub_ldh = ldh0;
+    const plx::hub::HubPlan *hp = nullptr;
     if (hub_bytes > 0) {
-        const auto &hr = plan->hub.h_rows_sorted;
+        auto fits = [&](int64_t q) {  // q-element vectors at 32-bit byte offsets
+            return D % q == 0 && ldh0 % q == 0 && reinterpret_cast<uintptr_t>(H0) % (q * sizeof(T)) == 0 && plan->K * ldh0 * kElem < plx::hub::kHubMaxBytes;
+        };
+        const HubChoice choice = hub_choice(plan, D, kElem, fits(8));
+        if (choice == kHubWide) hp = &plan->hub_wide;
+        else if (choice == kHubRegular && fits(4)) hp = &plan->hub;
+    }
+    if (hp != nullptr) {
+        const auto &hr = hp->h_rows_sorted;
         hub_in_range = std::lower_bound(hr.begin(), hr.end(), (int32_t)row_begin) != std::lower_bound(hr.begin(), hr.end(), (int32_t)row_end);
-        use_hub = (hub_in_range || hub_stage == 1) && D % 4 == 0 && ldh0 % 4 == 0 && reinterpret_cast<uintptr_t>(H0) % (4 * sizeof(T)) == 0 &&
-                  plan->K * ldh0 * kElem < plx::hub::kHubMaxBytes;
+        use_hub = hub_in_range || hub_stage == 1;
         if (h_is_staged && plan->K * ldh * kElem < plx::hub::kHubMaxBytes) {
             hub_h = H;
             hub_ldh = ldh;
@@ -737,12 +765,12 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
                          hub_bytes, seg_bytes, workspace_bytes);
     auto hub_pass = [&]() -> int {
         if (!use_hub || !(parts & 2)) return PLX_OK;
-        return plx::hub::launch(plan->hub, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st,
+        return plx::hub::launch(*hp, plan->col, val, hub_h, hub_ldh, D, D, sizeof(T) == 2, row_begin, row_end, Y, ldy, hub_partial, st,
                                 /*run_pass=*/hub_stage != 2, /*run_reduce=*/hub_in_range);
     };
 
     SpmmArgs a;
-    a.seg_skip = use_hub ? plan->hub.seg_is_hub : nullptr;
+    a.seg_skip = use_hub ? hp->seg_is_hub : nullptr;
     a.rowptr = plan->rowptr;
     a.col = plan->col;
     a.val = val;
@@ -768,7 +796,7 @@ int spmm_impl(const plx_spmm_plan *plan, int64_t row_begin, int64_t row_end, con
         if (q1 > q0) {
             dim3 rgrid((unsigned)(q1 - q0), (unsigned)plx::ceil_div(d, 64), 1);
             spmm_reduce_split_rows<T><<<rgrid, 256, 0, st>>>(a.ws, a.ldws, plan->long_rows, plan->seg_first, (int32_t)q0, (int32_t)d, y, ldy,
-                                                             use_hub ? plan->hub.long_is_hub : nullptr);
+                                                             use_hub ? hp->long_is_hub : nullptr);
             PLX_LAUNCH_CHECK("spmm_reduce_split_rows");
         }
         return PLX_OK;
@@ -872,15 +900,15 @@ int static_scratch(void **out)
     return PLX_OK;
 }
 
-// the tables of the hub pass, kept when the hub rows hold at least `min_entries` entries
-int build_hub(plx_spmm_plan *p, int64_t min_entries, hipStream_t st)
+// the tables of the hub pass (regular or wide layout), kept when the hub rows hold at least `min_entries` entries
+int build_hub(plx_spmm_plan *p, int64_t min_entries, bool wide, hipStream_t st)
 {
     if (p->n_long == 0) return PLX_OK;
     plx::hub::HubPlan hp;
     const int rc = plx::hub::build_hub_plan(p->M, p->K, p->nnz, p->rowptr, p->col, p->seg_len, p->n_long, p->n_seg, p->long_rows, p->seg_first,
-                                            p->h_long_rows, min_entries, st, hp);
+                                            p->h_long_rows, min_entries, wide, st, hp);
     if (rc != PLX_OK) return rc;
-    p->hub = std::move(hp);
+    (wide ? p->hub_wide : p->hub) = std::move(hp);
     return PLX_OK;
 }
 
@@ -992,7 +1020,7 @@ int plx_spmm_plan_create(plx_spmm_plan **out, int64_t M, int64_t K, int64_t nnz,
     // part of the entries: measured on the 2.45 M-node power-law graph, 128 fp32 columns, 33 % of the entries in hub
     // rows: 7.3 ms without, 5.7 ms with.
     if (t.n_long > 0 && M > 0 && nnz / M < 128 && K * 512 >= (128ll << 20)) {
-        const int hrc = build_hub(p, nnz / 8, st);
+        const int hrc = build_hub(p, nnz / 8, false, st);
         // no room for the tables, or rows whose columns do not ascend: the plan works without them
         if (hrc != PLX_OK && hrc != PLX_ERR_NOMEM && hrc != PLX_ERR_UNSUPPORTED) {
             plx_spmm_plan_destroy(p);
@@ -1007,7 +1035,14 @@ int plx_spmm_plan_build_hub(plx_spmm_plan *plan, void *stream)
 {
     PLX_REQUIRE(plan != nullptr, "plan_build_hub: plan is NULL");
     if (plan->hub.block != nullptr) return PLX_OK;
-    return build_hub(plan, 1, plx::as_stream(stream));
+    return build_hub(plan, 1, false, plx::as_stream(stream));
+}
+
+int plx_spmm_plan_build_hub_wide(plx_spmm_plan *plan, void *stream)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_build_hub_wide: plan is NULL");
+    if (plan->hub_wide.block != nullptr) return PLX_OK;
+    return build_hub(plan, 1, true, plx::as_stream(stream));
 }
 
 int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode)
@@ -1022,6 +1057,7 @@ int plx_spmm_plan_destroy(plx_spmm_plan *plan)
 {
     if (!plan) return PLX_OK;
     plx::hub::free_hub_plan(plan->hub);
+    plx::hub::free_hub_plan(plan->hub_wide);
     if (plan->tables) (void)hipFree(plan->tables);
     delete plan;
     return PLX_OK;
@@ -1039,7 +1075,9 @@ int64_t plx_spmm_plan_info(const plx_spmm_plan *plan, int what)
         case 5: return plan->seg_len;
         case 6: return plan->hub.n_rows;
         case 7: return plan->hub.entries;
-        case 8: return plan->hub.stored * 5;  // bytes of the streams
+        case 8: return (plan->hub.stored + plan->hub_wide.stored) * 5;  // bytes of the streams, both layouts
+        case 9: return plan->hub_wide.n_rows;
+        case 10: return plan->hub_wide.entries;
         default: return -1;
     }
 }

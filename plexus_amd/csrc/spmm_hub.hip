@@ -58,40 +58,57 @@ struct HubArgs {
     const int32_t *row_slot_first;
     const int32_t *row_slots;
     int32_t row_begin, row_end;
-    float *partial;  // [kHubRanges][kHubSlots][ldp]
+    float *partial;  // [kHubRanges][slot_cap][ldp]
     int64_t ldp;
+    int32_t slot_cap;  // slots of the plan's layout (kHubGroups * kWaves * sums per wavefront)
 };
 
+// The VEC elements of a row of H that a lane reads, as they lie in memory: converted to fp32 only where they are added
+// up, so that nothing between a load and its use touches the loaded registers.
 template <typename T, int VEC>
-__device__ __forceinline__ void load_vec(const T *p, float (&o)[VEC])
-{
-    if constexpr (sizeof(T) == 4) {
-        static_assert(VEC == 4, "16 bytes per lane");
-        const float4 t = *reinterpret_cast<const float4 *>(p);
-        o[0] = t.x;
-        o[1] = t.y;
-        o[2] = t.z;
-        o[3] = t.w;
-    } else if constexpr (VEC == 8) {
-        const uint4 t = *reinterpret_cast<const uint4 *>(p);
-        o[0] = __uint_as_float(t.x << 16);
-        o[1] = __uint_as_float(t.x & 0xffff0000u);
-        o[2] = __uint_as_float(t.y << 16);
-        o[3] = __uint_as_float(t.y & 0xffff0000u);
-        o[4] = __uint_as_float(t.z << 16);
-        o[5] = __uint_as_float(t.z & 0xffff0000u);
-        o[6] = __uint_as_float(t.w << 16);
-        o[7] = __uint_as_float(t.w & 0xffff0000u);
-    } else {
-        const uint2 t = *reinterpret_cast<const uint2 *>(p);
-        o[0] = __uint_as_float(t.x << 16);
-        o[1] = __uint_as_float(t.x & 0xffff0000u);
-        o[2] = __uint_as_float(t.y << 16);
-        o[3] = __uint_as_float(t.y & 0xffff0000u);
+struct RawVec;
+template <>
+struct RawVec<float, 4> {
+    float4 r;
+    __device__ __forceinline__ void load(const void *p) { r = *reinterpret_cast<const float4 *>(p); }
+    __device__ __forceinline__ void widen(float (&o)[4]) const
+    {
+        o[0] = r.x;
+        o[1] = r.y;
+        o[2] = r.z;
+        o[3] = r.w;
     }
-}
+};
+template <>
+struct RawVec<uint16_t, 4> {
+    uint2 r;
+    __device__ __forceinline__ void load(const void *p) { r = *reinterpret_cast<const uint2 *>(p); }
+    __device__ __forceinline__ void widen(float (&o)[4]) const
+    {
+        o[0] = __uint_as_float(r.x << 16);
+        o[1] = __uint_as_float(r.x & 0xffff0000u);
+        o[2] = __uint_as_float(r.y << 16);
+        o[3] = __uint_as_float(r.y & 0xffff0000u);
+    }
+};
+template <>
+struct RawVec<uint16_t, 8> {
+    uint4 r;
+    __device__ __forceinline__ void load(const void *p) { r = *reinterpret_cast<const uint4 *>(p); }
+    __device__ __forceinline__ void widen(float (&o)[8]) const
+    {
+        o[0] = __uint_as_float(r.x << 16);
+        o[1] = __uint_as_float(r.x & 0xffff0000u);
+        o[2] = __uint_as_float(r.y << 16);
+        o[3] = __uint_as_float(r.y & 0xffff0000u);
+        o[4] = __uint_as_float(r.z << 16);
+        o[5] = __uint_as_float(r.z & 0xffff0000u);
+        o[6] = __uint_as_float(r.w << 16);
+        o[7] = __uint_as_float(r.w & 0xffff0000u);
+    }
+};
 
-// One wavefront = one stream: the entries of its kHubRowsPerWave slots inside its range of columns, window after
+// One wavefront = one stream: the entries of its RPW slots inside its range of columns, window after
 // window, written out by the plan as positions in the CSR arrays (stream_pos) and slot numbers (stream_run), padded
 // to whole batches of 64.  A batch moves through four stages, one per turn of the loop, so that no load is waited for
 // in the turn that issues it: positions and slots (coalesced) -> column and value of every entry (gathered) -> byte
@@ -102,7 +119,7 @@ __device__ __forceinline__ void load_vec(const T *p, float (&o)[VEC])
 // loads of one set of steps in flight while the set before is added up.  Every turn issues the same
 // loads whatever it finds (past the end of the stream they repeat its last batch), so the counter of outstanding
 // loads the hardware waits on has a fixed meaning.
-template <typename T, int VEC, int LPR>
+template <typename T, int VEC, int LPR, int RPW>
 __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -124,15 +141,15 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
     const bool ok = d0 + VEC <= p.d_read;
     const int off = ok ? d0 : 0;
 
-    float *acc = lds + (size_t)wave * kHubRowsPerWave * TW;  // [kHubRowsPerWave][TW], this wavefront's sums
-    uint2 *ring = reinterpret_cast<uint2 *>(lds + (size_t)kWaves * kHubRowsPerWave * TW) + wave * 3 * kWave;  // [3][64] (offset, value)
-    for (int i = lane; i < kHubRowsPerWave * TW; i += kWave) acc[i] = 0.f;
+    float *acc = lds + (size_t)wave * RPW * TW;  // [RPW][TW], this wavefront's sums
+    uint2 *ring = reinterpret_cast<uint2 *>(lds + (size_t)kWaves * RPW * TW) + wave * 3 * kWave;  // [3][64] (offset, value)
+    for (int i = lane; i < RPW * TW; i += kWave) acc[i] = 0.f;
     // window each wavefront of the workgroup is in (pacing, below)
-    int *progress = reinterpret_cast<int *>(reinterpret_cast<uint2 *>(lds + (size_t)kWaves * kHubRowsPerWave * TW) + kWaves * 3 * kWave);
+    int *progress = reinterpret_cast<int *>(reinterpret_cast<uint2 *>(lds + (size_t)kWaves * RPW * TW) + kWaves * 3 * kWave);
     if (lane == 0) progress[wave] = 0;
     __syncthreads();
 
-    const int slot0 = (group * kWaves + wave) * kHubRowsPerWave;
+    const int slot0 = (group * kWaves + wave) * RPW;
     const int stream = (range * kHubGroups + group) * kWaves + wave;
     const int64_t sbase = p.stream_first[stream];
     const int total = p.stream_total[stream];
@@ -174,15 +191,15 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
             plx::wave_lds_fence();
             return z;
         };
-        struct Rows { float h[U][VEC]; float v[U]; };
+        struct Rows { RawVec<T, VEC> h[U]; float v[U]; };
         auto fetch = [&](const Ready &z, int g, Rows &r) {
 #pragma unroll
             for (int u = 0; u < U; u += 2) {
                 const uint4 e = *reinterpret_cast<const uint4 *>(z.mine + g * U + u);  // two entries of this group
                 r.v[u] = __uint_as_float(e.y);
                 r.v[u + 1] = __uint_as_float(e.w);
-                load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.x + lane_off)), r.h[u]);
-                load_vec<T, VEC>(reinterpret_cast<const T *>(Hb + (e.z + lane_off)), r.h[u + 1]);
+                r.h[u].load(Hb + (e.x + lane_off));
+                r.h[u + 1].load(Hb + (e.z + lane_off));
             }
         };
         int cur = -1;  // the slot this group is summing
@@ -225,8 +242,10 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
                     }
                 }
                 if (!decltype(checked)::value || grp * STEPS + i < z.left) {
+                    float hv[VEC];
+                    r.h[u].widen(hv);
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) sum[k] = fmaf(r.v[u], r.h[u][k], sum[k]);
+                    for (int k = 0; k < VEC; ++k) sum[k] = fmaf(r.v[u], hv[k], sum[k]);
                 }
             }
         };
@@ -304,9 +323,9 @@ __global__ void __launch_bounds__(kThreads, 1) spmm_hub_kernel(const HubArgs p)
 
     // the sums of this range: P[range][slot][ldp]
     if (grp == 0 && ok) {
-        for (int r = 0; r < kHubRowsPerWave; ++r) {
+        for (int r = 0; r < RPW; ++r) {
             if (p.hub_row[slot0 + r] < 0) continue;
-            float *dst = p.partial + ((int64_t)range * kHubSlots + slot0 + r) * p.ldp + blockIdx.y * TW + dl;
+            float *dst = p.partial + ((int64_t)range * p.slot_cap + slot0 + r) * p.ldp + blockIdx.y * TW + dl;
 #pragma unroll
             for (int k = 0; k < VEC; ++k)
                 if (blockIdx.y * TW + dl + k < p.D) dst[k] = acc[r * TW + dl + k];
@@ -327,11 +346,11 @@ __global__ void __launch_bounds__(256) spmm_hub_reduce_kernel(const HubArgs p, T
     const int s0 = p.row_slot_first[q], n = (p.row_slot_first[q + 1] - s0) * kHubRanges;
     const int chain = threadIdx.x >> 5, l = threadIdx.x & 31;
     for (int d0 = 0; d0 < p.D; d0 += kHubTile) {
-        const int d = d0 + l * 4;  // ldp is a multiple of kHubTile: the float4 at d lies inside the padded partial row
+        const int d = d0 + l * 4;  // ldp is a multiple of kHubTile (128 or 256): the float4 at d lies inside the padded partial row
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         auto at = [&](int j) {
             const int slot = p.row_slots[s0 + j / kHubRanges], x = j % kHubRanges;
-            return *reinterpret_cast<const float4 *>(p.partial + ((int64_t)x * kHubSlots + slot) * p.ldp + d);
+            return *reinterpret_cast<const float4 *>(p.partial + ((int64_t)x * p.slot_cap + slot) * p.ldp + d);
         };
         auto add = [&](const float4 &t) {
             acc.x += t.x;
@@ -381,9 +400,10 @@ __global__ void __launch_bounds__(256) spmm_hub_reduce_kernel(const HubArgs p, T
 struct BuildArgs {
     const int32_t *rowptr;
     const int32_t *col;
-    const int32_t *hub_row;   // [kHubSlots]
-    const int32_t *hub_part;  // [kHubSlots] part | parts << 16
+    const int32_t *hub_row;   // [slot cap]
+    const int32_t *hub_part;  // [slot cap] part | parts << 16
     int32_t window, windows_per_range, n_windows;
+    int32_t rows_per_wave;    // slots of a wavefront (at most 64: one lane follows one slot)
     const int64_t *stream_first;  // fill
     int32_t *stream_total;        // count
     int32_t *stream_pos;          // fill
@@ -403,8 +423,8 @@ __global__ void __launch_bounds__(64) hub_streams_kernel(const BuildArgs b)
     const int lane = threadIdx.x;
     const int stream = blockIdx.x;
     const int wave = stream % kWaves, group = (stream / kWaves) % kHubGroups, range = stream / (kWaves * kHubGroups);
-    const int slot = (group * kWaves + wave) * kHubRowsPerWave + min(lane, kHubRowsPerWave - 1);
-    const int row = lane < kHubRowsPerWave ? b.hub_row[slot] : -1;
+    const int slot = (group * kWaves + wave) * b.rows_per_wave + min(lane, b.rows_per_wave - 1);
+    const int row = lane < b.rows_per_wave ? b.hub_row[slot] : -1;
     int lo_pos = 0, end_pos = 0, part = 0, parts = 1;
     if (row >= 0) {
         lo_pos = b.rowptr[row];
@@ -447,7 +467,7 @@ __global__ void __launch_bounds__(64) hub_streams_kernel(const BuildArgs b)
             delta[lane] = begin - (incl - n);
             __syncthreads();
             for (int f = lane; f < total; f += kWave) {
-                int lo = 0, hi = kHubRowsPerWave;  // prefix[lo] <= f < prefix[hi] (prefix[kHubRowsPerWave ..] = total)
+                int lo = 0, hi = b.rows_per_wave;  // prefix[lo] <= f < prefix[hi] (prefix[rows_per_wave ..] = total)
                 while (hi - lo > 1) {
                     const int mid = (lo + hi) >> 1;
                     if (prefix[mid] <= f) lo = mid; else hi = mid;
@@ -521,17 +541,19 @@ struct DeviceBlock {  // freed on every way out
     }
 };
 
-template <typename T, int VEC, int LPR>
+template <typename T, int VEC, int LPR, int RPW = kHubRowsPerWave>
 int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st, bool run_pass, bool run_reduce)
 {
     constexpr int TW = LPR * VEC;
-    const size_t shm = ((size_t)kWaves * kHubRowsPerWave * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2) + kWaves * sizeof(int);
+    const size_t shm = ((size_t)kWaves * RPW * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2) + kWaves * sizeof(int);
+    static_assert(((size_t)kWaves * RPW * TW) * sizeof(float) + (size_t)kWaves * 3 * kWave * sizeof(uint2) + kWaves * sizeof(int) <= 160 * 1024,
+                  "the sums of a workgroup, its rings and its progress words fit the LDS of a compute unit");
     static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR>), shm, allowed);
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&spmm_hub_kernel<T, VEC, LPR, RPW>), shm, allowed);
     if (rc != PLX_OK) return rc;
     dim3 grid(kHubRanges * kHubGroups, (unsigned)plx::ceil_div(a.D, TW), 1);
     if (run_pass) {
-        spmm_hub_kernel<T, VEC, LPR><<<grid, kThreads, shm, st>>>(a);
+        spmm_hub_kernel<T, VEC, LPR, RPW><<<grid, kThreads, shm, st>>>(a);
         PLX_LAUNCH_CHECK("spmm_hub_kernel");
     }
     if (run_reduce) {
@@ -546,7 +568,11 @@ int launch_t(const HubArgs &a, void *Y, int64_t ldy, hipStream_t st, bool run_pa
 namespace plx {
 namespace hub {
 
-size_t partial_bytes(int64_t D) { return (size_t)kHubRanges * kHubSlots * (size_t)(ceil_div(D, kHubTile) * kHubTile) * sizeof(float); }
+size_t partial_bytes(int64_t D, bool wide)
+{
+    const int64_t tile = wide ? kHubTileWide : kHubTile, slots = (int64_t)kHubGroups * kWaves * (wide ? kHubRowsPerWaveWide : kHubRowsPerWave);
+    return (size_t)kHubRanges * (size_t)slots * (size_t)(ceil_div(D, tile) * tile) * sizeof(float);
+}
 
 void free_hub_plan(HubPlan &hp)
 {
@@ -556,10 +582,12 @@ void free_hub_plan(HubPlan &hp)
 
 int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, const int32_t *col, int32_t seg_len, int64_t n_long,
                    int64_t n_seg, const int32_t *long_rows, const int32_t *seg_first, const std::vector<int32_t> &h_long_rows,
-                   int64_t min_entries, hipStream_t st, HubPlan &out)
+                   int64_t min_entries, bool wide, hipStream_t st, HubPlan &out)
 {
     (void)M;
     out = HubPlan();
+    const int rows_per_wave = wide ? kHubRowsPerWaveWide : kHubRowsPerWave;
+    const int slot_cap = kHubGroups * kWaves * rows_per_wave;
     if (n_long <= 0 || K <= 0 || nnz <= 0) return PLX_OK;
 
     // lengths of the split rows, and whether their columns ascend, to the host
@@ -583,10 +611,10 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     // longest first (ties: lower row first); a row takes ceil(len / part_len) slots, rows are taken while slots last
     std::vector<int32_t> order((size_t)n_long);
     std::iota(order.begin(), order.end(), 0);
-    const size_t keep = std::min<size_t>((size_t)n_long, (size_t)kHubSlots);
+    const size_t keep = std::min<size_t>((size_t)n_long, (size_t)slot_cap);
     auto longer = [&](int32_t x, int32_t y) { return len[(size_t)x] != len[(size_t)y] ? len[(size_t)x] > len[(size_t)y] : x < y; };
     std::partial_sort(order.begin(), order.begin() + (ptrdiff_t)keep, order.end(), longer);
-    const int64_t part_len = (int64_t)seg_len * kHubPartFactor;
+    const int64_t part_len = (int64_t)seg_len * (wide ? kHubPartFactorWide : kHubPartFactor);
     struct Slot { int32_t row, part, parts, q; int64_t size; };
     std::vector<Slot> slots;
     std::vector<int32_t> rows, row_slot_first{0};
@@ -595,7 +623,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
         const int32_t q = order[i];
         const int64_t l = len[(size_t)q];
         const int64_t parts = ceil_div(l, part_len);
-        if ((int64_t)slots.size() + parts > kHubSlots) continue;  // a shorter row may still fit
+        if ((int64_t)slots.size() + parts > slot_cap) continue;  // a shorter row may still fit
         for (int64_t s = 0; s < parts; ++s) slots.push_back(Slot{h_long_rows[(size_t)q], (int32_t)s, (int32_t)parts, (int32_t)rows.size(), l / parts});
         rows.push_back(h_long_rows[(size_t)q]);
         row_slot_first.push_back((int32_t)slots.size());
@@ -608,7 +636,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     std::vector<int32_t> by_size(slots.size());
     std::iota(by_size.begin(), by_size.end(), 0);
     std::stable_sort(by_size.begin(), by_size.end(), [&](int32_t x, int32_t y) { return slots[(size_t)x].size > slots[(size_t)y].size; });
-    std::vector<int32_t> hub_row((size_t)kHubSlots, -1), hub_part((size_t)kHubSlots, 1 << 16), row_slots(slots.size());
+    std::vector<int32_t> hub_row((size_t)slot_cap, -1), hub_part((size_t)slot_cap, 1 << 16), row_slots(slots.size());
     {
         constexpr int kBins = kHubGroups * kWaves;
         using Bin = std::pair<int64_t, int32_t>;  // (entries, wavefront): the least loaded first, ties by number
@@ -621,12 +649,12 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
             Bin bin = bins.top();
             bins.pop();
             const int32_t b = bin.second, group = b % kHubGroups, wave = b / kHubGroups;
-            const int32_t id = (group * kWaves + wave) * kHubRowsPerWave + held[(size_t)b];
+            const int32_t id = (group * kWaves + wave) * rows_per_wave + held[(size_t)b];
             hub_row[(size_t)id] = sl.row;
             hub_part[(size_t)id] = sl.part | (sl.parts << 16);
             row_slots[(size_t)row_slot_first[(size_t)sl.q] + (size_t)sl.part] = id;
             bin.first += sl.size;
-            if (++held[(size_t)b] < kHubRowsPerWave) bins.push(bin);
+            if (++held[(size_t)b] < rows_per_wave) bins.push(bin);
         }
     }
 
@@ -638,7 +666,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     // the small tables and the stream lengths
     const size_t n_rows = rows.size(), n_slots = slots.size();
     auto up16 = [](size_t x) { return (x + 15) / 16 * 16; };
-    const size_t o_hub_row = 0, o_hub_part = o_hub_row + up16(sizeof(int32_t) * kHubSlots), o_rows = o_hub_part + up16(sizeof(int32_t) * kHubSlots),
+    const size_t o_hub_row = 0, o_hub_part = o_hub_row + up16(sizeof(int32_t) * slot_cap), o_rows = o_hub_part + up16(sizeof(int32_t) * slot_cap),
                  o_rsf = o_rows + up16(sizeof(int32_t) * n_rows), o_rs = o_rsf + up16(sizeof(int32_t) * (n_rows + 1)),
                  o_first = o_rs + up16(sizeof(int32_t) * n_slots), o_total = o_first + up16(sizeof(int64_t) * kHubStreams),
                  o_mark = o_total + up16(sizeof(int32_t) * kHubStreams), o_lflag = o_mark + up16(sizeof(int32_t) * (size_t)kHubStreams * (size_t)wpr),
@@ -647,8 +675,8 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     DeviceBlock small;
     PLX_HIP_CHECK(hipMalloc(&small.p, small_bytes));
     char *sb = static_cast<char *>(small.p);
-    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_row, hub_row.data(), sizeof(int32_t) * kHubSlots, hipMemcpyHostToDevice, st));
-    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_part, hub_part.data(), sizeof(int32_t) * kHubSlots, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_row, hub_row.data(), sizeof(int32_t) * slot_cap, hipMemcpyHostToDevice, st));
+    PLX_HIP_CHECK(hipMemcpyAsync(sb + o_hub_part, hub_part.data(), sizeof(int32_t) * slot_cap, hipMemcpyHostToDevice, st));
     BuildArgs b{};
     b.rowptr = rowptr;
     b.col = col;
@@ -657,6 +685,7 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     b.window = window;
     b.windows_per_range = wpr;
     b.n_windows = n_windows;
+    b.rows_per_wave = rows_per_wave;
     b.stream_total = reinterpret_cast<int32_t *>(sb + o_total);
     hub_streams_kernel<false><<<kHubStreams, 64, 0, st>>>(b);
     PLX_LAUNCH_CHECK("hub_streams_kernel (count)");
@@ -707,6 +736,8 @@ int build_hub_plan(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, con
     out.window = window;
     out.n_windows = n_windows;
     out.windows_per_range = wpr;
+    out.rows_per_wave = rows_per_wave;
+    out.slot_cap = slot_cap;
     out.block = block.p;
     block.p = nullptr;
     out.hub_row = reinterpret_cast<const int32_t *>(bb + o_hub_row);
@@ -752,6 +783,14 @@ int launch(const HubPlan &hp, const int32_t *col, const float *val, const void *
     a.row_begin = (int32_t)row_begin;
     a.row_end = (int32_t)row_end;
     a.partial = partial;
+    a.slot_cap = hp.slot_cap;
+    if (hp.rows_per_wave == kHubRowsPerWaveWide) {
+        // bf16 rows of 512 bytes and more: half a wavefront reads 256 columns, 16 bytes per lane, in one tile (in 128-column
+        // tiles every stream, column index and value is read once per tile and a load carries 8 bytes per lane)
+        PLX_REQUIRE(bf16 && d_read % 8 == 0, "hub pass: the wide layout takes bf16 rows in multiples of 8 columns");
+        a.ldp = ceil_div(D, kHubTileWide) * kHubTileWide;
+        return launch_t<uint16_t, 8, 32, kHubRowsPerWaveWide>(a, Y, ldy, st, run_pass, run_reduce);
+    }
     a.ldp = ceil_div(D, kHubTile) * kHubTile;  // every kernel's tile divides kHubTile
     // fp32 rows of at most 256 bytes are read by a quarter of a wavefront, four entries per load instruction
     // (bf16 rows read 16 bytes per lane by a quarter of a wavefront were measured too: no faster than 8 bytes by a half)

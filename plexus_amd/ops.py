@@ -148,6 +148,18 @@ class CsrMatrix:
         check(_lib.load().plx_spmm_plan_build_hub(self._plan, _stream()), "plx_spmm_plan_build_hub")
         self._ws = None
 
+    def build_hub_wide(self) -> None:
+        """Builds the hub tables in the layout for bf16 rows of 512 bytes and more (256 columns per tile, half as many
+        sums per wavefront).  The front end does this by itself before the first such product of a matrix that has the
+        regular tables."""
+        check(_lib.load().plx_spmm_plan_build_hub_wide(self._plan, _stream()), "plx_spmm_plan_build_hub_wide")
+        self._wide_tried = True
+        self._ws = None
+
+    @property
+    def n_hub_rows_wide(self) -> int:
+        return int(_lib.load().plx_spmm_plan_info(self._plan, 9))
+
     def set_hub(self, mode: int) -> None:
         """0 = products use the hub pass where the tables exist and the operands allow it (the default), -1 = never.
         With and without the pass a product agrees to fp32 rounding, not bit for bit."""
@@ -156,6 +168,9 @@ class CsrMatrix:
 
     def _workspace(self, d: int, dtype=torch.float32):
         lib = _lib.load()
+        # plan preparation, once per matrix: a bf16 product of 256 columns or more takes the hub pass in its wide layout
+        if dtype == torch.bfloat16 and d >= 256 and not getattr(self, "_wide_tried", False) and self.n_hub_rows > 0:
+            self.build_hub_wide()
         query = lib.plx_spmm_workspace_bytes_bf16 if dtype == torch.bfloat16 else lib.plx_spmm_workspace_bytes
         need = int(query(self._plan, d))
         if need == 0:

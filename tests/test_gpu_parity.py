@@ -1306,6 +1306,130 @@ def test_spmm_workspace_covers_the_hub_pass_of_either_storage_type():
     assert rel_err(yf.cpu(), oracle_spmm64(g, h32)) <= FP32_TOL
 
 
+def test_spmm_hub_pass_in_the_wide_layout_for_bf16_rows_of_512_bytes():
+    """bf16 products of 256 columns and more take the hub pass in its wide layout (256-column tiles, 18 sums per
+    wavefront, 16-byte loads) once the plan has those tables; widths and operands that do not allow 16-byte loads keep
+    the regular layout.  Both against the fp64 oracle, the wide one also bit-stable on repeat and in row ranges."""
+    say("spmm hub pass, wide layout (bf16, D >= 256)")
+    g, a = _hub_matrix(seed=36)
+    regular_only = to_dev(g, seg_len=16)
+    regular_only.build_hub()
+    regular_only._wide_tried = True  # keeps the front end from building the wide tables for this one
+    n = 3000
+    for d in (256, 264, 512, 1000):
+        h = torch.randn(n, d, generator=torch.Generator().manual_seed(d)).to(torch.bfloat16).to(DEV)
+        ref = oracle_spmm64(g, h.float().cpu())
+        y = ops.spmm(a, h)
+        assert a.n_hub_rows_wide > 0 and regular_only.n_hub_rows_wide == 0
+        assert rel_err(y.float().cpu(), ref) <= BF16_TOL, d
+        assert torch.equal(ops.spmm(a, h), y)
+        assert torch.equal(ops.chunked_spmm(a, h, max_rows_per_chunk=700), y)
+        y_reg = ops.spmm(regular_only, h)
+        assert rel_err(y_reg.float().cpu(), ref) <= BF16_TOL
+        # fp32 sums in another order, rounded to bf16 at the end: equal but for an element in a few thousand
+        assert (y != y_reg).float().mean().item() < 0.02 and rel_err(y.float(), y_reg.float()) <= 2.0 ** -7
+        # rows outside the pass are summed by the row kernel either way
+        rows = torch.ones(n, dtype=torch.bool)
+        rows[torch.nonzero((g.rowptr[1:] - g.rowptr[:-1]) > 16).reshape(-1)] = False
+        assert torch.equal(y.cpu()[rows], y_reg.cpu()[rows])
+    # a width that is no multiple of 8, and a view 8 bytes into a wider matrix: the regular tables, bit for bit
+    h = torch.randn(n, 260, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(DEV)
+    assert torch.equal(ops.spmm(a, h), ops.spmm(regular_only, h))
+    wide = torch.randn(n, 272, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(DEV)
+    view = wide[:, 4:260]
+    assert view.data_ptr() % 16 == 8
+    assert torch.equal(ops.spmm(a, view), ops.spmm(regular_only, view))
+    assert rel_err(ops.spmm(a, view).float().cpu(), oracle_spmm64(g, view.float().cpu().contiguous())) <= BF16_TOL
+    # fp32 products never take the wide tables
+    hf = torch.randn(n, 256, generator=torch.Generator().manual_seed(3)).to(DEV)
+    assert torch.equal(ops.spmm(a, hf), ops.spmm(regular_only, hf))
+    # switched off, the product is the row kernel's
+    a.set_hub(-1)
+    regular_only.set_hub(-1)
+    h = torch.randn(n, 256, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(DEV)
+    assert torch.equal(ops.spmm(a, h), ops.spmm(regular_only, h))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chunked_product_runs_the_hub_pass_once_and_keeps_every_bit(dtype):
+    """The two ways of computing a product range by range: plx_spmm_csr_rows_* (every range that holds a hub row runs the
+    whole pass) and plx_spmm_csr_chunk_* (the first chunk runs it for all, later chunks add up their own hub rows from
+    the partial sums it left).  Both must give the whole product's bits, also when the first chunk holds no hub row."""
+    say("chunk entry points with a hub pass, %s" % dtype)
+    from plexus_amd import _lib
+
+    lib = _lib.load()
+    g, a = _hub_matrix(seed=35)
+    n, d = 3000, 128 if dtype == torch.float32 else 256
+    h = torch.randn(n, d, generator=torch.Generator().manual_seed(3)).to(dtype).to(DEV)
+    whole = ops.spmm(a, h)
+    a.set_hub(-1)
+    assert not torch.equal(ops.spmm(a, h), whole) or dtype == torch.bfloat16  # the pass is taken at this width
+    a.set_hub(0)
+    rows_fn, chunk_fn = ((lib.plx_spmm_csr_rows_f32, lib.plx_spmm_csr_chunk_f32) if dtype == torch.float32 else
+                         (lib.plx_spmm_csr_rows_bf16, lib.plx_spmm_csr_chunk_bf16))
+    ws, ws_bytes = a._workspace(d, dtype)
+    st = torch.cuda.current_stream().cuda_stream
+    hub_rows = torch.nonzero((g.rowptr[1:] - g.rowptr[:-1]) > 16).reshape(-1)
+    gaps = hub_rows[1:] - hub_rows[:-1]
+    i = int(torch.argmax(gaps))
+    lo_free, hi_free = int(hub_rows[i]) + 1, int(hub_rows[i + 1])  # the longest run of rows without a hub row
+    assert hi_free - lo_free >= 2
+    # chunks in the order they are issued: the first one holds no hub row (it still runs the pass for the others); then
+    # the rows before it; an empty chunk; the rows after it
+    bounds = [(lo_free, hi_free), (0, lo_free), (lo_free, lo_free), (hi_free, n)]
+    y_rows = torch.zeros(n, d, dtype=dtype, device=DEV)
+    for lo, hi in bounds:
+        _lib.check(rows_fn(a._plan, lo, hi, a.val.data_ptr(), h.data_ptr(), d, d, y_rows.data_ptr(), d, ws.data_ptr(), ws_bytes, st), "rows")
+    assert torch.equal(y_rows, whole)
+    y_chunk = torch.zeros(n, d, dtype=dtype, device=DEV)
+    for i, (lo, hi) in enumerate(bounds):
+        ws[:64] = 0  # nothing in the front of the workspace (partial rows of split rows) is carried between chunks
+        _lib.check(chunk_fn(a._plan, lo, hi, int(i == 0), a.val.data_ptr(), h.data_ptr(), d, d, y_chunk.data_ptr(), d, ws.data_ptr(),
+                            ws_bytes, st), "chunk")
+    assert torch.equal(y_chunk, whole)
+    assert rel_err(whole.float().cpu(), oracle_spmm64(g, h.float().cpu())) <= (FP32_TOL if dtype == torch.float32 else BF16_TOL)
+    # a plan without hub tables: the chunk entry points are the row-range ones
+    plain = to_dev(g, seg_len=16)
+    y2 = torch.zeros(n, d, dtype=dtype, device=DEV)
+    ws2, ws2_bytes = plain._workspace(d, dtype)
+    for i, (lo, hi) in enumerate(bounds):
+        _lib.check(chunk_fn(plain._plan, lo, hi, int(i == 0), plain.val.data_ptr(), h.data_ptr(), d, d, y2.data_ptr(), d,
+                            ws2.data_ptr() if ws2 is not None else None, ws2_bytes, st), "chunk")
+    assert torch.equal(y2, ops.spmm(plain, h))
+
+
+def test_hub_tables_are_refused_for_rows_whose_columns_do_not_ascend():
+    say("hub tables on a matrix with unsorted columns in a long row")
+    from plexus_amd._lib import PlexusHipError
+
+    gen = torch.Generator().manual_seed(12)
+    m, k, seg_len = 50, 4000, 8
+    lens = torch.full((m,), 3, dtype=torch.int64)
+    lens[7] = 900
+    lens[20] = 1200
+    cols = [torch.randperm(k, generator=gen)[: int(n)].sort().values for n in lens]
+    cols[20] = cols[20][torch.randperm(1200, generator=gen)]  # one long row in arbitrary order
+    rowptr = torch.zeros(m + 1, dtype=torch.int64)
+    rowptr[1:] = torch.cumsum(lens, 0)
+    col = torch.cat(cols).to(torch.int32)
+    val = torch.randn(col.numel(), generator=gen)
+    a = ops.CsrMatrix(rowptr.to(torch.int32).to(DEV), col.to(DEV), val.to(DEV), (m, k), seg_len)
+    with pytest.raises(PlexusHipError, match="do not ascend"):
+        a.build_hub()
+    assert a.n_hub_rows == 0
+    # the product without the pass takes the columns of a row in any order
+    h = torch.randn(k, 128, generator=gen)
+    ref = oracle_c.csr_spmm(rowptr.to(torch.int32).numpy(), col.numpy(), val.numpy(), h.numpy())
+    assert rel_err(ops.spmm(a, h.to(DEV)).cpu(), ref) <= FP32_TOL
+    # sorted, the same matrix gets its tables and the same product
+    order = torch.cat([rowptr[r] + torch.argsort(col[rowptr[r]:rowptr[r + 1]].to(torch.int64)) for r in range(m)])
+    b = ops.CsrMatrix(rowptr.to(torch.int32).to(DEV), col[order].to(DEV), val[order].to(DEV), (m, k), seg_len)
+    b.build_hub()
+    assert b.n_hub_rows == 2
+    assert rel_err(ops.spmm(b, h.to(DEV)).cpu(), ref) <= FP32_TOL
+
+
 def test_spmm_hub_pass_is_left_out_where_the_operand_does_not_suit_it():
     say("spmm hub pass: widths and layouts it does not take")
     g, a = _hub_matrix(seed=32)
