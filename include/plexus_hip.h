@@ -160,6 +160,22 @@ int plx_spmm_plan_set_hub(plx_spmm_plan *plan, int mode);
  * multiple of 8 and H is 16-byte aligned with a pitch that is a multiple of 8 (other operands take the regular tables
  * by the rule above). */
 int plx_spmm_plan_build_hub_wide(plx_spmm_plan *plan, void *stream);
+/* The tables of the hub pass (wide == 0: the regular layout, else the wide one), for inspection and tests; synchronous.
+ * plx_spmm_plan_hub_info, what == 0: hub rows, 1: slots in use, 2: entries in hub rows, 3: stored stream entries (every
+ * stream padded to a multiple of 64), 4: columns per window, 5: windows, 6: windows per column range (8 ranges), 7: sums
+ * per wavefront, 8: slots of the layout (256 wavefronts x sums per wavefront), 9: streams (2,048: one per wavefront and
+ * range; 0 without tables).  plx_spmm_plan_hub_tables_host copies to host arrays (any of them may be NULL):
+ *   hub_row [slots of the layout]: row of a slot, -1 for an unused slot; wavefront w of a range owns slots
+ *     w * sums_per_wavefront ...;  rows [hub rows]; row_slot_first [hub rows + 1] and row_slots [slots in use]: the slots
+ *     of a hub row, one per part, in part order;
+ *   stream s = range * 256 + wavefront: stream_first [streams] its first stored entry, stream_total [streams] its
+ *     entries; stream_pos / stream_run [stored]: position of an entry in the CSR arrays and its slot among the
+ *     wavefront's own (padding: position 0, slot 255); stream_mark [streams x windows per range]: number of the 64-entry
+ *     batch in which a window of the range begins. */
+int64_t plx_spmm_plan_hub_info(const plx_spmm_plan *plan, int wide, int what);
+int plx_spmm_plan_hub_tables_host(const plx_spmm_plan *plan, int wide, int32_t *hub_row_host, int32_t *rows_host, int32_t *row_slot_first_host,
+                                  int32_t *row_slots_host, int64_t *stream_first_host, int32_t *stream_total_host, int32_t *stream_pos_host,
+                                  uint8_t *stream_run_host, int32_t *stream_mark_host);
 /* bytes of scratch an fp32 SpMM of width D needs (plx_spmm_workspace_bytes_bf16: a bf16 one -- the hub pass, the column
  * slices and the copy below go by the bytes of a row, so the two types differ, and a product given less than its own
  * query asks for returns PLX_ERR_WORKSPACE): fp32 partial sums of the split rows, the partial sums

@@ -40,6 +40,8 @@ SIGNATURES = {
     "plx_spmm_plan_set_slicing": (C.c_int, [_vp, C.c_int]),
     "plx_spmm_plan_build_hub": (C.c_int, [_vp, _vp]),
     "plx_spmm_plan_build_hub_wide": (C.c_int, [_vp, _vp]),
+    "plx_spmm_plan_hub_info": (_i64, [_vp, C.c_int, C.c_int]),
+    "plx_spmm_plan_hub_tables_host": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "plx_spmm_plan_set_hub": (C.c_int, [_vp, C.c_int]),
     "plx_spmm_workspace_bytes": (_sz, [_vp, _i64]),
     "plx_spmm_workspace_bytes_bf16": (_sz, [_vp, _i64]),

@@ -1098,6 +1098,46 @@ int plx_spmm_plan_tables_host(const plx_spmm_plan *plan, int32_t *long_rows_host
     return PLX_OK;
 }
 
+int64_t plx_spmm_plan_hub_info(const plx_spmm_plan *plan, int wide, int what)
+{
+    if (!plan) return -1;
+    const plx::hub::HubPlan &hp = wide ? plan->hub_wide : plan->hub;
+    switch (what) {
+        case 0: return hp.n_rows;
+        case 1: return hp.n_slots;
+        case 2: return hp.entries;
+        case 3: return hp.stored;
+        case 4: return hp.window;
+        case 5: return hp.n_windows;
+        case 6: return hp.windows_per_range;
+        case 7: return hp.rows_per_wave;
+        case 8: return hp.slot_cap;
+        case 9: return hp.block != nullptr ? plx::hub::kHubStreams : 0;
+        default: return -1;
+    }
+}
+
+int plx_spmm_plan_hub_tables_host(const plx_spmm_plan *plan, int wide, int32_t *hub_row_host, int32_t *rows_host, int32_t *row_slot_first_host,
+                                  int32_t *row_slots_host, int64_t *stream_first_host, int32_t *stream_total_host, int32_t *stream_pos_host,
+                                  uint8_t *stream_run_host, int32_t *stream_mark_host)
+{
+    PLX_REQUIRE(plan != nullptr, "plan_hub_tables_host: plan is NULL");
+    const plx::hub::HubPlan &hp = wide ? plan->hub_wide : plan->hub;
+    PLX_REQUIRE(hp.block != nullptr, "plan_hub_tables_host: the plan has no hub tables in that layout");
+    const size_t streams = (size_t)plx::hub::kHubStreams;
+    auto get = [](void *dst, const void *src, size_t bytes) { return (dst == nullptr || bytes == 0) ? hipSuccess : hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost); };
+    PLX_HIP_CHECK(get(hub_row_host, hp.hub_row, sizeof(int32_t) * (size_t)hp.slot_cap));
+    PLX_HIP_CHECK(get(rows_host, hp.rows, sizeof(int32_t) * (size_t)hp.n_rows));
+    PLX_HIP_CHECK(get(row_slot_first_host, hp.row_slot_first, sizeof(int32_t) * ((size_t)hp.n_rows + 1)));
+    PLX_HIP_CHECK(get(row_slots_host, hp.row_slots, sizeof(int32_t) * (size_t)hp.n_slots));
+    PLX_HIP_CHECK(get(stream_first_host, hp.stream_first, sizeof(int64_t) * streams));
+    PLX_HIP_CHECK(get(stream_total_host, hp.stream_total, sizeof(int32_t) * streams));
+    PLX_HIP_CHECK(get(stream_pos_host, hp.stream_pos, sizeof(int32_t) * (size_t)hp.stored));
+    PLX_HIP_CHECK(get(stream_run_host, hp.stream_run, (size_t)hp.stored));
+    PLX_HIP_CHECK(get(stream_mark_host, hp.stream_mark, sizeof(int32_t) * streams * (size_t)hp.windows_per_range));
+    return PLX_OK;
+}
+
 // The room for the line-aligned copy of H is decided for contiguous rows of the element type (an operand laid out
 // otherwise is staged only if it fits what the caller brought).
 size_t plx_spmm_workspace_bytes(const plx_spmm_plan *plan, int64_t D) { return workspace_need(plan, D, 4); }

@@ -195,36 +195,56 @@ __global__ void __launch_bounds__(256) softmax_xent_tiled_kernel(const XentArgs 
 // consecutive elements, copied in and out with 128-bit accesses into an unpadded LDS tile (CP == C) whose
 // per-row pass is free of bank conflicts because the row stride is odd.  (Rotating the visit order by the
 // lane index makes even C conflict-free too, but the run-time LDS addresses cost more than the copy saves.)
-template <typename T, int CMAX>
-__global__ void __launch_bounds__(256) softmax_xent_tiled_reg_kernel(const XentArgs p, int R)
+template <typename T, int CMAX, int R>
+__global__ void __launch_bounds__(256) softmax_xent_tiled_reg_kernel(const XentArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float tile[];
     __shared__ float wsum[4];
     constexpr int EPV = 16 / (int)sizeof(T);  // elements per 128-bit access
+    constexpr int kVecs = (R * CMAX + EPV * 256 - 1) / (EPV * 256);  // 128-bit vectors of a tile per thread, at most
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     const int C = (int)p.C;
     const int cv = (int)min(p.C, p.num_classes);
     const int64_t n_tiles = (p.M + R - 1) / R;
     float loss_acc = 0.f;
+    // The tile after the one being worked on is already on its way from memory: its vectors are requested into
+    // registers before the row phase of the current tile and written to LDS when that tile has been stored, so the
+    // loads of a workgroup overlap its own exponentials and stores, not only those of its neighbours on the compute unit.
+    u32x4 pre[kVecs];
+    auto request = [&](int64_t t) {
+        const int64_t row0 = t * R;
+        const int vecs = (int)min((int64_t)R, p.M - row0) * C / EPV;
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const T *>(p.logits) + row0 * C);
+#pragma unroll
+        for (int j = 0; j < kVecs; ++j) {
+            const int i = j * 256 + (int)threadIdx.x;
+            if (i < vecs) pre[j] = __builtin_nontemporal_load(src + i);
+        }
+    };
+    if ((int64_t)blockIdx.x < n_tiles) request(blockIdx.x);
     for (int64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
         const int64_t row0 = t * R;
         const int rows = (int)min((int64_t)R, p.M - row0);
         const int count = rows * C;
-        const T *src = static_cast<const T *>(p.logits) + row0 * C;
-        for (int i = threadIdx.x; i < count / EPV; i += 256) {
-            if constexpr (sizeof(T) == 4) {
-                reinterpret_cast<float4 *>(tile)[i] = reinterpret_cast<const float4 *>(src)[i];
-            } else {
-                const uint4 raw = reinterpret_cast<const uint4 *>(src)[i];
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        const int vecs = count / EPV;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    tile[i * 8 + 2 * j] = __uint_as_float(w[j] << 16);
-                    tile[i * 8 + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        for (int j = 0; j < kVecs; ++j) {
+            const int i = j * 256 + (int)threadIdx.x;
+            if (i < vecs) {
+                if constexpr (sizeof(T) == 4) {
+                    reinterpret_cast<u32x4 *>(tile)[i] = pre[j];
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        tile[i * 8 + 2 * q] = __uint_as_float(pre[j][q] << 16);
+                        tile[i * 8 + 2 * q + 1] = __uint_as_float(pre[j][q] & 0xffff0000u);
+                    }
                 }
             }
         }
-        for (int i = count / EPV * EPV + threadIdx.x; i < count; i += 256) tile[i] = ld_elem<T>(p.logits, row0 * C + i);
+        for (int i = vecs * EPV + threadIdx.x; i < count; i += 256) tile[i] = ld_elem<T>(p.logits, row0 * C + i);
         __syncthreads();
+        if (t + gridDim.x < n_tiles) request(t + gridDim.x);
         if ((int)threadIdx.x < rows) {
             float *x = tile + threadIdx.x * C;
             const int64_t row = row0 + threadIdx.x;
@@ -257,22 +277,27 @@ __global__ void __launch_bounds__(256) softmax_xent_tiled_reg_kernel(const XentA
         }
         __syncthreads();
         if (p.dlogits != nullptr) {
-            T *dst = static_cast<T *>(p.dlogits) + row0 * C;
-            for (int i = threadIdx.x; i < count / EPV; i += 256) {
-                if constexpr (sizeof(T) == 4) {
-                    reinterpret_cast<float4 *>(dst)[i] = reinterpret_cast<const float4 *>(tile)[i];
-                } else {
-                    const float4 lo = reinterpret_cast<const float4 *>(tile)[2 * i];
-                    const float4 hi = reinterpret_cast<const float4 *>(tile)[2 * i + 1];
-                    uint4 o;
-                    o.x = plx::pack_bf16x2(lo.x, lo.y);
-                    o.y = plx::pack_bf16x2(lo.z, lo.w);
-                    o.z = plx::pack_bf16x2(hi.x, hi.y);
-                    o.w = plx::pack_bf16x2(hi.z, hi.w);
-                    reinterpret_cast<uint4 *>(dst)[i] = o;
+            // the gradient is read next by another kernel, long after this one: stores that do not linger in the caches
+            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<T *>(p.dlogits) + row0 * C);
+#pragma unroll
+            for (int j = 0; j < kVecs; ++j) {
+                const int i = j * 256 + (int)threadIdx.x;
+                if (i < vecs) {
+                    if constexpr (sizeof(T) == 4) {
+                        __builtin_nontemporal_store(reinterpret_cast<const u32x4 *>(tile)[i], dst + i);
+                    } else {
+                        const float4 lo = reinterpret_cast<const float4 *>(tile)[2 * i];
+                        const float4 hi = reinterpret_cast<const float4 *>(tile)[2 * i + 1];
+                        u32x4 o;
+                        o[0] = plx::pack_bf16x2(lo.x, lo.y);
+                        o[1] = plx::pack_bf16x2(lo.z, lo.w);
+                        o[2] = plx::pack_bf16x2(hi.x, hi.y);
+                        o[3] = plx::pack_bf16x2(hi.z, hi.w);
+                        __builtin_nontemporal_store(o, dst + i);
+                    }
                 }
             }
-            for (int i = count / EPV * EPV + threadIdx.x; i < count; i += 256) st_elem<T>(p.dlogits, row0 * C + i, tile[i]);
+            for (int i = vecs * EPV + threadIdx.x; i < count; i += 256) st_elem<T>(p.dlogits, row0 * C + i, tile[i]);
         }
         __syncthreads();
     }
@@ -287,10 +312,13 @@ __global__ void __launch_bounds__(256) softmax_xent_tiled_reg_kernel(const XentA
 template <typename T>
 static void launch_tiled_reg(const XentArgs &a, int64_t C, int R, unsigned blocks, size_t shm, hipStream_t st)
 {
-    if (C <= 16) softmax_xent_tiled_reg_kernel<T, 16><<<blocks, 256, shm, st>>>(a, R);
-    else if (C <= 32) softmax_xent_tiled_reg_kernel<T, 32><<<blocks, 256, shm, st>>>(a, R);
-    else if (C <= 48) softmax_xent_tiled_reg_kernel<T, 48><<<blocks, 256, shm, st>>>(a, R);
-    else softmax_xent_tiled_reg_kernel<T, 64><<<blocks, 256, shm, st>>>(a, R);
+    if (R == 256) {  // C <= 47
+        if (C <= 16) softmax_xent_tiled_reg_kernel<T, 16, 256><<<blocks, 256, shm, st>>>(a);
+        else if (C <= 32) softmax_xent_tiled_reg_kernel<T, 32, 256><<<blocks, 256, shm, st>>>(a);
+        else softmax_xent_tiled_reg_kernel<T, 48, 256><<<blocks, 256, shm, st>>>(a);
+    } else {
+        softmax_xent_tiled_reg_kernel<T, 64, 128><<<blocks, 256, shm, st>>>(a);
+    }
 }
 
 __global__ void __launch_bounds__(256) xent_finish_kernel(const float *__restrict__ partials, int n, double inv_nodes,
