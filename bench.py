@@ -413,8 +413,9 @@ def bench_dense_kernels(args, dev):
             rec("GRAD_AGG = (G*mask).W^T %dx%d%s" % (n, k, "" if last else " (bit mask)"),
                 (lambda: ops.gemm_nt(g, w)) if last else (lambda: ops.gemm_nt(g, w, mask=act, mask_bits=bits)),
                 e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
-            rec("GRAD_W = AGG^T.(G*mask) %dx%d" % (k, n), lambda: ops.gemm_tn(a, g, mask=None if last else act),
-                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            rec("GRAD_W = AGG^T.(G*mask) %dx%d%s" % (k, n, "" if last else " (bit mask)"),
+                (lambda: ops.gemm_tn(a, g)) if last else (lambda: ops.gemm_tn(a, g, mask=act, mask_bits=bits)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
         del a, g, act
     logits = S.normal_features(m, dims[-1], dev, seed=3, dtype=torch.bfloat16 if bf16 else torch.float32)
     labels = S.uniform_labels(m, dims[-1], dev, seed=2)

@@ -308,6 +308,20 @@ int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
                     float *C, int64_t ldc, const float *mask, int64_t ldmask, void *workspace,
                     size_t workspace_bytes, void *stream);
 
+/* GRAD_W on the bf16 matrix cores with fp32-level accuracy, as the two split products above: both operands are split
+ * into three exact bf16 pieces on their way into LDS (transposed there, since the contraction runs over their rows), six
+ * piece products per block are accumulated in fp32, the rows are cut into one stretch per compute unit whose partial
+ * tiles are added in a fixed order in fp64, and the result is multiplied by alpha (1 / (1 - p) after a dropout layer).
+ * `mask_bits` (may be NULL; ldw >= ceil(N / 32)) is the mask of B as one bit per element, as plx_gemm_nn_f32_split_bits
+ * writes it; the fp32 `mask`, which must say the same, is read where no bits are given and by the fp32 MFMA launch
+ * that redoes the product when an operand holds Inf, NaN or a value next to FLT_MAX (always enqueued, returns at once
+ * otherwise).  Any alignment (128-bit loads when A, B and mask are 16-byte aligned with leading dimensions, K and N
+ * multiples of 4).  Same reference call site as plx_gemm_tn_f32: plexus/gcn_conv.py:237-239. */
+size_t plx_gemm_tn_f32_split_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int plx_gemm_tn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                          const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, float alpha, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
 /* ---- bf16 storage, fp32 accumulation (raw uint16 bit patterns; the reference has no reduced-precision
  *      path, these follow the same call sites as the fp32 entry points above) ----
  *

@@ -66,6 +66,8 @@ SIGNATURES = {
                                                _vp]),
     "plx_dropout_f32": (C.c_int, [_i64, _i64, _vp, _i64, _f32, C.c_uint64, C.c_uint64, _vp]),
     "plx_gemm_nt_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "plx_gemm_tn_f32_split_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_gemm_tn_f32_split": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz, _vp]),
     "plx_gemm_tn_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_f32": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "plx_copy_rows": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _vp]),

@@ -39,6 +39,16 @@ int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
 int gemm_nt_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                    int64_t ldc, const float *mask, int64_t ldmask, const unsigned *run_if, int n_run_if, void *stream, float alpha = 1.f);
 
+// GRAD_W on the fp32 MFMA (gemm.hip) for the split product of gemm_split_tn.hip: its workspace and split count, the
+// guarded form (runs, and writes C, only if *run_if is non-zero; the result times alpha), and the fixed-order sum of
+// partial tiles that both products end with
+size_t gemm_tn_f32_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int64_t gemm_tn_f32_splits(int64_t M, int64_t N, int64_t K);
+int gemm_tn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                   const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, const unsigned *run_if, float alpha, void *stream);
+int gemm_tn_reduce_tiles(const float *ws, int64_t ws_ld, int64_t ws_slab, int splits, int64_t K, int64_t N, float *C, int64_t ldc, float alpha,
+                         void *stream);
+
 #if defined(__HIPCC__)
 // Orders the LDS accesses of one wavefront for the compiler: lanes that exchange data through a tile private to their
 // wavefront (no workgroup barrier) put this between the stores of one phase and the loads of the next.  The hardware

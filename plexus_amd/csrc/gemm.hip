@@ -322,7 +322,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
             const int64_t r = row0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
             if (r < nrows) {
                 float x = acc[t][v];
-                if constexpr (MODE != kTN) x *= g.alpha;
+                if (MODE != kTN || g.ws == nullptr) x *= g.alpha;  // partial tiles are scaled when they are added up
                 if (relu) x = fmaxf(x, 0.f);
                 out[r * ldo + c] = x;
             }
@@ -550,7 +550,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
 #pragma unroll
                 for (int t = 0; t < TN; ++t) {
                     float x = acc[t][4 * v4 + vv];
-                    if constexpr (MODE != kTN) x *= g.alpha;
+                    if (MODE != kTN || g.ws == nullptr) x *= g.alpha;  // partial tiles are scaled when they are added up
                     if (relu) x = fmaxf(x, 0.f);
                     if (t * 32 < cols_left) q[t * 32] = x;
                 }
@@ -563,8 +563,9 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
 // added in chain order -- a fixed order, so the result does not depend on scheduling.
 __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ ws, int64_t ws_ld, int64_t ws_slab,
                                                       int splits, int64_t rows, int64_t cols, float *__restrict__ C,
-                                                      int64_t ldc)
+                                                      int64_t ldc, double alpha, const unsigned *__restrict__ run_if)
 {
+    if (run_if != nullptr && *run_if == 0u) return;  // the guarded redo of a split product: nothing to add up
     // 16 output elements per workgroup, 16 interleaved chains per element (chain j adds the partial tiles
     // j, j + 16, ... in order); the chains are then added in chain order: the same sum whatever the timing
     __shared__ double part[16][17];
@@ -596,7 +597,7 @@ __global__ void __launch_bounds__(256) gemm_tn_reduce(const float *__restrict__ 
         double t = part[0][e_local];
 #pragma unroll
         for (int j = 1; j < 16; ++j) t += part[j][e_local];
-        C[r * ldc + c] = (float)t;
+        C[r * ldc + c] = (float)(t * alpha);  // alpha = 1 changes nothing
     }
 }
 
@@ -688,10 +689,77 @@ int gemm_nt_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
     return PLX_OK;
 }
 
+size_t tn_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t splits = tn_splits(M, N, K);
+    if (splits <= 1) return 0;
+    const int64_t ld = (N + 3) / 4 * 4;
+    return (size_t)splits * (size_t)K * (size_t)ld * sizeof(float);
+}
+
+// run_if != NULL: nothing runs (and C is left alone) unless that device word is non-zero
+int gemm_tn_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                 const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, const unsigned *run_if, float alpha, void *stream)
+{
+    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_tn: negative dimension");
+    if (K == 0 || N == 0) return PLX_OK;
+    PLX_REQUIRE(C != nullptr, "gemm_tn: NULL output");
+    PLX_REQUIRE(M == 0 || (A != nullptr && B != nullptr), "gemm_tn: NULL operand");
+    PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_tn: leading dimension too small");
+    PLX_REQUIRE(mask == nullptr || ldmask >= N, "gemm_tn: mask leading dimension too small");
+    hipStream_t st = plx::as_stream(stream);
+    const int64_t splits = tn_splits(std::max<int64_t>(M, 1), N, K);
+    const size_t need = tn_workspace_bytes(M, N, K);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
+        return plx::fail(PLX_ERR_WORKSPACE, "gemm_tn: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
+    g.M = M; g.N = N; g.K = K; g.alpha = alpha;
+    g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
+    g.run_if = run_if; g.n_run_if = run_if != nullptr ? 1 : 0;
+    // every split covers a multiple of the 32-row chunk so that chunk boundaries do not depend on the split
+    g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;
+    const int64_t used = plx::ceil_div(std::max<int64_t>(M, 1), g.rows_per_split);
+    const bool through_ws = splits > 1;  // else one workgroup per tile writes C itself
+    if (through_ws) {
+        g.ws = static_cast<float *>(workspace);
+        g.ws_ld = (N + 3) / 4 * 4;
+        g.ws_slab = K * g.ws_ld;
+    }
+    const int tn = pick_tn(N);
+    dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
+    launch_gemm<kTN>(g, tn, grid, st);
+    PLX_LAUNCH_CHECK("gemm_f32_kernel<TN>");
+    if (through_ws) {
+        const int64_t total = K * N;
+        gemm_tn_reduce<<<(unsigned)plx::ceil_div(total, 16), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc, (double)alpha, run_if);
+        PLX_LAUNCH_CHECK("gemm_tn_reduce");
+    }
+    return PLX_OK;
+}
+
 }  // namespace
 
 // the same two products, launched so that they run only if a device flag is set (used by the split products)
 namespace plx {
+size_t gemm_tn_f32_workspace_bytes(int64_t M, int64_t N, int64_t K) { return tn_workspace_bytes(M, N, K); }
+int64_t gemm_tn_f32_splits(int64_t M, int64_t N, int64_t K) { return tn_splits(std::max<int64_t>(M, 1), N, K); }
+int gemm_tn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                   const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, const unsigned *run_if, float alpha, void *stream)
+{
+    return gemm_tn_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, workspace, workspace_bytes, run_if, alpha, stream);
+}
+// C[e] = alpha * (sum over the partial tiles ws[s][e], s < splits), the tiles added in 16 interleaved chains and the
+// chains in order, in fp64, rounded once
+int gemm_tn_reduce_tiles(const float *ws, int64_t ws_ld, int64_t ws_slab, int splits, int64_t K, int64_t N, float *C, int64_t ldc, float alpha,
+                         void *stream)
+{
+    gemm_tn_reduce<<<(unsigned)ceil_div(K * N, 16), 256, 0, as_stream(stream)>>>(ws, ws_ld, ws_slab, splits, K, N, C, ldc, (double)alpha, nullptr);
+    PLX_LAUNCH_CHECK("gemm_tn_reduce");
+    return PLX_OK;
+}
 int gemm_nn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C,
                    int64_t ldc, unsigned flags, const unsigned *run_if, int n_run_if, void *stream)
 {
@@ -720,53 +788,13 @@ int plx_gemm_nt_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
     return gemm_nt_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, nullptr, 0, stream);
 }
 
-size_t plx_gemm_tn_workspace_bytes(int64_t M, int64_t N, int64_t K)
-{
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    const int64_t splits = tn_splits(M, N, K);
-    if (splits <= 1) return 0;
-    const int64_t ld = (N + 3) / 4 * 4;
-    return (size_t)splits * (size_t)K * (size_t)ld * sizeof(float);
-}
+size_t plx_gemm_tn_workspace_bytes(int64_t M, int64_t N, int64_t K) { return tn_workspace_bytes(M, N, K); }
 
 int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb,
                     float *C, int64_t ldc, const float *mask, int64_t ldmask, void *workspace,
                     size_t workspace_bytes, void *stream)
 {
-    PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_tn: negative dimension");
-    if (K == 0 || N == 0) return PLX_OK;
-    PLX_REQUIRE(C != nullptr, "gemm_tn: NULL output");
-    PLX_REQUIRE(M == 0 || (A != nullptr && B != nullptr), "gemm_tn: NULL operand");
-    PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_tn: leading dimension too small");
-    PLX_REQUIRE(mask == nullptr || ldmask >= N, "gemm_tn: mask leading dimension too small");
-    hipStream_t st = plx::as_stream(stream);
-    const int64_t splits = tn_splits(std::max<int64_t>(M, 1), N, K);
-    const size_t need = plx_gemm_tn_workspace_bytes(M, N, K);
-    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
-        return plx::fail(PLX_ERR_WORKSPACE, "gemm_tn: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-
-    GemmArgs g{};
-    g.A = A; g.B = B; g.C = C; g.mask = mask; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
-    g.M = M; g.N = N; g.K = K; g.alpha = 1.f;
-    g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
-    // every split covers a multiple of the 32-row chunk so that chunk boundaries do not depend on the split
-    g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;
-    const int64_t used = plx::ceil_div(std::max<int64_t>(M, 1), g.rows_per_split);
-    if (splits > 1) {
-        g.ws = static_cast<float *>(workspace);
-        g.ws_ld = (N + 3) / 4 * 4;
-        g.ws_slab = K * g.ws_ld;
-    }
-    const int tn = pick_tn(N);
-    dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
-    launch_gemm<kTN>(g, tn, grid, st);
-    PLX_LAUNCH_CHECK("gemm_f32_kernel<TN>");
-    if (splits > 1) {
-        const int64_t total = K * N;
-        gemm_tn_reduce<<<(unsigned)plx::ceil_div(total, 16), 256, 0, st>>>(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc);
-        PLX_LAUNCH_CHECK("gemm_tn_reduce");
-    }
-    return PLX_OK;
+    return gemm_tn_impl(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, workspace, workspace_bytes, nullptr, 1.f, stream);
 }
 
 }  // extern "C"

@@ -206,7 +206,7 @@ class GCNConvFunction(torch.autograd.Function):
             if ctx.bf16:
                 grad_weight = ops.gemm_tn_bf16(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
             else:
-                grad_weight = ops.gemm_tn(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
+                grad_weight = ops.gemm_tn(agg, grad_output, mask=mask, alpha=ctx.grad_scale, mask_bits=bits)
             grad_weight = grad_weight.reshape(weight.shape)
             timers.stop("GRAD_W = AGG.T * GRAD_OUT")
 

@@ -535,8 +535,10 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
     return c if alpha == 1.0 else scale_by_scalar(c, _device_scalar(alpha, c.device))  # operands the split kernels do not take
 
 
-def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0) -> torch.Tensor:
-    """C[K x N] = alpha * A[M x K]^T.(B * [mask > 0])[M x N]."""
+def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0,
+            mask_bits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C[K x N] = alpha * A[M x K]^T.(B * [mask > 0])[M x N].  ``mask_bits`` (``sign_bits(mask)``) lets the product read
+    the mask as one bit per element."""
     _need_gpu(a, b, mask)
     _need_fp32("gemm_tn", a=a, b=b, mask=mask)
     a, b = _rowmajor(a), _rowmajor(b)
@@ -550,6 +552,21 @@ def gemm_tn(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = Non
             raise ValueError("gemm_tn: mask shape differs from B")
     lib = _lib.load()
     c = torch.empty((k, n), dtype=torch.float32, device=a.device)
+    if mask_bits is not None:
+        if mask is None or mask_bits.dtype != torch.int32 or mask_bits.dim() != 2 or mask_bits.shape[0] != m or \
+                mask_bits.shape[1] < (n + 31) // 32 or mask_bits.stride(1) != 1:
+            raise ValueError("gemm_tn: mask_bits must be int32 [%d x >= %d] beside the fp32 mask" % (m, (n + 31) // 32))
+    if SPLIT_GEMM and k > 0 and n > 0:
+        need = int(lib.plx_gemm_tn_f32_split_workspace_bytes(m, n, k))
+        ws = _aligned_workspace(need, a.device)
+        check(
+            lib.plx_gemm_tn_f32_split(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                      mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                                      mask_bits.data_ptr() if mask_bits is not None else None,
+                                      _ld(mask_bits) if mask_bits is not None else 0, float(alpha), ws.data_ptr(), need, _stream()),
+            "plx_gemm_tn_f32_split",
+        )
+        return c
     need = int(lib.plx_gemm_tn_workspace_bytes(m, n, k))
     ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need else None
     check(

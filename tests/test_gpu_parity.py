@@ -479,9 +479,10 @@ def test_sign_bits_follow_the_product_the_guarded_launch_redoes():
     assert torch.equal(bits.cpu(), _pack_bits(out.cpu()))
 
 
-@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(70000, 128, 100), (40000, 47, 128)])
-def test_gemm_tn_and_mask(m, n, k):
-    say("gemm_tn %dx%dx%d" % (m, n, k))
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(70000, 128, 100), (40000, 47, 128), (30011, 128, 128), (5000, 200, 150), (2500, 64, 300),
+                                                   (31, 128, 128), (1, 5, 3)])
+def test_gemm_tn_and_mask(m, n, k, fp32_gemm_path):
+    say("gemm_tn %dx%dx%d %s" % (m, n, k, fp32_gemm_path))
     gen = torch.Generator().manual_seed(m * 5 + n + k)
     a = torch.randn(m, k, generator=gen)
     g = torch.randn(m, n, generator=gen)
@@ -494,6 +495,50 @@ def test_gemm_tn_and_mask(m, n, k):
     assert rel_err(cm, oracle_c.gemm(a.numpy(), (g * (act > 0)).numpy(), ta=True)) <= FP32_TOL
     # run-to-run bit reproducibility (no atomics, fixed order)
     assert torch.equal(c, ops.gemm_tn(a.to(DEV), g.to(DEV)).cpu())
+    # the mask as one bit per element, and the factor of a dropout layer
+    bits = ops.sign_bits(act.to(DEV))
+    assert torch.equal(ops.gemm_tn(a.to(DEV), g.to(DEV), mask=act.to(DEV), mask_bits=bits).cpu(), cm)
+    c2 = ops.gemm_tn(a.to(DEV), g.to(DEV), mask=act.to(DEV), mask_bits=bits, alpha=2.0).cpu()
+    assert torch.equal(c2, 2.0 * cm)
+    # operands inside wider matrices, off 16-byte boundaries: element loads, same numbers as the oracle
+    wide_a = torch.zeros(m, k + 5)
+    wide_a[:, 3:3 + k] = a
+    wide_g = torch.zeros(m, n + 2)
+    wide_g[:, 1:1 + n] = g
+    cv = ops.gemm_tn(wide_a.to(DEV)[:, 3:3 + k], wide_g.to(DEV)[:, 1:1 + n], mask=act.to(DEV), mask_bits=bits).cpu()
+    assert rel_err(cv, oracle_c.gemm(a.numpy(), (g * (act > 0)).numpy(), ta=True)) <= FP32_TOL
+
+
+def test_gemm_tn_split_keeps_fp32_accuracy_over_millions_of_rows_and_handles_nonfinite_values():
+    say("gemm_tn split: long sums, hard values, Inf / NaN")
+    gen = torch.Generator().manual_seed(77)
+    m, n, k = 1 << 20, 128, 128
+    a = torch.randn(m, k, generator=gen)
+    g = torch.randn(m, n, generator=gen) * torch.exp2(torch.randint(-20, 20, (m, 1), generator=gen).float())  # rows spanning 40 binades
+    ad, gd = a.to(DEV), g.to(DEV)
+    c = ops.gemm_tn(ad, gd).cpu()
+    ref = (a.double().T @ g.double())
+    keep = ops.SPLIT_GEMM
+    ops.SPLIT_GEMM = False
+    c32 = ops.gemm_tn(ad, gd).cpu()
+    ops.SPLIT_GEMM = keep
+    e_split, e_mfma = rel_err(c, ref), rel_err(c32, ref)
+    print("rel err vs fp64: split %.2e, fp32 MFMA %.2e" % (e_split, e_mfma), flush=True)
+    assert e_split <= 2e-6 and e_split <= 4 * e_mfma + 1e-7
+    # exact small integers: every piece product and every partial sum is exact in fp32
+    ai = torch.randint(-3, 4, (4096, 100), generator=gen).float()
+    gi = torch.randint(-3, 4, (4096, 47), generator=gen).float()
+    assert torch.equal(ops.gemm_tn(ai.to(DEV), gi.to(DEV)).cpu(), (ai.double().T @ gi.double()).float())
+    # Inf / NaN in either operand: what torch.mm gives (the fp32 kernel redoes the product)
+    for where in ("a", "g"):
+        a2, g2 = a[:5000].clone(), torch.randn(5000, n, generator=gen)
+        (a2 if where == "a" else g2)[17, 5] = float("inf")
+        (a2 if where == "a" else g2)[99, 7] = float("nan")
+        got = ops.gemm_tn(a2.to(DEV), g2.to(DEV)).cpu()
+        want = torch.mm(a2.t(), g2)
+        assert torch.equal(torch.isnan(got), torch.isnan(want)) and torch.equal(torch.isinf(got), torch.isinf(want))
+        fin = torch.isfinite(want)
+        assert rel_err(got[fin], want[fin].double()) <= FP32_TOL
 
 
 def test_gemm_strided_views_and_tuned_matmul():
