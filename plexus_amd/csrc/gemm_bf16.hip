@@ -281,11 +281,18 @@ constexpr int kRCS = 36;                 // fp32 stride of the staged half tile
 constexpr size_t kRLdsBytes = ((size_t)kRMax * kRBS + (size_t)kRWaves * kRPrivate) * sizeof(uint16_t);
 static_assert(16 * kRCS * 4 <= kRPrivate * 2, "staged half tile must fit the private tile");
 
-template <int TN, bool MASKED>
+// KS: chunk positions of a panel, 8 (K <= 256) or 4 (K <= 128).
+// FAST: A (and the mask) take 16-byte loads and K is a multiple of 8, at least 8.  Every request is then an unconditional
+// load from an address clamped into the matrix (rows past the end repeat the last row and are never stored; columns
+// past K repeat the last eight and meet the zero padding of B), with no branch around it, and every position is
+// multiplied: the wait the compiler places before a chunk is used can then name how many younger requests may stay in
+// flight, where loads inside branches make it wait for all of them.
+template <int TN, bool MASKED, bool FAST = false, int KS = 8>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(const Bf16Args g)
 {
-    constexpr int kSteps = kRMax / kRCK;   // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = MASKED ? 4 : 8;  // register slots = positions ahead that a chunk is requested
+    constexpr int kSteps = KS;             // chunk positions of a panel (positions past K are skipped)
+    constexpr int kRing = MASKED ? 4 : KS; // register slots = positions ahead that a chunk is requested
+    static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;  // [kRMax][kRBS]
     const int lane = threadIdx.x & 63;
@@ -297,7 +304,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 
     // B[N x K] -> LDS, zero beyond N and K up to the tile edges that the MFMAs read
     {
-        const int kp = (K + kRCK - 1) / kRCK * kRCK, vec_per_row = kp / 8;
+        const int kp = FAST ? KS * kRCK : (K + kRCK - 1) / kRCK * kRCK, vec_per_row = kp / 8;
         const int items = 32 * TN * vec_per_row;
         for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
             const int row = id / vec_per_row, q = id % vec_per_row;
@@ -318,7 +325,19 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     int64_t f_panel = first;
     int f_kc = 0;
     uint4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
-    auto fetch = [&](uint4(&dst)[2], uint4(&mdst)[2]) __attribute__((always_inline)) {
+    // `pos`, `of_panel`: the position a request is for (the unconditional form takes them from its caller, where they are
+    // compile-time and loop-invariant values; the guarded form follows its cursor)
+    auto fetch = [&](uint4(&dst)[2], uint4(&mdst)[2], int pos, int64_t of_panel) __attribute__((always_inline)) {
+        if constexpr (FAST) {
+            const int64_t row = min(min(of_panel, n_panels - 1) * 32 + r, g.M - 1);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int k = min(pos * kRCK + half * 16 + 8 * j, K - 8);
+                dst[j] = *reinterpret_cast<const uint4 *>(g.A + row * g.lda + k);
+                if constexpr (MASKED) mdst[j] = *reinterpret_cast<const uint4 *>(g.mask + row * g.ldmask + k);
+            }
+            return;
+        }
         if (f_kc < n_kc && f_panel < n_panels) {
             const int64_t row = f_panel * 32 + r;
             const int k = f_kc * kRCK + half * 16;
@@ -352,15 +371,16 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     const uint16_t *const a_src = apriv + li * kRAS + 8 * h;
     const uint16_t *const b_src = bres + li * kRBS + 8 * h;
 
+    int64_t cur_panel = first;
     auto step = [&](int kc, uint4(&cur)[2], uint4(&mcur)[2]) __attribute__((always_inline)) {
-        const bool live = kc < n_kc;
+        const bool live = FAST || kc < n_kc;  // the unconditional kernel multiplies every position: no branch around its requests
         if (live) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 *reinterpret_cast<uint4 *>(a_dst + 8 * j) = MASKED ? mask8(cur[j], mcur[MASKED ? j : 0]) : cur[j];
             plx::wave_lds_fence();  // the chunk other lanes stored is read below
         }
-        fetch(cur, mcur);
+        fetch(cur, mcur, (kc + kRing) % kSteps, cur_panel + ((kc + kRing) / kSteps) * stride);
         if (live) {
 #pragma unroll
             for (int s = 0; s < kRCK / 16; ++s) {
@@ -382,8 +402,9 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     const int srow = lane >> 2, scq = lane & 3;  // staged half tile: this lane reads 8 columns of row srow
 
 #pragma unroll
-    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0]);
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
     for (int64_t panel = first; panel < n_panels; panel += stride) {
+        cur_panel = panel;
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
         // register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
@@ -422,14 +443,25 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     }
 }
 
+template <int TN, bool MASKED, bool FAST, int KS>
+int launch_nt_resident_one(const Bf16Args &g, unsigned blocks, hipStream_t st)
+{
+    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED, FAST, KS>), kRLdsBytes, allowed);
+    if (rc != PLX_OK) return rc;
+    gemm_bf16_nt_resident_kernel<TN, MASKED, FAST, KS><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    return PLX_OK;
+}
+
+// operands that take 16-byte loads go to the kernel whose requests are unconditional, with as many chunk positions as K needs
 template <int TN, bool MASKED>
 int launch_nt_resident(const Bf16Args &g, unsigned blocks, hipStream_t st)
 {
-    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED>), kRLdsBytes, allowed);
-    if (rc != PLX_OK) return rc;
-    gemm_bf16_nt_resident_kernel<TN, MASKED><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
-    return PLX_OK;
+    if (g.a_vec && g.m_vec && g.K % 8 == 0 && g.K >= 8) {
+        if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, MASKED, true, 4>(g, blocks, st);
+        return launch_nt_resident_one<TN, MASKED, true, 8>(g, blocks, st);
+    }
+    return launch_nt_resident_one<TN, MASKED, false, 8>(g, blocks, st);
 }
 
 // ------------------------------------------------------------------------------------------------

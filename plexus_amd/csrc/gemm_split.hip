@@ -312,13 +312,20 @@ constexpr size_t kRLdsBytes = ((size_t)3 * kRMaxN * kRBS + (size_t)kRWaves * 3 *
 
 // MASK: 0 none, 1 fp32 values beside A (mask > 0 keeps the element), 2 one bit per element
 // DROP: dropout after the ReLU, for N a multiple of 8 (a call of the generator then covers 8 columns of one row)
-template <int TN, int MASK, bool DROP = false>
+// KS: chunk positions of a panel, 8 (K <= 128) or 4 (K <= 64)
+// FAST: A (and the fp32 mask) take 128-bit loads and K >= 4.  Every request is then an unconditional load from an address
+// clamped into the matrix (rows past the end repeat the last row and are never stored; columns past K repeat the last
+// four and meet the zero padding of the planes), with no branch around it: the wait the compiler places before a
+// chunk is used can then name how many younger requests may stay in flight, where loads inside branches make it wait
+// for all of them -- which is what decides the speed of this kernel.
+template <int TN, int MASK, bool DROP = false, bool FAST = false, int KS = 8>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel(const SplitArgs g)
 {
     constexpr bool MASKED = MASK == 1;      // the fp32 mask travels in registers beside its chunk
     constexpr bool BITS = MASK == 2;        // the bit mask of a panel row is four words, loaded once per panel
-    constexpr int kSteps = kRMaxK / kRCK;   // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = MASKED ? 4 : 8;   // register slots = how many positions ahead a chunk is requested
+    constexpr int kSteps = KS;              // chunk positions of a panel (positions past K are skipped)
+    constexpr int kRing = MASKED ? 4 : KS;  // register slots = how many positions ahead a chunk is requested
+    static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;                               // [3][kRMaxN][kRBS]
     constexpr int kBPlane = kRMaxN * kRBS;
@@ -329,13 +336,16 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     uint16_t *const apriv = rlds + 3 * kBPlane + wave * 3 * kRAPlane;  // [3][32][kRAS], this wavefront's
 
     // the planes of B: [3][Np][Kp] in memory -> LDS, 16-byte vectors; rows and columns past Np / Kp stay unread
+    // (the unconditional kernel multiplies all KS chunk positions of all TN column tiles: what lies past Np x Kp is zero)
     {
-        const int vec_per_row = (int)g.Kp / 8;
-        const int items = 3 * (int)g.Np * vec_per_row;
+        const int rows = FAST ? 32 * TN : (int)g.Np;
+        const int vec_per_row = (FAST ? kRCK * KS : (int)g.Kp) / 8;
+        const int items = 3 * rows * vec_per_row;
         for (int id = threadIdx.x; id < items; id += kRWaves * 64) {
-            const int plane = id / ((int)g.Np * vec_per_row), rem = id % ((int)g.Np * vec_per_row);
+            const int plane = id / (rows * vec_per_row), rem = id % (rows * vec_per_row);
             const int row = rem / vec_per_row, q = rem % vec_per_row;
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(g.Bp + ((int64_t)plane * g.Np + row) * g.Kp + q * 8);
+            u32x4 v = u32x4{0u, 0u, 0u, 0u};
+            if (row < (int)g.Np && q * 8 < (int)g.Kp) v = *reinterpret_cast<const u32x4 *>(g.Bp + ((int64_t)plane * g.Np + row) * g.Kp + q * 8);
             *reinterpret_cast<u32x4 *>(bres + plane * kBPlane + row * kRBS + q * 8) = v;
             if (plane == 0 && __builtin_expect(plane0_nonfinite(v), 0)) *g.nonfinite = 1u;  // Inf / NaN in the small operand
         }
@@ -361,7 +371,23 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     u32x4 pb_cur[2], pb_next[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p] = u32x4{~0u, ~0u, ~0u, ~0u};
-    auto fetch = [&](float4(&dst)[2], float4(&mdst)[2]) __attribute__((always_inline)) {
+    // `pos`, `of_panel`: the position a request is for (the unconditional form takes them from its caller, where they are
+    // compile-time and loop-invariant values; the guarded form follows its cursor)
+    auto fetch = [&](float4(&dst)[2], float4(&mdst)[2], int pos, int64_t of_panel) __attribute__((always_inline)) {
+        if constexpr (FAST) {
+            const int64_t panel = min(of_panel, n_panels - 1);
+            const int k = min(pos * kRCK + kq * 4, K - 4);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int64_t row = min(panel * 32 + r + 16 * p, g.M - 1);
+                dst[p] = *reinterpret_cast<const float4 *>(g.A + row * g.lda + k);
+                if constexpr (MASKED) mdst[p] = *reinterpret_cast<const float4 *>(g.mask + row * g.ldmask + k);
+                if constexpr (BITS) {
+                    if (pos == 0) pb_next[p] = *reinterpret_cast<const u32x4 *>(g.mask_bits + row * g.ldw);
+                }
+            }
+            return;
+        }
         if (f_kc < n_kc && f_panel < n_panels) {
             const int64_t row = f_panel * 32 + r;
             const int k = f_kc * kRCK + kq * 4;
@@ -419,9 +445,10 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     const bool relu = (g.flags & PLX_GEMM_RELU) != 0;
     const int N = (int)g.N;
 
+    int64_t cur_panel = first;
     // one position: split the chunk into the private tile, hand its registers to the position kRing ahead, multiply
     auto step = [&](int kc, float4(&cur)[2], float4(&mcur)[2]) __attribute__((always_inline)) {
-        const bool live = kc < n_kc;
+        const bool live = FAST || kc < n_kc;  // the unconditional kernel multiplies every position: no branch around its requests
         if (live) {
             int care = 0;
 #pragma unroll
@@ -448,7 +475,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             if (__builtin_expect(care, 0)) *g.nonfinite = 1u;
             plx::wave_lds_fence();  // the pieces other lanes stored are read below
         }
-        fetch(cur, mcur);
+        fetch(cur, mcur, (kc + kRing) % kSteps, cur_panel + ((kc + kRing) / kSteps) * stride);
         if (live) {
             const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(a_src);
             const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(a_src + kRAPlane);
@@ -466,8 +493,9 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     };
 
 #pragma unroll
-    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0]);
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
     for (int64_t panel = first; panel < n_panels; panel += stride) {
+        cur_panel = panel;
         if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
 #pragma unroll
             for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
@@ -533,14 +561,26 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     }
 }
 
+template <int TN, int MASK, bool DROP, bool FAST, int KS>
+int launch_resident_one(const SplitArgs &g, unsigned blocks, hipStream_t st)
+{
+    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS>), kRLdsBytes,
+                                          allowed);
+    if (rc != PLX_OK) return rc;
+    gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    return PLX_OK;
+}
+
+// operands that take 128-bit loads go to the kernel whose requests are unconditional, with as many chunk positions as K needs
 template <int TN, int MASK, bool DROP = false>
 int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
 {
-    static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK, DROP>), kRLdsBytes, allowed);
-    if (rc != PLX_OK) return rc;
-    gemm_split_nt_resident_kernel<TN, MASK, DROP><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
-    return PLX_OK;
+    if (g.a_vec && g.K >= 4) {
+        if (g.K <= 64) return launch_resident_one<TN, MASK, DROP, true, 4>(g, blocks, st);
+        return launch_resident_one<TN, MASK, DROP, true, 8>(g, blocks, st);
+    }
+    return launch_resident_one<TN, MASK, DROP, false, 8>(g, blocks, st);
 }
 
 template <int MASK, bool DROP = false>
