@@ -70,7 +70,8 @@ int plx_csr_transpose_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *rowp
  * re-base them to the block, sort by (row, col) and add the weights of duplicate edges -- the sequence
  * mask / re-base / sparse_coo_tensor / to_sparse_csr of plexus/utils/dataloader.py:343-367 (and
  * benchmarking/spmm.py:67-84).  rowptr has r1 - r0 + 1 entries; col_out / val_out need room for n_edges entries;
- * the number of stored entries is returned in *nnz_host (the call synchronises `stream` twice to learn it). */
+ * the number of stored entries is returned in *nnz_host (the call synchronises `stream` twice to learn it).
+ * Duplicates of an edge are added one after the other in their input order. */
 size_t plx_coo_block_to_csr_workspace_bytes(int64_t n_edges, int64_t block_rows, int64_t block_cols);
 int plx_coo_block_to_csr_f32(int64_t n_edges, const int64_t *row, const int64_t *col, const float *weight, int64_t r0, int64_t r1,
                              int64_t c0, int64_t c1, int32_t *rowptr, int32_t *col_out, float *val_out, int64_t *nnz_host,
@@ -89,6 +90,33 @@ int plx_relabel_edges_i64(int64_t n_edges, const int64_t *row, const int64_t *co
                           const int64_t *map_col, int64_t n_cols, int64_t *row_out, int64_t *col_out, void *stream);
 int plx_csr_to_coo_i64(int64_t M, int64_t nnz, const int32_t *rowptr, const int32_t *col, int64_t *row_out, int64_t *col_out,
                        void *stream);
+
+/* The permuted adjacency from the CSR of the transpose, in one sort: with `in` an M x K matrix,
+ *   out[new_col[c], i] = in[perm_rows[i], c]   for every stored entry,
+ * a K x M CSR matrix, rows in order and columns ascending within a row.  Called on A^T with perm_rows = perm2 and
+ * new_col = the inverse of perm it yields P.A.P2^T of plexus/utils/dataset.py:137-190 (entry (i, j) of which is
+ * A[perm[i], perm2[j]]).  Whole rows of the source are walked in their new order and their column ids renumbered;
+ * one stable radix sort by the renumbered id then leaves every row of the result ascending, because the walk
+ * already was -- half the sorting passes of building the matrix from its relabelled edge list.  perm_rows must be
+ * a permutation of [0, M) and new_col of [0, K): ids out of range, or rows that do not select exactly nnz entries,
+ * give PLX_ERR_INVALID.  rowptr_out has K + 1 entries, col_out / val_out nnz; the call synchronises `stream` once. */
+size_t plx_csr_permute_transposed_workspace_bytes(int64_t M, int64_t K, int64_t nnz);
+int plx_csr_permute_transposed_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *rowptr, const int32_t *col, const float *val,
+                                   const int64_t *perm_rows, const int64_t *new_col, int32_t *rowptr_out, int32_t *col_out,
+                                   float *val_out, void *workspace, size_t workspace_bytes, void *stream);
+
+/* D^-1/2 (A + I) D^-1/2 as a CSR matrix straight from an edge list -- T.GCNNorm followed by the CSR conversion,
+ * plexus/utils/dataset.py:101 and :158-160.  A vertex without a self loop gets one of weight 1, d is the weighted
+ * in-degree (the sum over the edges that point at a vertex, loops included), duplicate edges are summed, and
+ * edges that name a vertex outside [0, N) are dropped.  `weight` may be NULL (unit weights).  With `transposed`
+ * the result is the transpose, which the reference aggregates with for directed graphs (dataset.py:166-168).
+ * One stable radix sort by column and one by row order the entries; the degrees are read off between the two, so
+ * neither a transpose nor a second pass over the edge list is needed.  rowptr has N + 1 entries; col_out / val_out
+ * need room for n_edges + N entries; *nnz_host receives the number stored (the call synchronises `stream` once). */
+size_t plx_gcn_norm_edges_workspace_bytes(int64_t n_edges, int64_t N);
+int plx_gcn_norm_edges_f32(int64_t n_edges, const int64_t *row, const int64_t *col, const float *weight, int64_t N, int transposed,
+                           int32_t *rowptr, int32_t *col_out, float *val_out, int64_t *nnz_host, void *workspace,
+                           size_t workspace_bytes, void *stream);
 
 /* Host-only row analysis behind plx_spmm_plan_create, exported so it can be tested without a GPU.
  * Rows longer than seg_len are split into ceil(len/seg_len) near-equal segments.  Writes at most

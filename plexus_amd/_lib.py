@@ -32,6 +32,10 @@ SIGNATURES = {
     "plx_invert_permutation_i64": (C.c_int, [_i64, _vp, _vp, _vp]),
     "plx_relabel_edges_i64": (C.c_int, [_i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "plx_csr_to_coo_i64": (C.c_int, [_i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "plx_csr_permute_transposed_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "plx_csr_permute_transposed_f32": (C.c_int, [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "plx_gcn_norm_edges_workspace_bytes": (_sz, [_i64, _i64]),
+    "plx_gcn_norm_edges_f32": (C.c_int, [_i64, _vp, _vp, _vp, _i64, C.c_int, _vp, _vp, _vp, C.POINTER(_i64), _vp, _sz, _vp]),
     "plx_spmm_segments_host": (C.c_int, [_i64, _vp, _i32, C.POINTER(_i64), C.POINTER(_i64), _vp, _vp, _i64, _vp, _vp, _i64]),
     "plx_spmm_plan_create": (C.c_int, [C.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _i32, _vp]),
     "plx_spmm_plan_destroy": (C.c_int, [_vp]),

@@ -48,6 +48,8 @@ int gemm_tn_f32_if(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                    const float *mask, int64_t ldmask, void *workspace, size_t workspace_bytes, const unsigned *run_if, float alpha, void *stream);
 int gemm_tn_reduce_tiles(const float *ws, int64_t ws_ld, int64_t ws_slab, int splits, int64_t K, int64_t N, float *C, int64_t ldc, float alpha,
                          void *stream);
+// dinv[r] = 1 / sqrt(sum of val[rowptr[r] .. rowptr[r + 1])), 0 where the sum is not positive (elementwise.hip)
+int row_sums_rsqrt(int64_t M, const int32_t *rowptr, const float *val, float *dinv, void *stream);
 
 #if defined(__HIPCC__)
 // Orders the LDS accesses of one wavefront for the compiler: lanes that exchange data through a tile private to their

@@ -316,6 +316,14 @@ int scale_common(int64_t n, const T *x, const float *scale, T *y, void *stream)
 
 }  // namespace
 
+int plx::row_sums_rsqrt(int64_t M, const int32_t *rowptr, const float *val, float *dinv, void *stream)
+{
+    if (M <= 0) return PLX_OK;
+    row_dinv_kernel<<<(unsigned)plx::ceil_div(M, 4), 256, 0, plx::as_stream(stream)>>>(M, rowptr, val, dinv);
+    PLX_LAUNCH_CHECK("row_dinv_kernel");
+    return PLX_OK;
+}
+
 extern "C" {
 
 int plx_scale_by_device_scalar_f32(int64_t n, const float *x, const float *scale, float *y, void *stream)
@@ -438,9 +446,8 @@ int plx_gcn_norm_csr_f32(int64_t M, const int32_t *rowptr, const int32_t *col, c
     if (M == 0) return PLX_OK;
     PLX_REQUIRE(rowptr && col && val_in && val_out && dinv, "gcn_norm: NULL operand");
     hipStream_t st = plx::as_stream(stream);
-    const unsigned blocks = (unsigned)plx::ceil_div(M, 4);
-    row_dinv_kernel<<<blocks, 256, 0, st>>>(M, rowptr, val_in, dinv);
-    PLX_LAUNCH_CHECK("row_dinv_kernel");
+    int rc = plx::row_sums_rsqrt(M, rowptr, val_in, dinv, stream);
+    if (rc != PLX_OK) return rc;
     gcn_scale_kernel<<<256 * 32, 256, 0, st>>>(M, rowptr, col, val_in, dinv, val_out);
     PLX_LAUNCH_CHECK("gcn_scale_kernel");
     return PLX_OK;

@@ -36,17 +36,35 @@ __global__ void __launch_bounds__(256) relabel_edges_kernel(int64_t n_edges, con
     }
 }
 
-// entry j belongs to the row r with rowptr[r] <= j < rowptr[r + 1]: binary search per entry (the row
-// pointer is small against the entries and stays in cache), so hub rows cost no more than others
+// entry j belongs to the row r with rowptr[r] <= j < rowptr[r + 1].  A workgroup takes 2,048 consecutive entries,
+// finds the rows of its first and last entry once, and every entry then searches only between those two (no steps
+// at all inside a long row), so hub rows cost no more than others.
+constexpr int kCooPerBlock = 2048;
 __global__ void __launch_bounds__(256) csr_to_coo_kernel(int64_t M, int64_t nnz, const int32_t *__restrict__ rowptr,
                                                          const int32_t *__restrict__ col, int64_t *__restrict__ row_out,
                                                          int64_t *__restrict__ col_out)
 {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < nnz; j += stride) {
+    __shared__ int32_t bounds[2];
+    const int64_t e0 = (int64_t)blockIdx.x * kCooPerBlock;
+    const int64_t e1 = min(e0 + kCooPerBlock, nnz) - 1;
+    if (threadIdx.x < 2) {
+        const int64_t j = threadIdx.x == 0 ? e0 : e1;
         int64_t lo = 0, hi = M;  // the answer r satisfies lo <= r < hi
         while (hi - lo > 1) {
             const int64_t mid = (lo + hi) >> 1;
+            if ((int64_t)rowptr[mid] <= j)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        bounds[threadIdx.x] = (int32_t)lo;
+    }
+    __syncthreads();
+    const int32_t r_first = bounds[0], r_last = bounds[1];
+    for (int64_t j = e0 + threadIdx.x; j <= e1; j += 256) {
+        int32_t lo = r_first, hi = r_last + 1;
+        while (hi - lo > 1) {
+            const int32_t mid = lo + ((hi - lo) >> 1);
             if ((int64_t)rowptr[mid] <= j)
                 lo = mid;
             else
@@ -92,7 +110,7 @@ int plx_csr_to_coo_i64(int64_t M, int64_t nnz, const int32_t *rowptr, const int3
     PLX_REQUIRE(M >= 0 && nnz >= 0 && M < (1ll << 31) - 1 && nnz < (1ll << 31), "csr_to_coo: bad shape");
     if (nnz == 0) return PLX_OK;
     PLX_REQUIRE(M > 0 && rowptr && col && row_out && col_out, "csr_to_coo: NULL operand or entries without rows");
-    csr_to_coo_kernel<<<grid_for(nnz), 256, 0, plx::as_stream(stream)>>>(M, nnz, rowptr, col, row_out, col_out);
+    csr_to_coo_kernel<<<(unsigned)plx::ceil_div(nnz, kCooPerBlock), 256, 0, plx::as_stream(stream)>>>(M, nnz, rowptr, col, row_out, col_out);
     PLX_LAUNCH_CHECK("csr_to_coo_kernel");
     return PLX_OK;
 }

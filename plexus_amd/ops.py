@@ -54,12 +54,13 @@ class CsrMatrix:
     """A CSR matrix prepared for the SpMM kernel: int32 indices, fp32 values and the row plan.
 
     Built from a torch sparse-CSR tensor (``from_torch``) or from raw arrays.  The plan (row binning
-    and the split of long rows into segments) is computed once; the int32 arrays are owned here and
-    outlive it.  The scratch of the products is cached on the object, so products of one matrix must
+    and the split of long rows into segments) is computed once (with ``defer_plan``: at the first
+    product); the int32 arrays are owned here and outlive it.  The scratch of the products is cached on the object, so products of one matrix must
     be ordered (one stream, or events between streams); different matrices are independent.
     """
 
-    def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, val: torch.Tensor, shape, seg_len: int = 0):
+    def __init__(self, rowptr: torch.Tensor, col: torch.Tensor, val: torch.Tensor, shape, seg_len: int = 0,
+                 defer_plan: bool = False):
         _need_gpu(rowptr, col, val)
         m, k = int(shape[0]), int(shape[1])
         nnz = int(col.numel())
@@ -86,15 +87,11 @@ class CsrMatrix:
         self.shape = (m, k)
         self.nnz = nnz
         self.device = val.device
-        self._plan = _lib.C.c_void_p()
-        check(
-            lib.plx_spmm_plan_create(
-                _lib.C.byref(self._plan), m, k, nnz, self.rowptr.data_ptr(), self.col.data_ptr() if nnz else None,
-                int(seg_len), _stream(),
-            ),
-            "plx_spmm_plan_create",
-        )
+        self._seg_len = int(seg_len)
+        self._plan_handle = None
         self._ws: Optional[torch.Tensor] = None
+        if not defer_plan:
+            self.prepare()  # checks the arrays too: a malformed matrix is refused here, not at its first product
 
     @classmethod
     def from_torch(cls, a: torch.Tensor, seg_len: int = 0) -> "CsrMatrix":
@@ -102,14 +99,37 @@ class CsrMatrix:
             raise ValueError("expected a sparse CSR tensor, got layout %s" % a.layout)
         return cls(a.crow_indices(), a.col_indices(), a.values(), a.shape, seg_len)
 
+    def prepare(self) -> "CsrMatrix":
+        """Build the row plan now (it allocates and waits for the device, so not under stream capture)."""
+        self._plan
+        return self
+
+    @property
+    def _plan(self):
+        """The row plan of the products (bins, segments, hub tables).  The builders of this module hand out
+        matrices whose arrays are well-formed by construction and defer it to the first product, so that a
+        matrix that is only converted or transposed never pays for it."""
+        if self._plan_handle is None:
+            handle = _lib.C.c_void_p()
+            m, k = self.shape
+            check(
+                _lib.load().plx_spmm_plan_create(
+                    _lib.C.byref(handle), m, k, self.nnz, self.rowptr.data_ptr(), self.col.data_ptr() if self.nnz else None,
+                    self._seg_len, _stream(),
+                ),
+                "plx_spmm_plan_create",
+            )
+            self._plan_handle = handle
+        return self._plan_handle
+
     def __del__(self):
-        plan = getattr(self, "_plan", None)
+        plan = getattr(self, "_plan_handle", None)
         if plan is not None and plan.value:
             try:
                 _lib.load().plx_spmm_plan_destroy(plan)
             except Exception:
                 pass
-            self._plan = None
+            self._plan_handle = None
 
     @property
     def n_long_rows(self) -> int:
@@ -207,7 +227,7 @@ def csr_transpose(a: CsrMatrix, seg_len: int = 0) -> CsrMatrix:
                                   val_t.data_ptr() if a.nnz else None, ws.data_ptr(), need, _stream()),
         "plx_csr_transpose_f32",
     )
-    return CsrMatrix(rowptr_t, col_t, val_t, (k, m), seg_len)
+    return CsrMatrix(rowptr_t, col_t, val_t, (k, m), seg_len, defer_plan=True)
 
 
 def csr_pair_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, shape, row_range=None, col_range=None,
@@ -247,14 +267,84 @@ def csr_from_edges(edge_index: torch.Tensor, edge_weight: torch.Tensor, shape, r
     )
     del ws
     k = int(nnz.value)
-    return CsrMatrix(rowptr, col_out[:k].clone(), val_out[:k].clone(), (mb, kb), seg_len)
+    return CsrMatrix(rowptr, _trimmed(col_out, k), _trimmed(val_out, k), (mb, kb), seg_len, defer_plan=True)
+
+
+def _trimmed(t: torch.Tensor, k: int) -> torch.Tensor:
+    """The first k entries of a buffer sized for the worst case: a view when little is wasted, else a copy."""
+    return t[:k] if k * 10 >= t.numel() * 9 else t[:k].clone()
+
+
+def gcn_norm_from_edges(edge_index: torch.Tensor, edge_weight: Optional[torch.Tensor], num_nodes: int,
+                        transposed: bool = False, seg_len: int = 0) -> "CsrMatrix":
+    """D^-1/2 (A + I) D^-1/2 (its transpose with ``transposed``) as a CSR matrix from an edge list, in one call:
+    missing self loops get weight 1, d is the weighted in-degree, duplicate edges are summed -- T.GCNNorm and the
+    CSR conversion of plexus/utils/dataset.py:101,158-168."""
+    _need_gpu(edge_index)
+    ei = edge_index.to(torch.int64)
+    rows, cols = ei[0].contiguous(), ei[1].contiguous()
+    w = None if edge_weight is None else edge_weight.to(torch.float32).contiguous()
+    n_edges, n = int(rows.numel()), int(num_nodes)
+    lib = _lib.load()
+    dev = edge_index.device
+    rowptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    col_out = torch.empty(max(n_edges + n, 1), dtype=torch.int32, device=dev)
+    val_out = torch.empty(max(n_edges + n, 1), dtype=torch.float32, device=dev)
+    need = int(lib.plx_gcn_norm_edges_workspace_bytes(n_edges, n))
+    ws = _aligned_workspace(need, dev)
+    nnz = _lib.C.c_int64(0)
+    check(
+        lib.plx_gcn_norm_edges_f32(n_edges, rows.data_ptr() if n_edges else None, cols.data_ptr() if n_edges else None,
+                                   w.data_ptr() if (w is not None and n_edges) else None, n, int(bool(transposed)),
+                                   rowptr.data_ptr(), col_out.data_ptr(), val_out.data_ptr(), _lib.C.byref(nnz), ws.data_ptr(), need,
+                                   _stream()),
+        "plx_gcn_norm_edges_f32",
+    )
+    del ws
+    k = int(nnz.value)
+    return CsrMatrix(rowptr, _trimmed(col_out, k), _trimmed(val_out, k), (n, n), seg_len, defer_plan=True)
+
+
+def csr_permute(a: "CsrMatrix", perm_rows: torch.Tensor, perm_cols: torch.Tensor, a_t: Optional["CsrMatrix"] = None,
+                seg_len: int = 0) -> "CsrMatrix":
+    """P_rows . A . P_cols^T with P[i, perm[i]] = 1 as a CSR matrix: entry (i, j) of the result is entry
+    (perm_rows[i], perm_cols[j]) of A (plexus/utils/dataset.py:137-190).
+
+    Works from the CSR of A^T (``a_t``; built here when not given -- pass it when several permutations of one
+    matrix are wanted): its rows are walked in the order perm_cols, the row ids in them renumbered, and one stable
+    sort by the new row id leaves every row of the result in ascending column order."""
+    a = as_csr(a)
+    _need_gpu(perm_rows, perm_cols)
+    m, k = a.shape
+    if perm_rows.numel() != m or perm_cols.numel() != k:
+        raise ValueError("csr_permute: a %dx%d matrix needs permutations of %d rows and %d columns" % (m, k, m, k))
+    if a_t is None:
+        a_t = csr_transpose(a)
+    elif a_t.shape != (k, m) or a_t.nnz != a.nnz:
+        raise ValueError("csr_permute: a_t is not the transpose of a")
+    walk = perm_cols.to(torch.int64).contiguous()
+    new_row = invert_permutation(perm_rows)
+    lib = _lib.load()
+    rowptr = torch.empty(m + 1, dtype=torch.int32, device=a.device)
+    col_out = torch.empty(a.nnz, dtype=torch.int32, device=a.device)
+    val_out = torch.empty(a.nnz, dtype=torch.float32, device=a.device)
+    need = int(lib.plx_csr_permute_transposed_workspace_bytes(k, m, a.nnz))
+    ws = _aligned_workspace(need, a.device)
+    check(
+        lib.plx_csr_permute_transposed_f32(k, m, a.nnz, a_t.rowptr.data_ptr(), a_t.col.data_ptr() if a.nnz else None,
+                                           a_t.val.data_ptr() if a.nnz else None, walk.data_ptr() if k else None,
+                                           new_row.data_ptr() if m else None, rowptr.data_ptr(), col_out.data_ptr() if a.nnz else None,
+                                           val_out.data_ptr() if a.nnz else None, ws.data_ptr(), need, _stream()),
+        "plx_csr_permute_transposed_f32",
+    )
+    return CsrMatrix(rowptr, col_out, val_out, (m, k), seg_len, defer_plan=True)
 
 
 def invert_permutation(perm: torch.Tensor) -> torch.Tensor:
     """inv with inv[perm[i]] = i (int64, on the device)."""
     _need_gpu(perm)
     perm = perm.to(torch.int64).contiguous()
-    inv = torch.empty_like(perm)
+    inv = torch.full_like(perm, -1)  # a slot no entry of perm names stays -1, which the users of the map refuse
     check(_lib.load().plx_invert_permutation_i64(perm.numel(), perm.data_ptr(), inv.data_ptr(), _stream()), "plx_invert_permutation_i64")
     return inv
 

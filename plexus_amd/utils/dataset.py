@@ -59,31 +59,13 @@ def normalize_features(x: torch.Tensor) -> torch.Tensor:
     return x / x.sum(dim=-1, keepdim=True).clamp_(min=1.0)
 
 
-def add_remaining_self_loops(edge_index: torch.Tensor, edge_weight: torch.Tensor, num_nodes: int, fill: float = 1.0):
-    """Every vertex gets exactly one self loop: an existing loop keeps its weight, the others get ``fill``
-    (the first step of T.GCNNorm, dataset.py:101).  Non-loop edges keep their order; loops are appended."""
-    row, col = edge_index[0], edge_index[1]
-    off_diag = row != col
-    loop_w = torch.full((num_nodes,), fill, dtype=edge_weight.dtype, device=edge_weight.device)
-    loop_w[row[~off_diag]] = edge_weight[~off_diag]
-    loops = torch.arange(num_nodes, dtype=edge_index.dtype, device=edge_index.device)
-    ei = torch.cat([edge_index[:, off_diag], torch.stack([loops, loops])], dim=1)
-    return ei, torch.cat([edge_weight[off_diag], loop_w])
-
-
 def gcn_norm(edge_index: torch.Tensor, edge_weight: Optional[torch.Tensor], num_nodes: int, directed: bool = False) -> ops.CsrMatrix:
     """D^-1/2 (A + I) D^-1/2 as a CSR matrix on the device, d = weighted in-degree (sum over the edges that
     point at a vertex, self loop included), as T.GCNNorm computes it (dataset.py:101).
 
     With ``directed`` the result is the transpose, which the reference aggregates with for directed graphs
     (dataset.py:166-168).  Duplicate edges are summed, as the CSR conversion of :158-160 does."""
-    if edge_weight is None:
-        edge_weight = torch.ones(edge_index.shape[1], dtype=torch.float32, device=edge_index.device)
-    ei, w = add_remaining_self_loops(edge_index.to(torch.int64), edge_weight.to(torch.float32), num_nodes)
-    # CSR of the transpose: row t holds the edges that point at t, so its row sum is the in-degree
-    at = ops.csr_from_edges(torch.stack([ei[1], ei[0]]), w, (num_nodes, num_nodes))
-    at_hat = ops.CsrMatrix(at.rowptr, at.col, ops.gcn_norm_csr(at), at.shape)
-    return at_hat if directed else ops.csr_transpose(at_hat)
+    return ops.gcn_norm_from_edges(edge_index, edge_weight, num_nodes, transposed=directed)
 
 
 def degree_bucket_labels(edge_index: torch.Tensor, num_nodes: int, num_classes: int) -> torch.Tensor:
@@ -100,13 +82,11 @@ def degree_bucket_labels(edge_index: torch.Tensor, num_nodes: int, num_classes: 
     return y
 
 
-def permute_adjacency(adj: ops.CsrMatrix, perm_rows: torch.Tensor, perm_cols: torch.Tensor):
+def permute_adjacency(adj: ops.CsrMatrix, perm_rows: torch.Tensor, perm_cols: torch.Tensor, adj_t: Optional[ops.CsrMatrix] = None):
     """(edge_index, edge_weight) of P_rows . A . P_cols^T with P[i, perm[i]] = 1, i.e. entry (i, j) of the result
-    is entry (perm_rows[i], perm_cols[j]) of A (dataset.py:137-216), sorted by (row, col)."""
-    n = adj.shape[0]
-    ei, w = ops.csr_to_edges(adj)
-    ei = ops.relabel_edges(ei, ops.invert_permutation(perm_rows), ops.invert_permutation(perm_cols))
-    return ops.csr_to_edges(ops.csr_from_edges(ei, w, (n, adj.shape[1])))
+    is entry (perm_rows[i], perm_cols[j]) of A (dataset.py:137-216), sorted by (row, col).  ``adj_t`` is the CSR of
+    A^T, which the permutation works from; give it when one matrix is permuted more than once."""
+    return ops.csr_to_edges(ops.csr_permute(adj, perm_rows, perm_cols, a_t=adj_t))
 
 
 def preprocess_graph(
@@ -136,8 +116,9 @@ def preprocess_graph(
     if x is None:
         x = normalize_features(torch.rand(n, num_features, generator=generator).to(dev))
     adj = gcn_norm(edge_index, edge_weight, n, directed=directed)
+    adj_t = ops.csr_transpose(adj)  # both permutations below work from it
     if y is None:
-        ei_norm, _ = ops.csr_to_edges(adj if not directed else ops.csr_transpose(adj))
+        ei_norm, _ = ops.csr_to_edges(adj if not directed else adj_t)
         y = degree_bucket_labels(ei_norm, n, num_classes)
     y = torch.nan_to_num(y.reshape(-1).to(torch.float64), nan=-1.0).to(torch.int64) if y.is_floating_point() else y.reshape(-1).to(torch.int64)
     if perm is None:
@@ -146,10 +127,10 @@ def preprocess_graph(
         perm2 = torch.randperm(n, generator=generator)
     perm = perm.to(dev)
     p_cols = perm2.to(dev) if double_perm else perm
-    ei, w = permute_adjacency(adj, perm, p_cols)
+    ei, w = permute_adjacency(adj, perm, p_cols, adj_t)
     out = ProcessedGraph(edge_index=ei, edge_weight=w, x=x.to(dev)[p_cols, :], y=y.to(dev)[perm], num_classes=int(num_classes))
     if double_perm:
-        out.edge_index_2, out.edge_weight_2 = permute_adjacency(adj, p_cols, perm)
+        out.edge_index_2, out.edge_weight_2 = permute_adjacency(adj, p_cols, perm, adj_t)
         out.y_2 = y.to(dev)[p_cols]
     return out
 

@@ -89,6 +89,97 @@ def test_gcn_norm_from_edge_list(directed):
     assert rel_err(got_w.cpu(), sorted_edges(ref64[0].flip(0) if directed else ref64[0], ref64[1], n)[1]) <= FP32_TOL
 
 
+@pytest.mark.parametrize("directed", [False, True])
+def test_gcn_norm_with_duplicates_loops_isolated_vertices_and_strays(directed):
+    """Raw (uncoalesced) edge lists: duplicate edges and duplicate self loops are summed, isolated vertices get their
+    loop, edges that name a vertex outside the graph are dropped, and a hub vertex collects a long column."""
+    say("dataset.gcn_norm raw edge list directed=%s" % directed)
+    n = 4000
+    g = torch.Generator().manual_seed(11)
+    ei = torch.randint(0, n - 50, (2, 30000), generator=g)  # the last 50 vertices stay isolated
+    hub = torch.stack([torch.randint(0, n - 50, (6000,), generator=g), torch.full((6000,), 17)])  # in-degree ~6000
+    dup = ei[:, :500]  # every one of these edges twice more
+    loops = torch.tensor([[3, 3, 3, 99], [3, 3, 3, 99]])  # vertex 3 has three loops, vertex 99 one
+    ei = torch.cat([ei, hub, dup, loops, dup], dim=1)
+    ei = ei[:, torch.randperm(ei.shape[1], generator=g)]
+    w = torch.rand(ei.shape[1], generator=g) + 0.1
+    ref_ei, ref_w = po.gcn_norm(ei, n, w)
+    ref64 = po.gcn_norm(ei, n, w, dtype=torch.float64)[1]
+    if directed:
+        ref_ei = ref_ei.flip(0)
+    coo = torch.sparse_coo_tensor(ref_ei, ref_w, (n, n)).coalesce()  # duplicates summed, sorted by (row, col)
+    coo64 = torch.sparse_coo_tensor(ref_ei, ref64, (n, n)).coalesce()
+    stray = torch.tensor([[-1, 5, n, 2], [4, n + 3, 1, -7]])
+    ei_dev = torch.cat([ei[:, :100], stray, ei[:, 100:]], dim=1).to(DEV)
+    w_dev = torch.cat([w[:100], torch.ones(4), w[100:]]).to(DEV)
+    a = D.gcn_norm(ei_dev, w_dev, n, directed=directed)
+    got_ei, got_w = ops.csr_to_edges(a)
+    assert a.nnz == coo.indices().shape[1] and int(a.rowptr[-1]) == a.nnz
+    assert torch.equal(got_ei.cpu(), coo.indices())
+    assert rel_err(got_w.cpu(), coo.values()) <= FP32_TOL and rel_err(got_w.cpu(), coo64.values()) <= FP32_TOL
+    # unit weights when none are given; integers, so the sums are exact and the values follow from the degrees alone
+    b = D.gcn_norm(ei.to(DEV), None, n, directed=directed)
+    ref1_ei, ref1_w = po.gcn_norm(ei, n, None)
+    coo1 = torch.sparse_coo_tensor(ref1_ei.flip(0) if directed else ref1_ei, ref1_w, (n, n)).coalesce()
+    b_ei, b_w = ops.csr_to_edges(b)
+    assert torch.equal(b_ei.cpu(), coo1.indices()) and rel_err(b_w.cpu(), coo1.values()) <= FP32_TOL
+
+
+def test_gcn_norm_of_a_graph_without_edges_is_the_identity():
+    say("dataset.gcn_norm without edges")
+    a = D.gcn_norm(torch.zeros((2, 0), dtype=torch.int64, device=DEV), None, 7)
+    assert torch.equal(a.rowptr.cpu(), torch.arange(8, dtype=torch.int32)) and torch.equal(a.col.cpu(), torch.arange(7, dtype=torch.int32))
+    assert torch.equal(a.val.cpu(), torch.ones(7))
+    h = torch.randn(7, 5, device=DEV)
+    assert torch.equal(ops.spmm(a, h), h)  # and the deferred plan is built by the first product
+
+
+def test_csr_permute_matches_the_sparse_products_and_refuses_a_non_permutation():
+    say("ops.csr_permute")
+    n, k = 3000, 2500  # rectangular, with empty rows and one hub row
+    g = torch.Generator().manual_seed(12)
+    counts = torch.randint(0, 9, (n,), generator=g)
+    counts[::13] = 0
+    counts[77] = 2400
+    rows = torch.repeat_interleave(torch.arange(n), counts)
+    cols = torch.cat([torch.randperm(k, generator=g)[:c] for c in counts.tolist()])
+    vals = torch.rand(rows.numel(), generator=g)
+    dense = torch.zeros(n, k)
+    dense[rows, cols] = vals
+    a = ops.csr_from_edges(torch.stack([rows, cols]).to(DEV), vals.to(DEV), (n, k))
+    p_r, p_c = torch.randperm(n, generator=g), torch.randperm(k, generator=g)
+    got = ops.csr_permute(a, p_r.to(DEV), p_c.to(DEV))
+    want = dense[p_r][:, p_c].to_sparse_csr()  # new[i, j] = old[perm_rows[i], perm_cols[j]]
+    assert torch.equal(got.rowptr.cpu().long(), want.crow_indices()) and torch.equal(got.col.cpu().long(), want.col_indices())
+    assert torch.equal(got.val.cpu(), want.values())  # values only move
+    h = torch.randn(k, 9, device=DEV)
+    assert rel_err(ops.spmm(got, h).cpu(), (dense[p_r][:, p_c].double() @ h.cpu().double()).float()) <= FP32_TOL
+    a_t = ops.csr_transpose(a)
+    again = ops.csr_permute(a, p_r.to(DEV), p_c.to(DEV), a_t=a_t)  # from a transpose built by the caller
+    assert torch.equal(again.rowptr, got.rowptr) and torch.equal(again.col, got.col) and torch.equal(again.val, got.val)
+    twice = p_r.clone()
+    twice[5] = twice[6]  # one row twice, another never
+    with pytest.raises(RuntimeError, match="outside"):
+        ops.csr_permute(a, twice.to(DEV), p_c.to(DEV), a_t=a_t)
+    stray = p_r.clone()
+    stray[3] = n
+    with pytest.raises(RuntimeError, match="outside"):
+        ops.csr_permute(a, stray.to(DEV), p_c.to(DEV), a_t=a_t)
+    col_counts = torch.bincount(cols, minlength=k)
+    twice = p_c.clone()
+    twice[5] = p_c[int((col_counts[p_c] != col_counts[p_c[5]]).nonzero()[0])]  # a column of another length in place of one
+    with pytest.raises(RuntimeError, match="not a permutation"):
+        ops.csr_permute(a, p_r.to(DEV), twice.to(DEV), a_t=a_t)
+    with pytest.raises(ValueError):
+        ops.csr_permute(a, p_r.to(DEV), p_c.to(DEV), a_t=a)  # not the transpose's shape
+    with pytest.raises(ValueError):
+        ops.csr_permute(a, p_r[:-1].to(DEV), p_c.to(DEV))
+    empty = ops.CsrMatrix(torch.zeros(5, dtype=torch.int64, device=DEV), torch.zeros(0, dtype=torch.int64, device=DEV),
+                          torch.zeros(0, device=DEV), (4, 4))
+    e = ops.csr_permute(empty, torch.randperm(4).to(DEV), torch.randperm(4).to(DEV))
+    assert e.nnz == 0 and torch.equal(e.rowptr.cpu(), torch.zeros(5, dtype=torch.int32))
+
+
 @pytest.mark.parametrize("double_perm,directed", [(True, False), (False, False), (True, True)])
 def test_preprocess_graph_matches_sparse_product_permutation(double_perm, directed):
     say("preprocess_graph double_perm=%s directed=%s" % (double_perm, directed))
