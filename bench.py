@@ -743,7 +743,7 @@ def main():
         line["prep_ms"] = dict(ctx["prep"])
         if not args.spmm_only:
             line["prep_ms"].update(bench_preprocessing(ctx, dev))
-        if args.config == 3 and not args.no_side_configs:
+        if args.config == 3 and not args.no_side_configs and not args.spmm_only:
             side = {}
             t5 = time.time()
             side["5"] = compact(bench_on_graph(args, dev, 5, ctx, headline=False))

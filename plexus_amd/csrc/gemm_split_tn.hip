@@ -46,13 +46,8 @@ struct TnArgs {
 
 __global__ void zero_flag_kernel(unsigned *flag) { *flag = 0u; }
 
-#ifndef PLX_TN_NP
-#define PLX_TN_NP 8  // wavefronts that fetch, split and store
-#endif
-#ifndef PLX_TN_NC
-#define PLX_TN_NC 4  // wavefronts that multiply
-#endif
-constexpr int kNP = PLX_TN_NP, kNC = PLX_TN_NC;
+constexpr int kNP = 8;  // wavefronts that fetch, split and store
+constexpr int kNC = 4;  // wavefronts that multiply
 constexpr int kThreads = 64 * (kNP + kNC);
 static_assert((kNP == 4 || kNP == 8) && (kNC == 4 || kNC == 8), "four or eight wavefronts per role");
 
@@ -179,11 +174,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint32_t p0, p1, p2;
-#ifdef PLX_TN_NO_SPLIT
-                p0 = __float_as_uint(x0[e]); p1 = __float_as_uint(x1[e]); p2 = p0 ^ p1;
-#else
                 split2(x0[e], x1[e], p0, p1, p2);
-#endif
                 dst[e * kSW] = p0;
                 dst[e * kSW + plane_words] = p1;
                 dst[e * kSW + 2 * plane_words] = p2;
@@ -297,11 +288,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
                 const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(bt);
                 const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(bt + BN * kSW * 2);
                 const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bt + 2 * BN * kSW * 2);
-#ifdef PLX_TN_NO_MFMA
-                acc[t][0] += (float)(a0[0] + a1[1] + a2[2] + b0[3] + b1[4] + b2[5]);
-#else
                 acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
-#endif
             }
         }
     };
