@@ -41,6 +41,7 @@ TRAFFIC_PROFILES = {
     "f32": os.path.join("profiles", "spmm_csr_config3_fp32_pmc.txt"),
     "bf16": os.path.join("profiles", "spmm_csr_config5_bf16_pmc.txt"),
     "c4": os.path.join("profiles", "spmm_csr_config4_fp32_pmc.txt"),
+    "c2": os.path.join("profiles", "spmm_csr_config2_fp32_pmc.txt"),
 }
 
 
@@ -222,7 +223,7 @@ def bench_side_config(args, dev, config):
     spmm, cpu_of = {}, {}
     for d in widths:
         rec, h = spmm_record(a, d, torch.float32, args.spmm_iters)
-        traffic, source = measured_spmm_traffic("c4", m, nnz, d) if config == 4 else (None, None)
+        traffic, source = measured_spmm_traffic("c%d" % config, m, nnz, d)
         rec["roofline"] = roofline_block(rec, "spmm_csr_kernel (A.H, D=%d, fp32%s)" % (d, ", passes over 64-column slices" if config == 2 else ""),
                                          traffic, source)
         if not args.no_cpu:
