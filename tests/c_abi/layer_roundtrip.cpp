@@ -270,6 +270,87 @@ int main()
     compare("GRAD_AGG = G.W^T", to_host(d_gagg, gagg_ref.size()), gagg_ref);
     compare("GRAD_H = A^T.GRAD_AGG", to_host(d_gh, gh_ref.size()), gh_ref);
 
+    // ---- GRAD_W on the bf16 matrix cores from exact splits, on operands whose rows take 128-bit loads: AGG^T . GRAD_AGG ----
+    {
+        const size_t sws2_bytes = plx_gemm_tn_f32_split_workspace_bytes(n, d_in, d_in);
+        char *d_sws2 = device_alloc<char>(sws2_bytes);
+        float *d_c2 = device_alloc<float>((size_t)(d_in * d_in));
+        PLX_OK_OR_DIE(plx_gemm_tn_f32_split(n, d_in, d_in, d_agg, d_in, d_gagg, d_in, d_c2, d_in, nullptr, 0, nullptr, 0, 2.0f, d_sws2,
+                                            sws2_bytes, st));
+        const std::vector<float> agg_dev = to_host(d_agg, agg_ref.size()), gagg_dev = to_host(d_gagg, gagg_ref.size());
+        std::vector<float> c2_ref((size_t)(d_in * d_in));
+        orc_gemm_f32_acc64(1, 0, d_in, d_in, n, agg_dev.data(), d_in, gagg_dev.data(), d_in, c2_ref.data(), d_in);
+        for (float &x : c2_ref) x *= 2.0f;
+        compare("2 AGG^T.GRAD_AGG from splits", to_host(d_c2, c2_ref.size()), c2_ref);
+        HIP_OK(hipFree(d_sws2));
+        HIP_OK(hipFree(d_c2));
+    }
+
+    // ---- graph preparation: the normalised CSR straight from an edge list that lacks some self loops, and a permuted copy ----
+    {
+        std::vector<int64_t> e_row, e_col;
+        for (int64_t r = 0; r < n; ++r)
+            for (int64_t j = a.rowptr[(size_t)r]; j < a.rowptr[(size_t)r + 1]; ++j) {
+                const int64_t c = a.col[(size_t)j];
+                if (r == c && r % 5 == 0) continue;  // these vertices get their loop from the call
+                e_row.push_back(r);
+                e_col.push_back(c);
+            }
+        std::reverse(e_row.begin(), e_row.end());  // any order will do
+        std::reverse(e_col.begin(), e_col.end());
+        const int64_t n_edges = (int64_t)e_row.size();
+        int64_t *d_erow = to_device(e_row), *d_ecol = to_device(e_col);
+        int32_t *d_rp2 = device_alloc<int32_t>((size_t)n + 1), *d_ci2 = device_alloc<int32_t>((size_t)(n_edges + n));
+        float *d_v2 = device_alloc<float>((size_t)(n_edges + n));
+        const size_t nws_bytes = plx_gcn_norm_edges_workspace_bytes(n_edges, n);
+        char *d_nws = device_alloc<char>(nws_bytes);
+        int64_t nnz2 = 0;
+        PLX_OK_OR_DIE(plx_gcn_norm_edges_f32(n_edges, d_erow, d_ecol, nullptr, n, 0, d_rp2, d_ci2, d_v2, &nnz2, d_nws, nws_bytes, st));
+        const std::vector<int32_t> rp2 = to_host(d_rp2, (size_t)n + 1), ci2 = to_host(d_ci2, (size_t)std::min(nnz2, nnz));
+        bool same = nnz2 == nnz;
+        for (size_t i = 0; same && i < rp2.size(); ++i) same = rp2[i] == (int32_t)a.rowptr[i];
+        for (size_t i = 0; same && i < ci2.size(); ++i) same = ci2[i] == (int32_t)a.col[i];
+        std::printf("%-28s %8lld entries   indices %s\n", "normalised CSR from edges", (long long)nnz2, same ? "identical  ok" : "DIFFER  FAILED");
+        if (!same) ++g_failures;
+        else compare("its values", to_host(d_v2, (size_t)nnz), norm_ref);
+
+        // out[new_col[c], i] = A^T[walk[i], c]: with A^T, walk = perm2 and new_col = the inverse of perm this is P.A.P2^T
+        std::vector<int64_t> walk((size_t)n), new_id((size_t)n);
+        for (int64_t i = 0; i < n; ++i) {
+            walk[(size_t)i] = n - 1 - i;
+            new_id[(size_t)i] = (i * 7 + 3) % n;  // a bijection: 7 and 5000 are coprime
+        }
+        int64_t *d_walk = to_device(walk), *d_new = to_device(new_id);
+        int32_t *d_rp3 = device_alloc<int32_t>((size_t)n + 1), *d_ci3 = device_alloc<int32_t>((size_t)nnz);
+        float *d_v3 = device_alloc<float>((size_t)nnz);
+        const size_t pws_bytes = plx_csr_permute_transposed_workspace_bytes(n, n, nnz);
+        char *d_pws = device_alloc<char>(pws_bytes);
+        PLX_OK_OR_DIE(plx_csr_permute_transposed_f32(n, n, nnz, d_rowptr_t, d_col_t, d_val_t, d_walk, d_new, d_rp3, d_ci3, d_v3, d_pws,
+                                                     pws_bytes, st));
+        std::vector<std::vector<std::pair<int64_t, float>>> rows3((size_t)n);
+        for (int64_t i = 0; i < n; ++i) {  // moved rows in ascending i, so every row of the result comes out ascending
+            const int64_t src = walk[(size_t)i];
+            for (int64_t j = at.rowptr[(size_t)src]; j < at.rowptr[(size_t)src + 1]; ++j)
+                rows3[(size_t)new_id[(size_t)at.col[(size_t)j]]].push_back({i, at.val[(size_t)j]});
+        }
+        const std::vector<int32_t> rp3 = to_host(d_rp3, (size_t)n + 1), ci3 = to_host(d_ci3, (size_t)nnz);
+        const std::vector<float> v3 = to_host(d_v3, (size_t)nnz);
+        bool same3 = true;
+        int64_t p = 0;
+        for (int64_t r = 0; r < n && same3; ++r) {
+            same3 = rp3[(size_t)r] == (int32_t)p;
+            for (const auto &e : rows3[(size_t)r]) {
+                same3 = same3 && ci3[(size_t)p] == (int32_t)e.first && v3[(size_t)p] == e.second;
+                ++p;
+            }
+        }
+        same3 = same3 && rp3[(size_t)n] == (int32_t)nnz;
+        std::printf("%-28s %8lld entries   %s\n", "permuted CSR from A^T", (long long)nnz, same3 ? "identical  ok" : "DIFFER  FAILED");
+        if (!same3) ++g_failures;
+        void *mine[] = {d_erow, d_ecol, d_rp2, d_ci2, d_v2, d_nws, d_walk, d_new, d_rp3, d_ci3, d_v3, d_pws};
+        for (void *q : mine) HIP_OK(hipFree(q));
+    }
+
     // ---- one AdamW step on the weight (examples/train.py:155-159: lr 3e-3, no weight decay) ----
     float *d_m = device_alloc<float>(w.size()), *d_v = device_alloc<float>(w.size());
     HIP_OK(hipMemsetAsync(d_m, 0, w.size() * sizeof(float), st));
