@@ -616,6 +616,152 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_tn_kernel(const Bf16Args g
     }
 }
 
+// The same product for K and N up to 256 where one of them exceeds 128: with 128 x 128 tiles a workgroup reads half of A
+// and half of B, so every operand crosses the memory system twice.  Here one workgroup of 16 wavefronts owns the whole
+// 256 x 256 tile of C for its stretch of rows: A, B and the mask are read once.  Wavefront w multiplies the 32 rows
+// 32 (w % 8) of C by the column half w / 8.  Operands take 128-bit loads (K and N multiples of 8).  A chunk is requested
+// right after the previous one has been stored to LDS, so its loads are in flight for a whole turn of the loop; whole
+// chunks are fetched without a branch (a thread whose columns lie beyond K or N reads column 0 and stores nothing), so
+// the compiler waits for exactly the loads it is about to use; the last, partial chunk of a stretch is fetched with guards.
+// Stretches, chunk order and the order of the products inside a chunk are those of the tiled kernel: the same bits.
+constexpr int kWThreads = 1024;
+constexpr int kWTile = 512 * kS;  // bf16 elements per buffer: 256 columns of A and 256 of B, one LDS row each
+constexpr size_t kWLdsBytes = 2 * (size_t)kWTile * sizeof(uint16_t);
+
+template <bool MASKED>
+__global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16Args g)
+{
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds_w[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 31;
+    const int h = lane >> 5;
+    const int rb = wave & 7, ch = wave >> 3;
+    const int64_t mbeg = (int64_t)blockIdx.x * g.rows_per_split;
+    const int64_t mend = min(mbeg + g.rows_per_split, g.M);
+
+    // thread (mp, cq): row pair (2 mp, 2 mp + 1) of a chunk, columns 8 cq .. 8 cq + 7 of A and of B
+    const int mp = threadIdx.x & 31;
+    const int cq = threadIdx.x >> 5;
+    const bool a_ok = cq * 8 < g.K, b_ok = cq * 8 < g.N;
+    const uint16_t *pa = g.A + (mbeg + 2 * mp) * g.lda + (a_ok ? cq * 8 : 0);
+    const uint16_t *pb = g.B + (mbeg + 2 * mp) * g.ldb + (b_ok ? cq * 8 : 0);
+    const uint16_t *pm = MASKED ? g.mask + (mbeg + 2 * mp) * g.ldmask + (b_ok ? cq * 8 : 0) : nullptr;
+
+    uint4 ra[2], rb2[2], rmk[2];
+    auto advance = [&]() {
+        pa += (int64_t)kBK * g.lda;
+        pb += (int64_t)kBK * g.ldb;
+        if constexpr (MASKED) pm += (int64_t)kBK * g.ldmask;
+    };
+    auto fetch_whole = [&]() {  // all 64 rows of the chunk exist
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
+            rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
+            if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
+        }
+        advance();
+    };
+    auto fetch_any = [&](int64_t m0) {
+        const int rows_left = (int)min(max(mend - m0 - 2 * mp, (int64_t)0), (int64_t)2);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ra[j] = zero4();
+            rb2[j] = zero4();
+            rmk[j] = zero4();
+            if (j < rows_left) {
+                ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
+                rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
+                if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
+            }
+        }
+        advance();
+    };
+    // transposed stash: word e of the pair holds (row 2 mp, row 2 mp + 1) of column 8 cq + e
+    auto stash_pair = [&](uint16_t *t, const uint4 &r0, const uint4 &r1) {
+        const uint32_t a[4] = {r0.x, r0.y, r0.z, r0.w};
+        const uint32_t b[4] = {r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t lo = (e & 1) ? (a[e >> 1] >> 16) : (a[e >> 1] & 0xffffu);
+            const uint32_t hi = (e & 1) ? (b[e >> 1] >> 16) : (b[e >> 1] & 0xffffu);
+            *reinterpret_cast<uint32_t *>(t + (cq * 8 + e) * kS + 2 * mp) = lo | (hi << 16);
+        }
+    };
+    auto stash = [&](int buf) {
+        uint16_t *at = lds_w + buf * kWTile;
+        uint16_t *bt = at + 256 * kS;
+        if (a_ok) stash_pair(at, ra[0], ra[1]);
+        if (b_ok) {
+            if constexpr (MASKED)
+                stash_pair(bt, mask8(rb2[0], rmk[0]), mask8(rb2[1], rmk[1]));
+            else
+                stash_pair(bt, rb2[0], rb2[1]);
+        }
+    };
+
+    floatx16 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    const bool works = rb * 32 < g.K && ch * 128 < g.N;  // uniform over the wavefront
+    auto compute = [&](int buf) {
+        if (!works) return;
+        const uint16_t *at = lds_w + buf * kWTile;
+        const uint16_t *bt = at + (256 + ch * 128) * kS;
+#pragma unroll
+        for (int s = 0; s < kBK / 16; ++s) {
+            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(at + (rb * 32 + li) * kS + 16 * s + 8 * h);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(bt + (t * 32 + li) * kS + 16 * s + 8 * h);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+    };
+
+    const int64_t rows = max(mend - mbeg, (int64_t)0);
+    const int64_t n_chunks = (rows + kBK - 1) / kBK;
+    const int64_t n_whole = rows / kBK;  // chunks 0 .. n_whole - 1 have all their rows
+    // chunk 0 into buffer 0, chunk 1 requested
+    if (n_chunks > 0) {
+        if (n_whole > 0) fetch_whole(); else fetch_any(mbeg);
+        stash(0);
+    }
+    if (n_chunks > 1) {
+        if (n_whole > 1) fetch_whole(); else fetch_any(mbeg + kBK);
+    }
+    __syncthreads();
+    int64_t c = 0;
+    for (; c + 2 < n_whole; ++c) {  // steady state: chunk c in LDS, c + 1 in registers, c + 2 whole and about to be requested
+        compute((int)(c & 1));
+        stash((int)((c + 1) & 1));
+        fetch_whole();
+        __syncthreads();
+    }
+    for (; c < n_chunks; ++c) {
+        compute((int)(c & 1));
+        if (c + 1 < n_chunks) stash((int)((c + 1) & 1));
+        if (c + 2 < n_chunks) fetch_any(mbeg + (c + 2) * kBK);
+        __syncthreads();
+    }
+
+    float *out = g.ws + (int64_t)blockIdx.x * g.ws_slab;  // always split over the rows: alpha is applied when the partial tiles are added
+    if (works) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int64_t col = ch * 128 + t * 32 + li;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t r = rb * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                if (col < g.N && r < g.K) out[r * g.ws_ld + col] = acc[t][v];
+            }
+        }
+    }
+}
+
 // C[e] = alpha * sum over splits of ws[s][e]; four interleaved chains, added in chain order
 __global__ void __launch_bounds__(256) gemm_bf16_tn_reduce(const float *__restrict__ ws, int64_t ws_ld, int64_t ws_slab,
                                                            int splits, int64_t rows, int64_t cols, float alpha,
@@ -797,7 +943,20 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     const int tn = pick_tn(N);
     dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0 && N % 8 == 0;
-    if (mask != nullptr) {
+    if (vec && splits > 1 && K <= 256 && N <= 256 && (K > kBM || N > 128)) {
+        // more than one 128 x 128 tile, at most 256 x 256: one workgroup per stretch holds the whole tile and reads every operand once
+        static std::atomic<uint64_t> allowed_m{0}, allowed_p{0};
+        int rc;
+        if (mask != nullptr) {
+            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<true>), kWLdsBytes, allowed_m);
+            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<true><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+        } else {
+            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<false>), kWLdsBytes, allowed_p);
+            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<false><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+        }
+        if (rc != PLX_OK) return rc;
+        PLX_LAUNCH_CHECK("gemm_bf16_tn_wide_kernel");
+    } else if (mask != nullptr) {
         if (vec) launch_tn<true, true>(g, tn, grid, st);
         else launch_tn<true, false>(g, tn, grid, st);
     } else {

@@ -975,7 +975,8 @@ def test_gemm_nt_bf16_dropout_mask_is_the_oracles(m, n, k, p):
     assert not torch.equal(c2 > 0, keep)
 
 
-@pytest.mark.parametrize("m,n,k", BF16_GEMM_SHAPES + [(70000, 256, 256), (40000, 47, 256)])
+# the last three: more than one 128 x 128 tile and at most 256 x 256, which one workgroup per stretch of rows holds whole
+@pytest.mark.parametrize("m,n,k", BF16_GEMM_SHAPES + [(70000, 256, 256), (40000, 47, 256), (70001, 256, 136), (33333, 200, 256), (20011, 136, 248)])
 def test_gemm_tn_bf16(m, n, k):
     say("gemm_tn_bf16 %dx%dx%d" % (m, n, k))
     gen = torch.Generator().manual_seed(m * 5 + n + k)
