@@ -44,6 +44,7 @@ struct SplitArgs {
     unsigned flags;
     unsigned *nonfinite;  // device word raised when an operand holds a value the split cannot carry
     int a_vec;  // A (and mask) 16-byte aligned, leading dimensions and K multiples of 4: 128-bit loads
+    int c_vec;  // C 16-byte aligned, ldc and N multiples of 4: 128-bit stores
     // dropout after the ReLU (resident NT kernel): element e = row * N + col is kept iff 16-bit lane e % 8 of
     // Philox-4x32-10(counter = (e / 8, offset), key = seed) is >= thresh16, and then scaled by keep_scale
     uint32_t thresh16, seed_lo, seed_hi, off_lo, off_hi;
@@ -529,6 +530,46 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             }
             plx::wave_lds_fence();
         }
+        // C in 128-bit stores: a 64-lane store takes the memory pipeline as long for 4 bytes per lane as for 16, and the 64
+        // narrow stores of a panel fill the wavefront's queue of outstanding memory operations, behind which the requests of
+        // the next panel wait.  The tile goes through the private LDS tile (32 rows of 36 floats: exactly its size), where a
+        // lane picks up four consecutive columns of four rows; 16 stores per panel instead of 64.
+        if constexpr (FAST && !DROP) {
+            if (g.c_vec) {
+                float *const stage = reinterpret_cast<float *>(apriv);  // [32][36]
+                const int rr = lane >> 3, c4 = (lane & 7) * 4;
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    const bool col_ok = li + t * 32 < N;
+                    uint32_t word = 0;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int d = 8 * (v / 4) + (v % 4);
+                        float x = acc[t][v];
+                        if (relu) x = fmaxf(x, 0.f);
+                        stage[(d + 4 * h) * 36 + li] = x;
+                        if (g.relu_bits != nullptr) {
+                            const uint64_t votes = __ballot(col_ok && x > 0.f);
+                            if (li == v) word = h ? (uint32_t)(votes >> 32) : (uint32_t)votes;
+                        }
+                        acc[t][v] = 0.f;
+                    }
+                    if (g.relu_bits != nullptr && li < 16) {
+                        const int d = 8 * (li / 4) + (li % 4);
+                        if (d < rows_left && t * 32 < N) g.relu_bits[(r0 + d) * g.ldw + t] = word;
+                    }
+                    plx::wave_lds_fence();
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int64_t row = panel * 32 + rr + 8 * j;
+                        const float4 x4 = *reinterpret_cast<const float4 *>(stage + (rr + 8 * j) * 36 + c4);
+                        if (row < g.M && t * 32 + c4 < N) *reinterpret_cast<float4 *>(g.C + row * g.ldc + t * 32 + c4) = x4;
+                    }
+                    plx::wave_lds_fence();  // the next tile, or the next panel's first chunk, overwrites the staging
+                }
+                continue;
+            }
+        }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
             const bool col_ok = li + t * 32 < N;
@@ -747,6 +788,7 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     SplitArgs g{};
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = mm_flags; g.a_vec = vec;
+    g.c_vec = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 4 == 0 && N % 4 == 0) ? 1 : 0;
     g.nonfinite = flag_words;
     g.ldw = ldw;
     if (drop != nullptr) {
