@@ -375,11 +375,21 @@ def bench_dense_kernels(args, dev):
     rows = []
 
     def rec(name, fn, bytes_, flops):
-        ms = time_gpu(fn, 3, args.spmm_iters)
+        ms = time_gpu(fn, 10, args.spmm_iters)  # ten warm-up launches: the first kernels of a process meet a cold clock
         rows.append({"kernel": name, "ms": ms, "GBps": bytes_ / ms / 1e6, "TFLOPs": flops / ms / 1e9,
                      "frac_hbm_peak": bytes_ / ms / 1e6 / HBM_PEAK_GBPS})
         note("%-44s %7.3f ms  %7.0f GB/s (%4.1f %% of HBM peak)  %6.1f TFLOP/s" % (name, ms, rows[-1]["GBps"], 100 * rows[-1]["frac_hbm_peak"],
                                                                              rows[-1]["TFLOPs"]))
+
+    # the chip comes out of idle slowly: a kernel timed in the first tenths of a second of load runs 15-20 % longer than the
+    # same kernel later on, however many warm-up launches of its own it gets.  Half a second of streaming work first.
+    burn = torch.empty(1 << 28, device=dev)
+    t_burn = time.time()
+    while time.time() - t_burn < 0.5:
+        for _ in range(20):
+            burn.add_(1.0)
+        torch.cuda.synchronize()
+    del burn
 
     for li in range(3):
         k, n = dims[li], dims[li + 1]
