@@ -400,13 +400,18 @@ def bench_dense_kernels(args, dev):
             w = torch.randn(k, n, device=dev) * 0.1
             wt16, w16 = ops.cast_bf16(w, transpose=True), ops.cast_bf16(w)
             act = torch.relu(S.normal_features(m, n, dev, seed=20 + li)).to(torch.bfloat16)
-            rec("OUT = AGG.W %dx%d bf16%s" % (k, n, "" if last else " +ReLU +dropout"),
-                (lambda: ops.gemm_nt_bf16(a, wt16)) if last else (lambda: ops.gemm_nt_bf16(a, wt16, relu=True, dropout_p=0.5, seed=1, offset=li)),
-                e * m * (k + n), 2.0 * m * k * n)
-            rec("GRAD_AGG = (G*mask).W^T %dx%d bf16" % (n, k), (lambda: ops.gemm_nt_bf16(g, w16)) if last else (lambda: ops.gemm_nt_bf16(g, w16, mask=act, alpha=2.0)),
-                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
-            rec("GRAD_W = AGG^T.(G*mask) %dx%d bf16" % (k, n), (lambda: ops.gemm_tn_bf16(a, g)) if last else (lambda: ops.gemm_tn_bf16(a, g, mask=act, alpha=2.0)),
-                e * m * (k + n) + (0 if last else e * m * n), 2.0 * m * k * n)
+            # a hidden layer's product also writes the sign bits of its result, and the backward products read the mask in that form
+            bits = None if last else ops.sign_bits(act.float())
+            rec("OUT = AGG.W %dx%d bf16%s" % (k, n, "" if last else " +ReLU +dropout +sign bits"),
+                (lambda: ops.gemm_nt_bf16(a, wt16)) if last else (lambda: ops.gemm_nt_bf16(a, wt16, relu=True, dropout_p=0.5, seed=1, offset=li,
+                                                                                          want_bits=True)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
+            rec("GRAD_AGG = (G*mask).W^T %dx%d bf16%s" % (n, k, "" if last else " (bit mask)"),
+                (lambda: ops.gemm_nt_bf16(g, w16)) if last else (lambda: ops.gemm_nt_bf16(g, w16, mask=act, mask_bits=bits, alpha=2.0)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
+            rec("GRAD_W = AGG^T.(G*mask) %dx%d bf16%s" % (k, n, "" if last else " (bit mask)"),
+                (lambda: ops.gemm_tn_bf16(a, g)) if last else (lambda: ops.gemm_tn_bf16(a, g, mask=act, mask_bits=bits, alpha=2.0)),
+                e * m * (k + n) + (0 if last else m * n // 8), 2.0 * m * k * n)
         else:
             a = S.normal_features(m, k, dev, seed=li)
             g = S.normal_features(m, n, dev, seed=10 + li)

@@ -371,6 +371,26 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
                      float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, void *workspace,
                      size_t workspace_bytes, void *stream);
 
+/* The mask of a bf16 hidden layer as one bit per element, as for fp32 storage above (bit c % 32 of word
+ * [row * ldw + c / 32] says that element (row, c) is positive; examples/train.py:77-78 is the ReLU it stands for).
+ *   plx_gemm_nt_bf16_bits: plx_gemm_nt_bf16 that also writes the bits of its result C (after ReLU and dropout) to
+ *     `relu_bits` (may be NULL; ldw_out >= ceil(N / 32)) -- for N, K <= 256 with N a multiple of 8 and 16-byte rows of C,
+ *     PLX_ERR_UNSUPPORTED otherwise -- and reads the mask of A from `mask_bits` (may be NULL; ldw >= ceil(K / 32)) where
+ *     it can: N, K <= 256, A in 16-byte rows with K a multiple of 8, rows of bits 16-byte aligned with ldw a multiple
+ *     of 4 and at least 4 (K <= 128) or 8 words.  The bf16 `mask`, which must say the same, is read elsewhere.
+ *   plx_gemm_tn_bf16_bits: plx_gemm_tn_bf16 reading the mask of B from `mask_bits` (ldw >= ceil(N / 32)) in the kernel
+ *     that holds a whole tile of up to 256 x 256 (16-byte rows, K and N multiples of 8, more than one 128 x 128 tile),
+ *     from `mask` elsewhere.
+ * A hidden layer of 2,449,029 x 256 then reads 78 MB of mask in each backward product in place of 1.25 GB.  Same
+ * results bit for bit as with the bf16 mask.   Reference call sites as plx_gemm_nt_bf16 / plx_gemm_tn_bf16. */
+int plx_gemm_nt_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                          uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw,
+                          uint32_t *relu_bits, int64_t ldw_out, float alpha, unsigned flags, float dropout_p, uint64_t seed,
+                          uint64_t offset, void *stream);
+int plx_gemm_tn_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                          float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw,
+                          float alpha, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Y = bf16(X) (transpose = 0, Y is [M x N]) or bf16(X^T) (transpose = 1, Y is [N x M]); X is [M x N] fp32. */
 int plx_cast_f32_bf16(int64_t M, int64_t N, const float *X, int64_t ldx, uint16_t *Y, int64_t ldy, int transpose,
                       void *stream);

@@ -88,6 +88,9 @@ SIGNATURES = {
                                    C.c_uint64, C.c_uint64, _vp]),
     "plx_gemm_tn_bf16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "plx_gemm_tn_bf16": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz, _vp]),
+    "plx_gemm_nt_bf16_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _u32,
+                                        _f32, C.c_uint64, C.c_uint64, _vp]),
+    "plx_gemm_tn_bf16_bits": (C.c_int, [_i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _f32, _vp, _sz, _vp]),
     "plx_cast_f32_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, C.c_int, _vp]),
     "plx_softmax_xent_bf16": (C.c_int, [_i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _f32, _vp, _vp, _i64, _vp, _sz, _vp]),
 }

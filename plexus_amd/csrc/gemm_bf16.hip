@@ -47,6 +47,12 @@ struct Bf16Args {
     float keep_scale;    // 1 / (1 - p)
     uint32_t seed_lo, seed_hi, off_lo, off_hi;
     int a_vec, b_vec, c_vec, m_vec;
+    // the mask as one bit per element (bit c % 32 of word [row * ldw + c / 32]): read in place of `mask` by the resident NT
+    // kernel and the whole-tile TN kernel, written for C (its positive elements) by the resident NT kernel
+    const uint32_t *mask_bits;
+    int64_t ldw;
+    uint32_t *relu_bits;
+    int64_t ldw_out;
     // TN only
     int64_t rows_per_split;
     float *ws;
@@ -71,6 +77,10 @@ __device__ __forceinline__ uint32_t mask2(uint32_t v, uint32_t m)
     const uint32_t hi = plx::bf16_positive(m >> 16) ? 0xffff0000u : 0u;
     return v & (lo | hi);
 }
+
+// the same with the mask as 8 bits, bit e for element e
+__device__ __forceinline__ uint32_t keep2(uint32_t v, uint32_t b) { return v & (((b & 1u) ? 0x0000ffffu : 0u) | ((b & 2u) ? 0xffff0000u : 0u)); }
+__device__ __forceinline__ uint4 mask8_bits(uint4 v, uint32_t b) { return make_uint4(keep2(v.x, b), keep2(v.y, b >> 2), keep2(v.z, b >> 4), keep2(v.w, b >> 6)); }
 
 __device__ __forceinline__ uint4 mask8(uint4 v, uint4 m) { return make_uint4(mask2(v.x, m.x), mask2(v.y, m.y), mask2(v.z, m.z), mask2(v.w, m.w)); }
 
@@ -287,11 +297,17 @@ static_assert(16 * kRCS * 4 <= kRPrivate * 2, "staged half tile must fit the pri
 // past K repeat the last eight and meet the zero padding of B), with no branch around it, and every position is
 // multiplied: the wait the compiler places before a chunk is used can then name how many younger requests may stay in
 // flight, where loads inside branches make it wait for all of them.
-template <int TN, bool MASKED, bool FAST = false, int KS = 8>
+// MASK: 0 none, 1 bf16 values beside A (positive keeps the element), 2 one bit per element (FAST only; the KS words of a
+// panel row come with the panel's first chunk and stay in registers, so the ring is as deep as without a mask)
+// WBITS: also write the sign bits of C (a kernel of its own, so that the others do not carry its registers)
+template <int TN, int MASK, bool FAST = false, int KS = 8, bool WBITS = false>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(const Bf16Args g)
 {
+    constexpr bool MASKED = MASK == 1;
+    constexpr bool BITS = MASK == 2;
+    static_assert(!BITS || FAST, "the bit mask is read by the unconditional kernel only");
     constexpr int kSteps = KS;             // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = MASKED ? 4 : KS; // register slots = positions ahead that a chunk is requested
+    constexpr int kRing = (MASKED || ((WBITS || BITS) && TN > 4)) ? 4 : KS; // register slots = positions ahead that a chunk is requested
     static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;  // [kRMax][kRBS]
@@ -325,11 +341,20 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     int64_t f_panel = first;
     int f_kc = 0;
     uint4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
+    uint4 pb_cur[KS / 4], pb_next[KS / 4];  // bit mask: word kc of the lane's row covers chunk position kc
+#pragma unroll
+    for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q] = make_uint4(~0u, ~0u, ~0u, ~0u);
     // `pos`, `of_panel`: the position a request is for (the unconditional form takes them from its caller, where they are
     // compile-time and loop-invariant values; the guarded form follows its cursor)
     auto fetch = [&](uint4(&dst)[2], uint4(&mdst)[2], int pos, int64_t of_panel) __attribute__((always_inline)) {
         if constexpr (FAST) {
             const int64_t row = min(min(of_panel, n_panels - 1) * 32 + r, g.M - 1);
+            if constexpr (BITS) {
+                if (pos == 0) {
+#pragma unroll
+                    for (int q = 0; q < KS / 4; ++q) pb_next[q] = *reinterpret_cast<const uint4 *>(g.mask_bits + row * g.ldw + 4 * q);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int k = min(pos * kRCK + half * 16 + 8 * j, K - 8);
@@ -376,8 +401,16 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
         const bool live = FAST || kc < n_kc;  // the unconditional kernel multiplies every position: no branch around its requests
         if (live) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                *reinterpret_cast<uint4 *>(a_dst + 8 * j) = MASKED ? mask8(cur[j], mcur[MASKED ? j : 0]) : cur[j];
+            for (int j = 0; j < 2; ++j) {
+                uint4 v = cur[j];
+                if constexpr (MASKED) v = mask8(v, mcur[j]);
+                if constexpr (BITS) {
+                    const uint4 w4 = pb_cur[kc >> 2];
+                    const uint32_t word = (kc & 3) == 0 ? w4.x : ((kc & 3) == 1 ? w4.y : ((kc & 3) == 2 ? w4.z : w4.w));
+                    v = mask8_bits(v, word >> (16 * half + 8 * j));
+                }
+                *reinterpret_cast<uint4 *>(a_dst + 8 * j) = v;
+            }
             plx::wave_lds_fence();  // the chunk other lanes stored is read below
         }
         fetch(cur, mcur, (kc + kRing) % kSteps, cur_panel + ((kc + kRing) / kSteps) * stride);
@@ -403,8 +436,13 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 
 #pragma unroll
     for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
+    uint32_t wkeep[2][(TN + 3) / 4] = {};
     for (int64_t panel = first; panel < n_panels; panel += stride) {
         cur_panel = panel;
+        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
+#pragma unroll
+            for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q];
+        }
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
         // register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
@@ -420,6 +458,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
                 plx::wave_lds_fence();  // before the next pass (or the next panel's chunks) overwrites the tile
                 const int64_t row = panel * 32 + 16 * pass + srow;
                 const int col = t * 32 + scq * 8;
+                uint32_t positive = 0;  // bit e: element col + e of this row is stored positive
                 if (row < g.M && col < N) {
                     float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
@@ -433,35 +472,90 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
 #pragma unroll
                         for (int e = 0; e < 8; ++e) x[e] = plx::dropout_lane16(rnd, e) >= g.thresh16 ? x[e] * g.keep_scale : 0.f;
                     }
-                    *reinterpret_cast<uint4 *>(C + row * g.ldc + col) = make_uint4(plx::pack_bf16x2(x[0], x[1]), plx::pack_bf16x2(x[2], x[3]),
-                                                                                   plx::pack_bf16x2(x[4], x[5]), plx::pack_bf16x2(x[6], x[7]));
+                    const uint4 packed = make_uint4(plx::pack_bf16x2(x[0], x[1]), plx::pack_bf16x2(x[2], x[3]),
+                                                    plx::pack_bf16x2(x[4], x[5]), plx::pack_bf16x2(x[6], x[7]));
+                    *reinterpret_cast<uint4 *>(C + row * g.ldc + col) = packed;
+                    if constexpr (WBITS) {
+                        // a stored bf16 is positive exactly when its 16 bits, read as a signed integer, are: two packed
+                        // integer operations turn both halves of a word into 0 or 1
+                        typedef short short2_t __attribute__((ext_vector_type(2)));
+                        const uint32_t pk[4] = {packed.x, packed.y, packed.z, packed.w};
+                        uint32_t both = 0;  // bit 2 e: element 2 e; bit 16 + 2 e: element 2 e + 1
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            short2_t hv = __builtin_bit_cast(short2_t, pk[e]);
+                            hv = __builtin_elementwise_max(__builtin_elementwise_min(hv, (short2_t){1, 1}), (short2_t){0, 0});
+                            both |= __builtin_bit_cast(uint32_t, hv) << (2 * e);
+                        }
+                        positive = (both & 0x55u) | ((both >> 15) & 0xaau);
+                    }
+                }
+                if constexpr (WBITS) {
+                    // the four lanes of a row hold its 32 columns of this tile: one word, which lane t % 4 of them keeps, so
+                    // that a row's words leave in two stores of all 64 lanes per half panel rather than one of 16 per tile
+                    int word = (int)(positive << (8 * scq));
+                    word |= __builtin_amdgcn_update_dpp(0, word, 0xB1, 0xF, 0xF, true);  // lanes 1 0 3 2 of the quad
+                    word |= __builtin_amdgcn_update_dpp(0, word, 0x4E, 0xF, 0xF, true);  // lanes 2 3 0 1
+                    if ((t & 3) == scq) wkeep[pass][t >> 2] = (uint32_t)word;
                 }
             }
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
         }
+        if constexpr (WBITS) {
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                const int64_t row = panel * 32 + 16 * pass + srow;
+#pragma unroll
+                for (int q = 0; q < (TN + 3) / 4; ++q)
+                    if (row < g.M && (scq + 4 * q) * 32 < N) g.relu_bits[row * g.ldw_out + scq + 4 * q] = wkeep[pass][q];
+            }
+        }
     }
 }
 
-template <int TN, bool MASKED, bool FAST, int KS>
+template <int TN, int MASK, bool FAST, int KS, bool WBITS = false>
 int launch_nt_resident_one(const Bf16Args &g, unsigned blocks, hipStream_t st)
 {
     static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASKED, FAST, KS>), kRLdsBytes, allowed);
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_nt_resident_kernel<TN, MASK, FAST, KS, WBITS>), kRLdsBytes,
+                                          allowed);
     if (rc != PLX_OK) return rc;
-    gemm_bf16_nt_resident_kernel<TN, MASKED, FAST, KS><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    gemm_bf16_nt_resident_kernel<TN, MASK, FAST, KS, WBITS><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
     return PLX_OK;
 }
 
 // operands that take 16-byte loads go to the kernel whose requests are unconditional, with as many chunk positions as K needs
+// whether the resident kernel can read the mask of this product as bits: the unconditional form, rows of bits that take
+// 16-byte loads and hold a word for every chunk position the kernel walks
+bool resident_takes_bits(const Bf16Args &g)
+{
+    if (g.mask_bits == nullptr || !(g.a_vec && g.K % 8 == 0 && g.K >= 8)) return false;
+    const int64_t words = g.K <= 4 * kRCK ? 4 : 8;
+    return reinterpret_cast<uintptr_t>(g.mask_bits) % 16 == 0 && g.ldw % 4 == 0 && g.ldw >= words;
+}
+
 template <int TN, bool MASKED>
 int launch_nt_resident(const Bf16Args &g, unsigned blocks, hipStream_t st)
 {
-    if (g.a_vec && g.m_vec && g.K % 8 == 0 && g.K >= 8) {
-        if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, MASKED, true, 4>(g, blocks, st);
-        return launch_nt_resident_one<TN, MASKED, true, 8>(g, blocks, st);
+    if constexpr (MASKED) {
+        if (resident_takes_bits(g)) {
+            if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, 2, true, 4>(g, blocks, st);
+            return launch_nt_resident_one<TN, 2, true, 8>(g, blocks, st);
+        }
     }
-    return launch_nt_resident_one<TN, MASKED, false, 8>(g, blocks, st);
+    constexpr int MASK = MASKED ? 1 : 0;
+    if (g.a_vec && g.m_vec && g.K % 8 == 0 && g.K >= 8) {
+        if constexpr (!MASKED) {
+            if (g.relu_bits != nullptr) {
+                if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, 0, true, 4, true>(g, blocks, st);
+                return launch_nt_resident_one<TN, 0, true, 8, true>(g, blocks, st);
+            }
+        }
+        if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, MASK, true, 4>(g, blocks, st);
+        return launch_nt_resident_one<TN, MASK, true, 8>(g, blocks, st);
+    }
+    return launch_nt_resident_one<TN, MASK, false, 8>(g, blocks, st);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -628,9 +722,12 @@ constexpr int kWThreads = 1024;
 constexpr int kWTile = 512 * kS;  // bf16 elements per buffer: 256 columns of A and 256 of B, one LDS row each
 constexpr size_t kWLdsBytes = 2 * (size_t)kWTile * sizeof(uint16_t);
 
-template <bool MASKED>
+// MASK: 0 none, 1 bf16 values beside B, 2 one bit per element (a thread's 8 columns of a row are one byte)
+template <int MASK>
 __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16Args g)
 {
+    constexpr bool MASKED = MASK == 1;
+    constexpr bool BITS = MASK == 2;
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_w[];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -647,12 +744,15 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
     const uint16_t *pa = g.A + (mbeg + 2 * mp) * g.lda + (a_ok ? cq * 8 : 0);
     const uint16_t *pb = g.B + (mbeg + 2 * mp) * g.ldb + (b_ok ? cq * 8 : 0);
     const uint16_t *pm = MASKED ? g.mask + (mbeg + 2 * mp) * g.ldmask + (b_ok ? cq * 8 : 0) : nullptr;
+    const uint8_t *pbit = BITS ? reinterpret_cast<const uint8_t *>(g.mask_bits) + (mbeg + 2 * mp) * g.ldw * 4 + (b_ok ? cq : 0) : nullptr;
 
     uint4 ra[2], rb2[2], rmk[2];
+    uint32_t rbit[2] = {0u, 0u};
     auto advance = [&]() {
         pa += (int64_t)kBK * g.lda;
         pb += (int64_t)kBK * g.ldb;
         if constexpr (MASKED) pm += (int64_t)kBK * g.ldmask;
+        if constexpr (BITS) pbit += (int64_t)kBK * g.ldw * 4;
     };
     auto fetch_whole = [&]() {  // all 64 rows of the chunk exist
 #pragma unroll
@@ -660,6 +760,7 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
             ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
             rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
             if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
+            if constexpr (BITS) rbit[j] = pbit[j * g.ldw * 4];
         }
         advance();
     };
@@ -674,6 +775,7 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
                 ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
                 rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
                 if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
+                if constexpr (BITS) rbit[j] = pbit[j * g.ldw * 4];
             }
         }
         advance();
@@ -696,6 +798,8 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
         if (b_ok) {
             if constexpr (MASKED)
                 stash_pair(bt, mask8(rb2[0], rmk[0]), mask8(rb2[1], rmk[1]));
+            else if constexpr (BITS)
+                stash_pair(bt, mask8_bits(rb2[0], rbit[0]), mask8_bits(rb2[1], rbit[1]));
             else
                 stash_pair(bt, rb2[0], rb2[1]);
         }
@@ -848,6 +952,15 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
                      uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, unsigned flags,
                      float dropout_p, uint64_t seed, uint64_t offset, void *stream)
 {
+    return plx_gemm_nt_bf16_bits(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, nullptr, 0, nullptr, 0, alpha, flags, dropout_p, seed,
+                                 offset, stream);
+}
+
+int plx_gemm_nt_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                          uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw,
+                          uint32_t *relu_bits, int64_t ldw_out, float alpha, unsigned flags, float dropout_p, uint64_t seed,
+                          uint64_t offset, void *stream)
+{
     PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_bf16: negative dimension");
     PLX_REQUIRE(N < (1ll << 30) && K < (1ll << 30), "gemm_nt_bf16: dimension too large");
     PLX_REQUIRE(M < (1ll << 40), "gemm_nt_bf16: too many rows");
@@ -856,6 +969,9 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     PLX_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "gemm_nt_bf16: NULL operand");
     PLX_REQUIRE(lda >= K && ldb >= K && ldc >= N, "gemm_nt_bf16: leading dimension too small");
     PLX_REQUIRE(mask == nullptr || ldmask >= K, "gemm_nt_bf16: mask leading dimension too small");
+    PLX_REQUIRE(mask_bits == nullptr || (mask != nullptr && ldw >= (K + 31) / 32),
+                "gemm_nt_bf16: a bit mask comes with the bf16 mask it stands for and a pitch of at least ceil(K / 32) words");
+    PLX_REQUIRE(relu_bits == nullptr || ldw_out >= (N + 31) / 32, "gemm_nt_bf16: pitch of the sign bits smaller than ceil(N / 32) words");
     PLX_REQUIRE(!(flags & PLX_GEMM_DROPOUT) || (dropout_p >= 0.f && dropout_p < 1.f), "gemm_nt_bf16: dropout p=%g outside [0, 1)",
                 (double)dropout_p);
     Bf16Args g{};
@@ -868,6 +984,7 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     g.seed_lo = (uint32_t)seed; g.seed_hi = (uint32_t)(seed >> 32);
     g.off_lo = (uint32_t)offset; g.off_hi = (uint32_t)(offset >> 32);
     g.a_vec = vec16(A, lda); g.b_vec = vec16(B, ldb); g.c_vec = vec16(C, ldc); g.m_vec = vec16(mask, ldmask);
+    g.mask_bits = mask_bits; g.ldw = ldw; g.relu_bits = relu_bits; g.ldw_out = ldw_out;
     const int tn = pick_tn(N);
     // one workgroup per (row panel, column tile); row panels are rounded up to a multiple of 8 for the XCD mapping
     const int64_t n_ct = plx::ceil_div(N, 32 * tn);
@@ -876,7 +993,11 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     dim3 grid((unsigned)blocks, 1, 1);
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0;
     hipStream_t st = plx::as_stream(stream);
-    if (g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0) {
+    const bool resident = g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0;
+    if (relu_bits != nullptr && !(resident && mask == nullptr && g.a_vec && K % 8 == 0 && K >= 8))  // only one form of the kernel writes them
+        return plx::fail(PLX_ERR_UNSUPPORTED, "gemm_nt_bf16: sign bits are written for N, K <= %d with N and K multiples of 8, 16-byte rows of A "
+                                              "and C, and no mask", kRMax);
+    if (resident) {
         const unsigned rblocks = (unsigned)std::min<int64_t>(plx::ceil_div(M, 32 * kRWaves), 256);
         const int rtn = (int)plx::ceil_div(N, 32);
         int rc = PLX_OK;
@@ -917,12 +1038,21 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
                      float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, void *workspace,
                      size_t workspace_bytes, void *stream)
 {
+    return plx_gemm_tn_bf16_bits(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, nullptr, 0, alpha, workspace, workspace_bytes, stream);
+}
+
+int plx_gemm_tn_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
+                          float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw,
+                          float alpha, void *workspace, size_t workspace_bytes, void *stream)
+{
     PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_tn_bf16: negative dimension");
     if (K == 0 || N == 0) return PLX_OK;
     PLX_REQUIRE(C != nullptr, "gemm_tn_bf16: NULL output");
     PLX_REQUIRE(M == 0 || (A != nullptr && B != nullptr), "gemm_tn_bf16: NULL operand");
     PLX_REQUIRE(lda >= K && ldb >= N && ldc >= N, "gemm_tn_bf16: leading dimension too small");
     PLX_REQUIRE(mask == nullptr || ldmask >= N, "gemm_tn_bf16: mask leading dimension too small");
+    PLX_REQUIRE(mask_bits == nullptr || (mask != nullptr && ldw >= (N + 31) / 32),
+                "gemm_tn_bf16: a bit mask comes with the bf16 mask it stands for and a pitch of at least ceil(N / 32) words");
     hipStream_t st = plx::as_stream(stream);
     const int64_t splits = tn_splits(std::max<int64_t>(M, 1), N, K);
     const size_t need = plx_gemm_tn_bf16_workspace_bytes(M, N, K);
@@ -933,6 +1063,7 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldmask = ldmask;
     g.M = M; g.N = N; g.K = K; g.alpha = alpha;
     g.a_vec = vec16(A, lda); g.b_vec = vec16(B, ldb); g.m_vec = vec16(mask, ldmask);
+    g.mask_bits = mask_bits; g.ldw = ldw;  // read by the whole-tile kernel; the tiled one takes the values
     g.rows_per_split = plx::ceil_div(plx::ceil_div(std::max<int64_t>(M, 1), splits), kBK) * kBK;
     const int64_t used = plx::ceil_div(std::max<int64_t>(M, 1), g.rows_per_split);
     if (splits > 1) {
@@ -945,14 +1076,17 @@ int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0 && N % 8 == 0;
     if (vec && splits > 1 && K <= 256 && N <= 256 && (K > kBM || N > 128)) {
         // more than one 128 x 128 tile, at most 256 x 256: one workgroup per stretch holds the whole tile and reads every operand once
-        static std::atomic<uint64_t> allowed_m{0}, allowed_p{0};
+        static std::atomic<uint64_t> allowed_b{0}, allowed_m{0}, allowed_p{0};
         int rc;
-        if (mask != nullptr) {
-            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<true>), kWLdsBytes, allowed_m);
-            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<true><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+        if (g.mask_bits != nullptr) {  // a row of bits holds at least ceil(N / 32) words: the bytes this kernel reads
+            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<2>), kWLdsBytes, allowed_b);
+            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<2><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+        } else if (mask != nullptr) {
+            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<1>), kWLdsBytes, allowed_m);
+            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<1><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
         } else {
-            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<false>), kWLdsBytes, allowed_p);
-            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<false><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+            rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<0>), kWLdsBytes, allowed_p);
+            if (rc == PLX_OK) gemm_bf16_tn_wide_kernel<0><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
         }
         if (rc != PLX_OK) return rc;
         PLX_LAUNCH_CHECK("gemm_bf16_tn_wide_kernel");

@@ -83,9 +83,15 @@ class GCNConvFunction(torch.autograd.Function):
 
         W = weight.detach().reshape(local_weight_shape)
         timers.start("OUT = AGG * W")
+        BITS = None
         if bf16:
+            # a hidden layer's mask (ReLU and dropout) also as one bit per element where the kernel writes it: the two
+            # backward products then read 1/16 of the mask's bytes
+            want_bits = fuse_relu and ops.bf16_bits_supported(W.shape[1], W.shape[0])
             OUT = ops.gemm_nt_bf16(AGG, ops.cast_bf16(W, transpose=True), relu=fuse_relu, dropout_p=dropout_p,
-                                   seed=dropout_seed, offset=dropout_offset)
+                                   seed=dropout_seed, offset=dropout_offset, want_bits=want_bits)
+            if want_bits:
+                OUT, BITS = OUT
         elif fuse_relu:
             # the mask (ReLU, and dropout where it applies) also as one bit per element, written by the product itself:
             # GRAD_AGG reads it in place of OUT
@@ -95,7 +101,7 @@ class GCNConvFunction(torch.autograd.Function):
         timers.stop("OUT = AGG * W")
 
         # the reference saves AGG, weight and the transposed adjacency (plexus/gcn_conv.py:194)
-        ctx.save_for_backward(AGG, weight, OUT if fuse_relu else None, BITS if fuse_relu and not bf16 else None)
+        ctx.save_for_backward(AGG, weight, OUT if fuse_relu else None, BITS if fuse_relu else None)
         ctx.adj_t = At
         ctx.local_weight_shape = tuple(local_weight_shape)
         ctx.x_shape = x.shape
@@ -204,7 +210,7 @@ class GCNConvFunction(torch.autograd.Function):
         if ctx.needs_input_grad[3]:
             timers.start("GRAD_W = AGG.T * GRAD_OUT")
             if ctx.bf16:
-                grad_weight = ops.gemm_tn_bf16(agg, grad_output, mask=mask, alpha=ctx.grad_scale)
+                grad_weight = ops.gemm_tn_bf16(agg, grad_output, mask=mask, alpha=ctx.grad_scale, mask_bits=bits)
             else:
                 grad_weight = ops.gemm_tn(agg, grad_output, mask=mask, alpha=ctx.grad_scale, mask_bits=bits)
             grad_weight = grad_weight.reshape(weight.shape)
@@ -214,7 +220,7 @@ class GCNConvFunction(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             timers.start("GRAD_AGG = GRAD_OUT * W.T")
             if ctx.bf16:
-                grad_agg = ops.gemm_nt_bf16(grad_output, ops.cast_bf16(W), mask=mask, alpha=ctx.grad_scale)
+                grad_agg = ops.gemm_nt_bf16(grad_output, ops.cast_bf16(W), mask=mask, alpha=ctx.grad_scale, mask_bits=bits)
             else:
                 grad_agg = ops.gemm_nt(grad_output, W, mask=mask, mask_bits=bits, alpha=ctx.grad_scale)
             timers.stop("GRAD_AGG = GRAD_OUT * W.T")

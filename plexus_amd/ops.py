@@ -681,9 +681,19 @@ def cast_bf16(x: torch.Tensor, transpose: bool = False) -> torch.Tensor:
     return y
 
 
+def bf16_bits_supported(n: int, k: int) -> bool:
+    """Whether ``gemm_nt_bf16(want_bits=True)`` can write the sign bits of an M x n result of a k-wide contraction."""
+    return 0 < n <= 256 and 8 <= k <= 256 and n % 8 == 0 and k % 8 == 0
+
+
 def gemm_nt_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0,
-                 relu: bool = False, dropout_p: float = 0.0, seed: int = 0, offset: int = 0) -> torch.Tensor:
-    """bf16 C = epilogue(alpha * (A * [mask > 0]) . B^T), B stored [N x K]; optional ReLU then dropout."""
+                 relu: bool = False, dropout_p: float = 0.0, seed: int = 0, offset: int = 0,
+                 mask_bits: Optional[torch.Tensor] = None, want_bits: bool = False):
+    """bf16 C = epilogue(alpha * (A * [mask > 0]) . B^T), B stored [N x K]; optional ReLU then dropout.
+
+    ``mask_bits``: the same mask as one bit per element (int32 words, as ``want_bits`` returns them), read in its place
+    where the kernel can.  With ``want_bits`` the result is (C, bits): bit c % 32 of word [r, c // 32] says that C[r, c]
+    is positive (``bf16_bits_supported`` tells for which shapes)."""
     _need_gpu(a, b, mask)
     a, b = _rowmajor(a), _rowmajor(b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
@@ -696,19 +706,30 @@ def gemm_nt_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] 
         mask = _rowmajor(mask)
         if mask.shape != a.shape or mask.dtype != torch.bfloat16:
             raise ValueError("gemm_nt_bf16: mask must be bf16 with the shape of A")
+    if mask_bits is not None:
+        _need_gpu(mask_bits)
+        if mask is None or mask_bits.dtype != torch.int32 or mask_bits.dim() != 2 or mask_bits.shape[0] != m \
+                or mask_bits.stride(1) != 1 or mask_bits.shape[1] * 32 < k:
+            raise ValueError("gemm_nt_bf16: mask_bits must be int32 words [M, >= ceil(K / 32)] beside the bf16 mask")
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    bits = _new_bits(m, n, a.device) if want_bits else None
     flags = (PLX_GEMM_RELU if relu else 0) | (PLX_GEMM_DROPOUT if dropout_p > 0.0 else 0)
     check(
-        _lib.load().plx_gemm_nt_bf16(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
-                                     mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
-                                     float(alpha), flags, float(dropout_p), int(seed), int(offset), _stream()),
-        "plx_gemm_nt_bf16",
+        _lib.load().plx_gemm_nt_bf16_bits(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                          mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                                          mask_bits.data_ptr() if mask_bits is not None else None,
+                                          _ld(mask_bits) if mask_bits is not None else 0,
+                                          bits.data_ptr() if bits is not None else None, _ld(bits) if bits is not None else 0,
+                                          float(alpha), flags, float(dropout_p), int(seed), int(offset), _stream()),
+        "plx_gemm_nt_bf16_bits",
     )
-    return c
+    return (c, bits) if want_bits else c
 
 
-def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0) -> torch.Tensor:
-    """fp32 C[K x N] = alpha * A[M x K]^T . (B * [mask > 0])[M x N] from bf16 operands."""
+def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] = None, alpha: float = 1.0,
+                 mask_bits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 C[K x N] = alpha * A[M x K]^T . (B * [mask > 0])[M x N] from bf16 operands; ``mask_bits``: the mask as one
+    bit per element (int32 words [M, >= ceil(N / 32)]), read in its place where the kernel can."""
     _need_gpu(a, b, mask)
     a, b = _rowmajor(a), _rowmajor(b)
     if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
@@ -721,15 +742,22 @@ def gemm_tn_bf16(a: torch.Tensor, b: torch.Tensor, mask: Optional[torch.Tensor] 
         mask = _rowmajor(mask)
         if mask.shape != b.shape or mask.dtype != torch.bfloat16:
             raise ValueError("gemm_tn_bf16: mask must be bf16 with the shape of B")
+    if mask_bits is not None:
+        _need_gpu(mask_bits)
+        if mask is None or mask_bits.dtype != torch.int32 or mask_bits.dim() != 2 or mask_bits.shape[0] != m \
+                or mask_bits.stride(1) != 1 or mask_bits.shape[1] * 32 < n:
+            raise ValueError("gemm_tn_bf16: mask_bits must be int32 words [M, >= ceil(N / 32)] beside the bf16 mask")
     lib = _lib.load()
     c = torch.empty((k, n), dtype=torch.float32, device=a.device)
     need = int(lib.plx_gemm_tn_bf16_workspace_bytes(m, n, k))
     ws = torch.empty(need, dtype=torch.uint8, device=a.device) if need else None
     check(
-        lib.plx_gemm_tn_bf16(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
-                             mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
-                             float(alpha), ws.data_ptr() if ws is not None else None, need, _stream()),
-        "plx_gemm_tn_bf16",
+        lib.plx_gemm_tn_bf16_bits(m, n, k, a.data_ptr(), _ld(a), b.data_ptr(), _ld(b), c.data_ptr(), _ld(c),
+                                  mask.data_ptr() if mask is not None else None, _ld(mask) if mask is not None else 0,
+                                  mask_bits.data_ptr() if mask_bits is not None else None,
+                                  _ld(mask_bits) if mask_bits is not None else 0,
+                                  float(alpha), ws.data_ptr() if ws is not None else None, need, _stream()),
+        "plx_gemm_tn_bf16_bits",
     )
     return c
 

@@ -994,6 +994,53 @@ def test_gemm_tn_bf16(m, n, k):
     assert torch.equal(c, ops.gemm_tn_bf16(a.to(DEV), g.to(DEV)).cpu())  # bit-reproducible
 
 
+@pytest.mark.parametrize("m,n,k,kin", [(40000, 256, 256, 256), (3001, 128, 256, 200), (777, 64, 96, 64), (20011, 256, 136, 248),
+                                         (33, 8, 8, 16)])
+def test_bf16_mask_as_bits(m, n, k, kin):
+    """The forward product writes the sign bits of its bf16 result; the two backward products read the mask in that form
+    and give the same bits as with the bf16 mask.  A mask of all ones in the bits, against the real mask in the values,
+    shows which of the two a kernel read."""
+    say("bf16 sign bits M=%d N=%d K=%d, backward into %d" % (m, n, k, kin))
+    gen = torch.Generator().manual_seed(m + n + k)
+    a = bf(torch.randn(m, k, generator=gen)).to(DEV)
+    wt = bf(torch.randn(n, k, generator=gen) * 0.1).to(DEV)
+    c, bits = ops.gemm_nt_bf16(a, wt, relu=True, want_bits=True)
+    assert torch.equal(c, ops.gemm_nt_bf16(a, wt, relu=True))
+    assert torch.equal(bits.cpu(), _pack_bits(c.float().cpu()))
+    cd, bits_d = ops.gemm_nt_bf16(a, wt, relu=True, dropout_p=0.5, seed=99, offset=3, want_bits=True)
+    assert torch.equal(cd, ops.gemm_nt_bf16(a, wt, relu=True, dropout_p=0.5, seed=99, offset=3))
+    assert torch.equal(bits_d.cpu(), _pack_bits(cd.float().cpu()))
+    assert not torch.equal(bits_d, bits)
+    # GRAD_AGG = (G * mask) . W^T with W stored [kin x n]; GRAD_W = AGG^T . (G * mask)
+    g = bf(torch.randn(m, n, generator=gen)).to(DEV)
+    w = bf(torch.randn(kin, n, generator=gen) * 0.1).to(DEV)
+    agg = bf(torch.randn(m, kin, generator=gen)).to(DEV)
+    ones = torch.full((m, bits.stride(0) if m > 1 else 4), -1, dtype=torch.int32, device=DEV)[:, :bits.shape[1]]  # the pitch of the real ones
+    by_values = ops.gemm_nt_bf16(g, w, mask=cd, alpha=2.0)
+    assert torch.equal(ops.gemm_nt_bf16(g, w, mask=cd, alpha=2.0, mask_bits=bits_d), by_values)
+    read_bits = ops.gemm_nt_bf16(g, w, mask=cd, alpha=2.0, mask_bits=ones)
+    assert torch.equal(read_bits, ops.gemm_nt_bf16(g, w, alpha=2.0))  # N = kin and K = n are at most 256: this kernel reads the bits
+    assert not torch.equal(read_bits, by_values)
+    tn_values = ops.gemm_tn_bf16(agg, g, mask=cd, alpha=0.5)
+    assert torch.equal(ops.gemm_tn_bf16(agg, g, mask=cd, alpha=0.5, mask_bits=bits_d), tn_values)
+    whole_tile = (kin > 128 or n > 128) and m >= 1024  # more than one 128 x 128 tile and more than one stretch of rows
+    tn_ones = ops.gemm_tn_bf16(agg, g, mask=cd, alpha=0.5, mask_bits=ones)
+    assert torch.equal(tn_ones, ops.gemm_tn_bf16(agg, g, alpha=0.5) if whole_tile else tn_values)
+    with pytest.raises(ValueError):
+        ops.gemm_nt_bf16(g, w, mask_bits=bits_d)  # bits come beside the bf16 mask they stand for
+    ref = oracle_c.gemm(agg.float().cpu().numpy(), (g.float() * (cd > 0)).cpu().numpy(), ta=True) * 0.5
+    assert rel_err(tn_values.cpu(), ref) <= FP32_TOL
+
+
+def test_bf16_sign_bits_are_refused_for_shapes_without_them():
+    say("bf16 sign bits beyond 256 columns")
+    a = bf(torch.randn(100, 64)).to(DEV)
+    wt = bf(torch.randn(264, 64)).to(DEV)
+    assert not ops.bf16_bits_supported(264, 64)
+    with pytest.raises(RuntimeError, match="sign bits"):
+        ops.gemm_nt_bf16(a, wt, relu=True, want_bits=True)
+
+
 @pytest.mark.parametrize("m,c", [(10, 7), (1000, 47), (257, 100), (50, 1000), (1031, 41), (333, 64)])
 def test_softmax_xent_bf16(m, c):
     say("softmax_xent bf16 %dx%d" % (m, c))
