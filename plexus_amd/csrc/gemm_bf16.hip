@@ -307,7 +307,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     constexpr bool BITS = MASK == 2;
     static_assert(!BITS || FAST, "the bit mask is read by the unconditional kernel only");
     constexpr int kSteps = KS;             // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = (MASKED || ((WBITS || BITS) && TN > 4)) ? 4 : KS; // register slots = positions ahead that a chunk is requested
+    constexpr int kRing = (MASKED || TN > 4) ? 4 : KS; // register slots = positions ahead that a chunk is requested
     static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;  // [kRMax][kRBS]
