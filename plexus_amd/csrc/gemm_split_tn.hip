@@ -57,16 +57,20 @@ static_assert((kNP == 4 || kNP == 8) && (kNC == 4 || kNC == 8), "four or eight w
 // kNC multiply them (matrix cores, LDS reads), so that the splitting of chunk c + 1 runs beside the products of chunk c.
 // The hardware deals the wavefronts of a workgroup to the four SIMDs of its compute unit in turn (w, w + 4, w + 8, ...
 // share one), so the first kNC wavefronts multiply and the rest split: every SIMD gets its share of both.
-template <int TNW, int MASK>
+// BVEC = false: B is read element by element (rows that are not 16-byte aligned, any N: the 47-wide gradient of a last
+// layer), without a mask; a splitting thread then owns single columns cq, cq + kQ, ... of B's tile instead of groups of four.
+template <int TNW, int MASK, bool BVEC = true>
 __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs g)
 {
+    static_assert(BVEC || MASK == 0, "element loads of B come without a mask");
     constexpr int BN = 32 * TNW;
     constexpr int TNH = kNC == 8 ? TNW / 2 : TNW;               // tiles per multiplying wavefront
     constexpr int kAWords = 3 * kTileK * kSW, kBWords = 3 * BN * kSW;  // words of the planes of one buffer
     constexpr int kBuf = kAWords + kBWords;
     constexpr int kQ = kNP * 4;                                 // 4-column groups covered by one pass of the splitting threads
     constexpr int kAItems = 32 / kQ;                            // (row pair, 4-column group) items of A per splitting thread
-    constexpr int kBItems = (BN / 4 + kQ - 1) / kQ;             // ... of B
+    constexpr int kBItems = BVEC ? (BN / 4 + kQ - 1) / kQ : 1;  // ... of B
+    constexpr int kBCols = BVEC ? 1 : (BN + kQ - 1) / kQ;       // (row pair, column) items of B per splitting thread, element loads
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];  // [2][kBuf]
 
     const int hw_wave = threadIdx.x >> 6;
@@ -94,6 +98,14 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
         const float *pa[kAItems], *pb[kBItems], *pm[MASK == 1 ? kBItems : 1];
         const uint32_t *pw[MASK == 2 ? kBItems : 1];
         int bit0[kBItems];
+        bool bs_ok[kBCols];
+        const float *pbs[kBCols];
+#pragma unroll
+        for (int p = 0; p < kBCols; ++p) {
+            const int c = cq + kQ * p;
+            bs_ok[p] = !BVEC && c < BN && col0 + c < g.N;
+            pbs[p] = g.B + (mbeg + 2 * mp) * g.ldb + (bs_ok[p] ? col0 + c : col0);
+        }
 #pragma unroll
         for (int p = 0; p < kAItems; ++p) {
             const int64_t col = row0 + 4 * (cq + kQ * p);
@@ -103,7 +115,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
 #pragma unroll
         for (int p = 0; p < kBItems; ++p) {
             const int64_t col = col0 + 4 * (cq + kQ * p);
-            b_ok[p] = 4 * (cq + kQ * p) < BN && col < g.N;
+            b_ok[p] = BVEC && 4 * (cq + kQ * p) < BN && col < g.N;
             const int64_t c = b_ok[p] ? col : col0;
             pb[p] = g.B + (mbeg + 2 * mp) * g.ldb + c;
             if constexpr (MASK == 1) pm[p] = g.mask + (mbeg + 2 * mp) * g.ldmask + c;
@@ -114,6 +126,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
         struct Regs {
             float4 a[kAItems][2], b[kBItems][2], m[MASK == 1 ? kBItems : 1][2];
             uint32_t w[MASK == 2 ? kBItems : 1][2];
+            float bs[kBCols][2];
         };
         int64_t m_next = mbeg;  // first row of the chunk the next fetch brings
         auto advance = [&]() {
@@ -125,6 +138,10 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
                 if constexpr (MASK == 1) pm[p] += (int64_t)kRows * g.ldmask;
                 if constexpr (MASK == 2) pw[p] += (int64_t)kRows * g.ldw;
             }
+            if constexpr (!BVEC) {
+#pragma unroll
+                for (int p = 0; p < kBCols; ++p) pbs[p] += (int64_t)kRows * g.ldb;
+            }
             m_next += kRows;
         };
         // a chunk whose 32 rows all exist: loads and nothing else (no branch, so that the waits the compiler places before
@@ -134,11 +151,16 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
             for (int j = 0; j < 2; ++j) {
 #pragma unroll
                 for (int p = 0; p < kAItems; ++p) r.a[p][j] = *reinterpret_cast<const float4 *>(pa[p] + j * g.lda);
+                if constexpr (BVEC) {
 #pragma unroll
-                for (int p = 0; p < kBItems; ++p) {
-                    r.b[p][j] = *reinterpret_cast<const float4 *>(pb[p] + j * g.ldb);
-                    if constexpr (MASK == 1) r.m[p][j] = *reinterpret_cast<const float4 *>(pm[p] + j * g.ldmask);
-                    if constexpr (MASK == 2) r.w[p][j] = pw[p][j * g.ldw];
+                    for (int p = 0; p < kBItems; ++p) {
+                        r.b[p][j] = *reinterpret_cast<const float4 *>(pb[p] + j * g.ldb);
+                        if constexpr (MASK == 1) r.m[p][j] = *reinterpret_cast<const float4 *>(pm[p] + j * g.ldmask);
+                        if constexpr (MASK == 2) r.w[p][j] = pw[p][j * g.ldw];
+                    }
+                } else {
+#pragma unroll
+                    for (int p = 0; p < kBCols; ++p) r.bs[p][j] = pbs[p][j * g.ldb];
                 }
             }
             advance();
@@ -152,11 +174,16 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
                 const bool row_ok = j < rows_left;
 #pragma unroll
                 for (int p = 0; p < kAItems; ++p) r.a[p][j] = row_ok ? *reinterpret_cast<const float4 *>(pa[p] + j * g.lda) : zero;
+                if constexpr (BVEC) {
 #pragma unroll
-                for (int p = 0; p < kBItems; ++p) {
-                    r.b[p][j] = row_ok ? *reinterpret_cast<const float4 *>(pb[p] + j * g.ldb) : zero;
-                    if constexpr (MASK == 1) r.m[p][j] = row_ok ? *reinterpret_cast<const float4 *>(pm[p] + j * g.ldmask) : zero;
-                    if constexpr (MASK == 2) r.w[p][j] = row_ok ? pw[p][j * g.ldw] : 0u;
+                    for (int p = 0; p < kBItems; ++p) {
+                        r.b[p][j] = row_ok ? *reinterpret_cast<const float4 *>(pb[p] + j * g.ldb) : zero;
+                        if constexpr (MASK == 1) r.m[p][j] = row_ok ? *reinterpret_cast<const float4 *>(pm[p] + j * g.ldmask) : zero;
+                        if constexpr (MASK == 2) r.w[p][j] = row_ok ? pw[p][j * g.ldw] : 0u;
+                    }
+                } else {
+#pragma unroll
+                    for (int p = 0; p < kBCols; ++p) r.bs[p][j] = row_ok ? pbs[p][j * g.ldb] : 0.f;
                 }
             }
             advance();
@@ -188,8 +215,22 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
                 care |= needs_care(r.a[p][0]) | needs_care(r.a[p][1]);
                 stash_quad(a_ok[p] ? base + a_dst[p] : lds + a_dst[p], a_ok[p] ? kTileK * kSW : 0, r.a[p][0], r.a[p][1]);
             }
+            if constexpr (!BVEC) {
+#pragma unroll
+                for (int p = 0; p < kBCols; ++p) {
+                    care |= needs_care(r.bs[p][0]) | needs_care(r.bs[p][1]);
+                    uint32_t p0, p1, p2;
+                    split2(r.bs[p][0], r.bs[p][1], p0, p1, p2);
+                    uint32_t *dst = bs_ok[p] ? base + kAWords + (cq + kQ * p) * kSW + mp : lds + 2 * kBuf + mp;
+                    const int plane_words = bs_ok[p] ? BN * kSW : 0;
+                    dst[0] = p0;
+                    dst[plane_words] = p1;
+                    dst[2 * plane_words] = p2;
+                }
+            }
 #pragma unroll
             for (int p = 0; p < kBItems; ++p) {
+                if constexpr (!BVEC) continue;
                 if (4 * (cq + kQ * p) >= BN && kBItems * kQ * 4 > BN) continue;  // a pass that reaches past the tile (compile-time shape)
                 float4 b0 = r.b[p][0], b1 = r.b[p][1];
                 if constexpr (MASK == 1) {
@@ -317,16 +358,16 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
     }
 }
 
-template <int TNW, int MASK>
+template <int TNW, int MASK, bool BVEC = true>
 int launch_one(const TnArgs &g, dim3 grid, hipStream_t st)
 {
     // two buffers of planes and the corner that takes the pieces of column groups outside the matrices
     constexpr size_t shm = ((size_t)2 * 3 * (kTileK + 32 * TNW) * kSW + 4 * kSW) * sizeof(uint32_t);
     static_assert(shm <= 160 * 1024, "two buffers of planes fit the LDS of a compute unit");
     static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_tn_kernel<TNW, MASK>), shm, allowed);
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_tn_kernel<TNW, MASK, BVEC>), shm, allowed);
     if (rc != PLX_OK) return rc;
-    gemm_split_tn_kernel<TNW, MASK><<<grid, kThreads, shm, st>>>(g);
+    gemm_split_tn_kernel<TNW, MASK, BVEC><<<grid, kThreads, shm, st>>>(g);
     PLX_LAUNCH_CHECK("gemm_split_tn_kernel");
     return PLX_OK;
 }
@@ -407,12 +448,17 @@ int plx_gemm_tn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64
     g.nonfinite = flag;
     // the split kernel reads with 128-bit loads; operands that do not allow them go to the fp32 MFMA kernel as they are
     const bool bits = mask_bits != nullptr && reinterpret_cast<uintptr_t>(mask_bits) % 4 == 0;
-    const bool vec = M > 0 && aligned16(A, lda) && aligned16(B, ldb) && (bits || aligned16(mask, ldmask)) && K % 4 == 0 && N % 4 == 0;
-    if (!vec) return plx::gemm_tn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, workspace, need - kFlagBytes, nullptr, alpha, stream);
+    const bool a_vec = M > 0 && aligned16(A, lda) && K % 4 == 0;
+    const bool vec = a_vec && aligned16(B, ldb) && (bits || aligned16(mask, ldmask)) && N % 4 == 0;
+    // B in rows that do not take 128-bit loads (the 47-wide gradient of a last layer): read element by element, when it is at most
+    // 64 columns wide and comes without a mask
+    const bool b_scalar = !vec && a_vec && mask == nullptr && N <= 64;
+    if (!vec && !b_scalar)
+        return plx::gemm_tn_f32_if(M, N, K, A, lda, B, ldb, C, ldc, mask, ldmask, workspace, need - kFlagBytes, nullptr, alpha, stream);
     const int mode = mask == nullptr ? 0 : (bits ? 2 : 1);
     const int bn = tile_cols(N);
     dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kTileK), (unsigned)plx::ceil_div(N, bn));
-    int rc = bn == 64 ? launch_mask<2>(g, mode, grid, st) : launch_mask<4>(g, mode, grid, st);
+    int rc = b_scalar ? launch_one<2, 0, false>(g, grid, st) : (bn == 64 ? launch_mask<2>(g, mode, grid, st) : launch_mask<4>(g, mode, grid, st));
     if (rc != PLX_OK) return rc;
     rc = plx::gemm_tn_reduce_tiles(g.ws, g.ws_ld, g.ws_slab, (int)used, K, N, C, ldc, alpha, stream);
     if (rc != PLX_OK) return rc;

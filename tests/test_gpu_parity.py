@@ -479,8 +479,9 @@ def test_sign_bits_follow_the_product_the_guarded_launch_redoes():
     assert torch.equal(bits.cpu(), _pack_bits(out.cpu()))
 
 
+# (40000, 47, 128), (50001, 33, 100), (3000, 7, 64): B in rows without 16-byte alignment, read element by element by the split kernel
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(70000, 128, 100), (40000, 47, 128), (30011, 128, 128), (5000, 200, 150), (2500, 64, 300),
-                                                   (31, 128, 128), (1, 5, 3)])
+                                                   (31, 128, 128), (1, 5, 3), (50001, 33, 100), (3000, 7, 64)])
 def test_gemm_tn_and_mask(m, n, k, fp32_gemm_path):
     say("gemm_tn %dx%dx%d %s" % (m, n, k, fp32_gemm_path))
     gen = torch.Generator().manual_seed(m * 5 + n + k)
