@@ -722,12 +722,15 @@ constexpr int kWThreads = 1024;
 constexpr int kWTile = 512 * kS;  // bf16 elements per buffer: 256 columns of A and 256 of B, one LDS row each
 constexpr size_t kWLdsBytes = 2 * (size_t)kWTile * sizeof(uint16_t);
 
-// MASK: 0 none, 1 bf16 values beside B, 2 one bit per element (a thread's 8 columns of a row are one byte)
+// MASK: 0 none, 1 bf16 values beside B, 2 one bit per element (a thread's 8 columns of a row are one byte), 3 none and B of at
+// most 64 columns in rows that take no 16-byte loads (the 47-wide gradient of a last layer), read element by element: a thread
+// then owns columns cq and cq + 32 of B
 template <int MASK>
 __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16Args g)
 {
     constexpr bool MASKED = MASK == 1;
     constexpr bool BITS = MASK == 2;
+    constexpr bool BSC = MASK == 3;
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_w[];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -740,7 +743,10 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
     // thread (mp, cq): row pair (2 mp, 2 mp + 1) of a chunk, columns 8 cq .. 8 cq + 7 of A and of B
     const int mp = threadIdx.x & 31;
     const int cq = threadIdx.x >> 5;
-    const bool a_ok = cq * 8 < g.K, b_ok = cq * 8 < g.N;
+    const bool a_ok = cq * 8 < g.K, b_ok = !BSC && cq * 8 < g.N;
+    const bool bs_ok[2] = {BSC && cq < g.N, BSC && cq + 32 < g.N};
+    const uint16_t *pbs = g.B + (mbeg + 2 * mp) * g.ldb;
+    uint32_t rbs[2][2] = {{0u, 0u}, {0u, 0u}};
     const uint16_t *pa = g.A + (mbeg + 2 * mp) * g.lda + (a_ok ? cq * 8 : 0);
     const uint16_t *pb = g.B + (mbeg + 2 * mp) * g.ldb + (b_ok ? cq * 8 : 0);
     const uint16_t *pm = MASKED ? g.mask + (mbeg + 2 * mp) * g.ldmask + (b_ok ? cq * 8 : 0) : nullptr;
@@ -753,14 +759,19 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
         pb += (int64_t)kBK * g.ldb;
         if constexpr (MASKED) pm += (int64_t)kBK * g.ldmask;
         if constexpr (BITS) pbit += (int64_t)kBK * g.ldw * 4;
+        if constexpr (BSC) pbs += (int64_t)kBK * g.ldb;
     };
     auto fetch_whole = [&]() {  // all 64 rows of the chunk exist
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
-            rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
+            if constexpr (!BSC) rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
             if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
             if constexpr (BITS) rbit[j] = pbit[j * g.ldw * 4];
+            if constexpr (BSC) {
+#pragma unroll
+                for (int p = 0; p < 2; ++p) rbs[p][j] = pbs[j * g.ldb + (bs_ok[p] ? cq + 32 * p : 0)];
+            }
         }
         advance();
     };
@@ -773,9 +784,13 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
             rmk[j] = zero4();
             if (j < rows_left) {
                 ra[j] = *reinterpret_cast<const uint4 *>(pa + j * g.lda);
-                rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
+                if constexpr (!BSC) rb2[j] = *reinterpret_cast<const uint4 *>(pb + j * g.ldb);
                 if constexpr (MASKED) rmk[j] = *reinterpret_cast<const uint4 *>(pm + j * g.ldmask);
                 if constexpr (BITS) rbit[j] = pbit[j * g.ldw * 4];
+            }
+            if constexpr (BSC) {
+#pragma unroll
+                for (int p = 0; p < 2; ++p) rbs[p][j] = j < rows_left ? (uint32_t)pbs[j * g.ldb + (bs_ok[p] ? cq + 32 * p : 0)] : 0u;
             }
         }
         advance();
@@ -795,6 +810,11 @@ __global__ void __launch_bounds__(kWThreads) gemm_bf16_tn_wide_kernel(const Bf16
         uint16_t *at = lds_w + buf * kWTile;
         uint16_t *bt = at + 256 * kS;
         if (a_ok) stash_pair(at, ra[0], ra[1]);
+        if constexpr (BSC) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+                if (bs_ok[p]) *reinterpret_cast<uint32_t *>(bt + (cq + 32 * p) * kS + 2 * mp) = rbs[p][0] | (rbs[p][1] << 16);
+        }
         if (b_ok) {
             if constexpr (MASKED)
                 stash_pair(bt, mask8(rb2[0], rmk[0]), mask8(rb2[1], rmk[1]));
@@ -1074,7 +1094,15 @@ int plx_gemm_tn_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, in
     const int tn = pick_tn(N);
     dim3 grid((unsigned)used, (unsigned)plx::ceil_div(K, kBM), (unsigned)plx::ceil_div(N, 32 * tn));
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0 && N % 8 == 0;
-    if (vec && splits > 1 && K <= 256 && N <= 256 && (K > kBM || N > 128)) {
+    const bool b_scalar = !vec && splits > 1 && g.a_vec && K % 8 == 0 && K <= 256 && N <= 64 && mask == nullptr;
+    if (b_scalar) {
+        // a narrow B in rows without 16-byte alignment: the whole-tile kernel reads it element by element
+        static std::atomic<uint64_t> allowed_s{0};
+        const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_bf16_tn_wide_kernel<3>), kWLdsBytes, allowed_s);
+        if (rc != PLX_OK) return rc;
+        gemm_bf16_tn_wide_kernel<3><<<(unsigned)used, kWThreads, kWLdsBytes, st>>>(g);
+        PLX_LAUNCH_CHECK("gemm_bf16_tn_wide_kernel");
+    } else if (vec && splits > 1 && K <= 256 && N <= 256 && (K > kBM || N > 128)) {
         // more than one 128 x 128 tile, at most 256 x 256: one workgroup per stretch holds the whole tile and reads every operand once
         static std::atomic<uint64_t> allowed_b{0}, allowed_m{0}, allowed_p{0};
         int rc;
