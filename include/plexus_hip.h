@@ -343,8 +343,10 @@ int plx_gemm_tn_f32(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda
  * `mask_bits` (may be NULL; ldw >= ceil(N / 32)) is the mask of B as one bit per element, as plx_gemm_nn_f32_split_bits
  * writes it; the fp32 `mask`, which must say the same, is read where no bits are given and by the fp32 MFMA launch
  * that redoes the product when an operand holds Inf, NaN or a value next to FLT_MAX (always enqueued, returns at once
- * otherwise).  Any alignment (128-bit loads when A, B and mask are 16-byte aligned with leading dimensions, K and N
- * multiples of 4).  Same reference call site as plx_gemm_tn_f32: plexus/gcn_conv.py:237-239. */
+ * otherwise).  Any alignment: the split kernel takes operands that are 16-byte aligned with leading dimensions, K and N
+ * multiples of 4, and also an unmasked B of at most 64 columns in rows of any alignment beside such an A (the 47-wide gradient
+ * of a last layer, read element by element); every other shape goes to the fp32 MFMA kernel of plx_gemm_tn_f32.  Same
+ * reference call site: plexus/gcn_conv.py:237-239. */
 size_t plx_gemm_tn_f32_split_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int plx_gemm_tn_f32_split(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
                           const float *mask, int64_t ldmask, const uint32_t *mask_bits, int64_t ldw, float alpha, void *workspace,
@@ -365,7 +367,9 @@ int plx_gemm_nt_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t
                      uint16_t *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, unsigned flags,
                      float dropout_p, uint64_t seed, uint64_t offset, void *stream);
 
-/* C[K x N] (fp32) = alpha * A[M x K]^T . (B ⊙ [mask > 0])[M x N]      GRAD_W = AGG^T . GRAD_OUT */
+/* C[K x N] (fp32) = alpha * A[M x K]^T . (B ⊙ [mask > 0])[M x N]      GRAD_W = AGG^T . GRAD_OUT
+ * For K and N up to 256 with more than one 128 x 128 tile, and for an unmasked B of at most 64 columns in rows that take no
+ * 16-byte loads, one workgroup per stretch of rows holds the whole tile of C and every operand is read once. */
 size_t plx_gemm_tn_bf16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int plx_gemm_tn_bf16(int64_t M, int64_t N, int64_t K, const uint16_t *A, int64_t lda, const uint16_t *B, int64_t ldb,
                      float *C, int64_t ldc, const uint16_t *mask, int64_t ldmask, float alpha, void *workspace,
