@@ -325,13 +325,13 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     constexpr bool MASKED = MASK == 1;      // the fp32 mask travels in registers beside its chunk
     constexpr bool BITS = MASK == 2;        // the bit mask of a panel row is four words, loaded once per panel
     constexpr int kSteps = KS;              // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = MASKED ? 4 : KS;  // register slots = how many positions ahead a chunk is requested
+    constexpr int kRing = (MASKED || FAST) ? 4 : KS;  // register slots = how many positions ahead a chunk is requested
     static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;                               // [3][kRMaxN][kRBS]
     constexpr int kBPlane = kRMaxN * kRBS;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: panel arithmetic stays scalar
     const int li = lane & 31;
     const int h = lane >> 5;
     uint16_t *const apriv = rlds + 3 * kBPlane + wave * 3 * kRAPlane;  // [3][32][kRAS], this wavefront's
@@ -368,23 +368,46 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     float4 ring[kRing][2], mring[MASKED ? kRing : 1][2];
     // Bit mask: a 64-lane load takes the memory pipeline as long for 4 bytes per lane as for 16, so the bits are not
     // fetched chunk by chunk; the 128 bits of rows r and r + 16 of a panel come with its first chunk and stay in registers.
-    static_assert(!BITS || kRing == kSteps, "the chunks in flight are those of exactly one panel ahead");
+    static_assert(!BITS || FAST || kRing == kSteps, "the guarded kernel makes the bits that came with a panel's first chunk current at the panel's start");
     u32x4 pb_cur[2], pb_next[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p] = u32x4{~0u, ~0u, ~0u, ~0u};
+    // byte offsets of a lane's two rows inside a panel (in the last panel: rows clamped to the last row of the matrix) and of
+    // the last four columns, to which a lane's four columns are clamped; the host keeps 128 leading dimensions below 2^32
+    // bytes for this kernel
+    uint32_t a_off[2], a_off_last[2], m_off[2], m_off_last[2], w_off[2], w_off_last[2];
+    const uint32_t k_last = 4u * (uint32_t)(K - 4);
+    if constexpr (FAST) {
+        const int rows_last = (int)(g.M - (n_panels - 1) * 32);  // 1 ... 32
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const uint32_t row = r + 16 * p, row_last = min(r + 16 * p, rows_last - 1);
+            a_off[p] = row * (uint32_t)g.lda * 4u;
+            a_off_last[p] = row_last * (uint32_t)g.lda * 4u;
+            m_off[p] = MASKED ? row * (uint32_t)g.ldmask * 4u : 0u;
+            m_off_last[p] = MASKED ? row_last * (uint32_t)g.ldmask * 4u : 0u;
+            w_off[p] = BITS ? row * (uint32_t)g.ldw * 4u : 0u;
+            w_off_last[p] = BITS ? row_last * (uint32_t)g.ldw * 4u : 0u;
+        }
+    }
     // `pos`, `of_panel`: the position a request is for (the unconditional form takes them from its caller, where they are
     // compile-time and loop-invariant values; the guarded form follows its cursor)
     auto fetch = [&](float4(&dst)[2], float4(&mdst)[2], int pos, int64_t of_panel) __attribute__((always_inline)) {
         if constexpr (FAST) {
+            // the panel's address is the same in every lane (scalar arithmetic); a lane adds a 32-bit byte offset that does
+            // not depend on the panel, except that the rows of the last panel are clamped into the matrix
             const int64_t panel = min(of_panel, n_panels - 1);
-            const int k = min(pos * kRCK + kq * 4, K - 4);
+            const bool last = panel == n_panels - 1;
+            const char *const pa = reinterpret_cast<const char *>(g.A) + panel * 128 * g.lda;
+            const char *const pm = MASKED ? reinterpret_cast<const char *>(g.mask) + panel * 128 * g.ldmask : nullptr;
+            const char *const pw = BITS ? reinterpret_cast<const char *>(g.mask_bits) + panel * 128 * g.ldw : nullptr;
+            const uint32_t k_off = min((uint32_t)(pos * kRCK * 4 + kq * 16), k_last);
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                const int64_t row = min(panel * 32 + r + 16 * p, g.M - 1);
-                dst[p] = *reinterpret_cast<const float4 *>(g.A + row * g.lda + k);
-                if constexpr (MASKED) mdst[p] = *reinterpret_cast<const float4 *>(g.mask + row * g.ldmask + k);
+                dst[p] = *reinterpret_cast<const float4 *>(pa + ((last ? a_off_last[p] : a_off[p]) + k_off));
+                if constexpr (MASKED) mdst[p] = *reinterpret_cast<const float4 *>(pm + ((last ? m_off_last[p] : m_off[p]) + k_off));
                 if constexpr (BITS) {
-                    if (pos == 0) pb_next[p] = *reinterpret_cast<const u32x4 *>(g.mask_bits + row * g.ldw);
+                    if (pos == 0) pb_next[p] = *reinterpret_cast<const u32x4 *>(pw + (last ? w_off_last[p] : w_off[p]));
                 }
             }
             return;
@@ -493,16 +516,8 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
         }
     };
 
-#pragma unroll
-    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
-    for (int64_t panel = first; panel < n_panels; panel += stride) {
-        cur_panel = panel;
-        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
-#pragma unroll
-            for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
-        }
-#pragma unroll
-        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+    // a finished panel: ReLU, dropout, sign bits, stores; leaves the accumulators zero
+    auto finish_panel = [&](int64_t panel) __attribute__((always_inline)) {
         // the panel is complete: register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
         const int64_t r0 = panel * 32 + 4 * h;
         float *pc = g.C + r0 * g.ldc + li;
@@ -567,7 +582,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                     }
                     plx::wave_lds_fence();  // the next tile, or the next panel's first chunk, overwrites the staging
                 }
-                continue;
+                return;
             }
         }
 #pragma unroll
@@ -599,6 +614,162 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             }
         }
         if constexpr (DROP) plx::wave_lds_fence();  // the next panel's first chunk overwrites the keep bits
+    };
+
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
+
+    if constexpr (FAST) {
+        // The positions run as a pipeline inside the wavefront.  While the matrix cores multiply position i out of registers,
+        // the vector ALU splits position i + 1, the pieces go to the private tile (free once the pieces of position i have
+        // been read), come back as the operands of position i + 1, and the pieces of B are read one column tile ahead of
+        // their products.  A wavefront issues in order, so what shall overlap has to alternate in the instruction stream:
+        // every product is followed by at most one half split (six or seven vector instructions, less than the 28 cycles a
+        // product leaves free), and the order written here is pinned -- an empty asm statement after each product and each
+        // half split takes their results as operands, and a scheduling barrier follows.
+        constexpr int kStoreAt = TN >= 4 ? 18 : (TN == 2 ? 8 : 4);  // the product before which the next position is stored
+        static_assert((kSteps * TN) % 2 == 0, "operand buffers alternate with the parity of a compile-time count");
+        constexpr bool kAheadB = !(MASKED && TN > 1);
+        bool unsplittable = false;  // a value the split cannot carry was met
+        bf16x8 aa[2][3], bb[2][3];
+        auto load_a = [&](bf16x8(&a)[3]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 3; ++q) a[q] = *reinterpret_cast<const bf16x8 *>(a_src + q * kRAPlane);
+        };
+        auto load_b = [&](bf16x8(&b)[3], int kc, int t) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 3; ++q) b[q] = *reinterpret_cast<const bf16x8 *>(b_src + kc * kRCK + t * 32 * kRBS + q * kBPlane);
+        };
+        auto masked = [&](const float4 &a, const float4 &m, const u32x4 &bits, int kc) __attribute__((always_inline)) -> float4 {
+            float4 v = a;
+            if constexpr (MASKED) v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
+            if constexpr (BITS) {
+                // chunk kc holds contraction elements 16 kc ...: bits 16 (kc % 2) + 4 kq ... of word kc / 2
+                const uint32_t mb = bits[kc >> 1] >> (16 * (kc & 1) + 4 * kq);
+                v = make_float4((mb & 1u) ? v.x : 0.f, (mb & 2u) ? v.y : 0.f, (mb & 4u) ? v.z : 0.f, (mb & 8u) ? v.w : 0.f);
+            }
+            return v;
+        };
+        auto store_pieces = [&](const uint32_t(&w)[2][6]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                uint16_t *dst = a_dst + 16 * p * kRAS;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(w[p][0], w[p][3]);
+                *reinterpret_cast<uint2 *>(dst + kRAPlane) = make_uint2(w[p][1], w[p][4]);
+                *reinterpret_cast<uint2 *>(dst + 2 * kRAPlane) = make_uint2(w[p][2], w[p][5]);
+            }
+        };
+
+        // position 0 of the first panel, with nothing to multiply meanwhile
+        {
+            if constexpr (BITS) {
+#pragma unroll
+                for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
+            }
+            uint32_t w[2][6];
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const float4 v = masked(ring[0][p], mring[0][p], pb_cur[p], 0);
+                float rx, ry;
+                split2_first(v.x, v.y, w[p][0], rx, ry);
+                unsplittable |= split2_second(rx, ry, w[p][1], w[p][2]);
+                split2_first(v.z, v.w, w[p][3], rx, ry);
+                unsplittable |= split2_second(rx, ry, w[p][4], w[p][5]);
+            }
+            store_pieces(w);
+            plx::wave_lds_fence();
+            load_a(aa[0]);
+            if constexpr (kAheadB) load_b(bb[0], 0, 0);
+            plx::wave_lds_fence();
+        }
+
+        for (int64_t panel = first; panel < n_panels; panel += stride) {
+#pragma unroll
+            for (int kc = 0; kc < kSteps; ++kc) {
+                const bool wrap = kc + 1 == kSteps;  // the next position is the first of this wavefront's next panel
+                const int nc = wrap ? 0 : kc + 1, slot = (kc + 1) % kRing;
+                float4(&nxt)[2] = ring[slot];
+                float4(&mnxt)[2] = mring[MASKED ? slot : 0];
+                // the next position: eight values of a lane, four half-split pairs (j = 2 p + half of the float4)
+                float x[4], y[4], rx[4], ry[4];
+                uint32_t w[2][6];
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const float4 v = masked(nxt[p], mnxt[p], wrap ? pb_next[p] : pb_cur[p], nc);
+                    x[2 * p] = v.x, y[2 * p] = v.y, x[2 * p + 1] = v.z, y[2 * p + 1] = v.w;
+                }
+                if constexpr (BITS) {
+                    if (wrap) {  // before the request below replaces them with the bits of the panel after
+#pragma unroll
+                        for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+                    const int group = kc * TN + t;  // which of the two buffers of B holds this column tile's pieces
+                    // the pieces of B one column tile ahead (the first tile of the next position after the last); the kernel
+                    // that also carries fp32 mask values has no registers for that and reads them where they are used
+                    if constexpr (kAheadB) {
+                        if (t + 1 < TN) load_b(bb[(group + 1) & 1], kc, t + 1);
+                        else load_b(bb[(group + 1) & 1], nc, 0);
+                    } else {
+                        load_b(bb[group & 1], kc, t);
+                    }
+#pragma unroll
+                    for (int m = 0; m < 6; ++m) {
+                        const int idx = 6 * t + m;
+                        if (idx == kStoreAt) {  // every half split lies before this product
+                            plx::wave_lds_fence();  // after the loads of this position's pieces (and a finished panel's staging)
+                            store_pieces(w);
+                            // requests go out for two positions at a time, which share their 128-byte lines: positions
+                            // kc + 4 and kc + 5 into the slots of positions kc and kc + 1, both split by now
+                            if ((kc & 1) == 0) {
+                                fetch(ring[kc % kRing], mring[MASKED ? kc % kRing : 0], (kc + kRing) % kSteps, panel + ((kc + kRing) / kSteps) * stride);
+                                fetch(nxt, mnxt, (kc + 1 + kRing) % kSteps, panel + ((kc + 1 + kRing) / kSteps) * stride);
+                            }
+                            plx::wave_lds_fence();
+                            load_a(aa[(kc + 1) & 1]);
+                            plx::wave_lds_fence();
+                        }
+                        // the six piece products in the order of mfma6 (the smallest terms first)
+                        const bf16x8(&a)[3] = aa[kc & 1];
+                        const bf16x8(&b)[3] = bb[group & 1];
+                        const bf16x8 am = (m == 0) ? a[2] : (m == 2 || m == 3) ? a[1] : a[0];
+                        const bf16x8 bm = (m == 0 || m == 3 || m == 5) ? b[0] : (m == 1) ? b[2] : b[1];
+                        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bm, acc[t], 0, 0, 0);
+                        asm volatile("" : "+v"(acc[t]));
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {  // half split k = 2 j + second half, after product k kStoreAt / 8
+                            if (k * kStoreAt / 8 != idx) continue;
+                            const int j = k >> 1, p = j >> 1, o = 3 * (j & 1);
+                            if ((k & 1) == 0) {
+                                split2_first(x[j], y[j], w[p][o], rx[j], ry[j]);
+                                asm volatile("" : "+v"(w[p][o]), "+v"(rx[j]), "+v"(ry[j]));
+                            } else {
+                                unsplittable |= split2_second(rx[j], ry[j], w[p][o + 1], w[p][o + 2]);
+                                asm volatile("" : "+v"(w[p][o + 1]), "+v"(w[p][o + 2]));
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if (__builtin_expect(unsplittable, 0)) *g.nonfinite = 1u;
+            plx::wave_lds_fence();  // the staging of the panel comes after the loads of the next position's pieces
+            finish_panel(panel);
+        }
+        return;
+    }
+
+    for (int64_t panel = first; panel < n_panels; panel += stride) {
+        cur_panel = panel;
+        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
+#pragma unroll
+            for (int p = 0; p < 2; ++p) pb_cur[p] = pb_next[p];
+        }
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+        finish_panel(panel);
     }
 }
 
@@ -617,7 +788,9 @@ int launch_resident_one(const SplitArgs &g, unsigned blocks, hipStream_t st)
 template <int TN, int MASK, bool DROP = false>
 int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
 {
-    if (g.a_vec && g.K >= 4) {
+    // (its lanes address a panel with 32-bit byte offsets)
+    const int64_t ld_max = (int64_t)1 << 24;
+    if (g.a_vec && g.K >= 4 && g.lda < ld_max && g.ldmask < ld_max && g.ldw < ld_max) {
         if (g.K <= 64) return launch_resident_one<TN, MASK, DROP, true, 4>(g, blocks, st);
         return launch_resident_one<TN, MASK, DROP, true, 8>(g, blocks, st);
     }

@@ -26,6 +26,24 @@ __device__ __forceinline__ void split2(float x, float y, uint32_t &p0, uint32_t 
     p2 = plx::pack_bf16x2(sx, sy);
 }
 
+// The same split in two halves, for kernels that place them between other instructions: the first half gives the first
+// piece and what it leaves, the second the other two pieces.  `second` returns true if x or y was a value the split cannot
+// carry (see needs_care): the first piece of such a value is Inf or NaN, which leaves NaN as the last residual, and no
+// other value does -- one compare for the two values.
+__device__ __forceinline__ void split2_first(float x, float y, uint32_t &p0, float &rx, float &ry)
+{
+    p0 = plx::pack_bf16x2(x, y);
+    rx = x - __uint_as_float(p0 << 16);
+    ry = y - __uint_as_float(p0 & 0xffff0000u);
+}
+__device__ __forceinline__ bool split2_second(float rx, float ry, uint32_t &p1, uint32_t &p2)
+{
+    p1 = plx::pack_bf16x2(rx, ry);
+    const float sx = rx - __uint_as_float(p1 << 16), sy = ry - __uint_as_float(p1 & 0xffff0000u);
+    p2 = plx::pack_bf16x2(sx, sy);
+    return __builtin_isunordered(sx, sy);
+}
+
 // Values the split cannot carry: Inf and NaN (Inf times a zero piece is NaN, where the fp32 product gives Inf), and finite
 // values of 0x7f7f8000 (3.3895e38) or more in magnitude, whose rounding to bf16 overflows.  One compare per element
 // (NaN fails the "less than").  A kernel that meets one raises the flag word of its call, and the whole product is then
