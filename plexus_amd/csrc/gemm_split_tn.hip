@@ -196,31 +196,31 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
 #pragma unroll
         for (int p = 0; p < kBItems; ++p) b_dst[p] = b_ok[p] ? kAWords + (4 * (cq + kQ * p)) * kSW + mp : 2 * kBuf + mp;
         // the pieces of (row 2 mp, row 2 mp + 1) of one column are one word per plane
-        auto stash_quad = [&](uint32_t *dst, int plane_words, const float4 &r0, const float4 &r1) {
+        // (returns true if one of the eight values is one the split cannot carry)
+        auto stash_quad = [&](uint32_t *dst, int plane_words, const float4 &r0, const float4 &r1) -> bool {
             const float x0[4] = {r0.x, r0.y, r0.z, r0.w}, x1[4] = {r1.x, r1.y, r1.z, r1.w};
+            bool care = false;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 uint32_t p0, p1, p2;
-                split2(x0[e], x1[e], p0, p1, p2);
+                care |= split2_checked(x0[e], x1[e], p0, p1, p2);
                 dst[e * kSW] = p0;
                 dst[e * kSW + plane_words] = p1;
                 dst[e * kSW + 2 * plane_words] = p2;
             }
+            return care;
         };
         auto stash = [&](int buf, const Regs &r) {
             uint32_t *base = lds + buf * kBuf;
-            int care = 0;
+            bool care = false;
 #pragma unroll
-            for (int p = 0; p < kAItems; ++p) {
-                care |= needs_care(r.a[p][0]) | needs_care(r.a[p][1]);
-                stash_quad(a_ok[p] ? base + a_dst[p] : lds + a_dst[p], a_ok[p] ? kTileK * kSW : 0, r.a[p][0], r.a[p][1]);
-            }
+            for (int p = 0; p < kAItems; ++p)
+                care |= stash_quad(a_ok[p] ? base + a_dst[p] : lds + a_dst[p], a_ok[p] ? kTileK * kSW : 0, r.a[p][0], r.a[p][1]);
             if constexpr (!BVEC) {
 #pragma unroll
                 for (int p = 0; p < kBCols; ++p) {
-                    care |= needs_care(r.bs[p][0]) | needs_care(r.bs[p][1]);
                     uint32_t p0, p1, p2;
-                    split2(r.bs[p][0], r.bs[p][1], p0, p1, p2);
+                    care |= split2_checked(r.bs[p][0], r.bs[p][1], p0, p1, p2);
                     uint32_t *dst = bs_ok[p] ? base + kAWords + (cq + kQ * p) * kSW + mp : lds + 2 * kBuf + mp;
                     const int plane_words = bs_ok[p] ? BN * kSW : 0;
                     dst[0] = p0;
@@ -243,8 +243,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
                     b0 = make_float4((w0 & 1u) ? b0.x : 0.f, (w0 & 2u) ? b0.y : 0.f, (w0 & 4u) ? b0.z : 0.f, (w0 & 8u) ? b0.w : 0.f);
                     b1 = make_float4((w1 & 1u) ? b1.x : 0.f, (w1 & 2u) ? b1.y : 0.f, (w1 & 4u) ? b1.z : 0.f, (w1 & 8u) ? b1.w : 0.f);
                 }
-                care |= needs_care(b0) | needs_care(b1);
-                stash_quad(b_ok[p] ? base + b_dst[p] : lds + b_dst[p], b_ok[p] ? BN * kSW : 0, b0, b1);
+                care |= stash_quad(b_ok[p] ? base + b_dst[p] : lds + b_dst[p], b_ok[p] ? BN * kSW : 0, b0, b1);
             }
             if (__builtin_expect(care, 0)) *g.nonfinite = 1u;
         };

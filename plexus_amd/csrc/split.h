@@ -26,10 +26,20 @@ __device__ __forceinline__ void split2(float x, float y, uint32_t &p0, uint32_t 
     p2 = plx::pack_bf16x2(sx, sy);
 }
 
+// The same split; true if x or y is a value the split cannot carry (see needs_care): the first piece of such a value is Inf
+// or NaN, which leaves NaN as the last residual, and no other value does.  One compare for the two values.
+__device__ __forceinline__ bool split2_checked(float x, float y, uint32_t &p0, uint32_t &p1, uint32_t &p2)
+{
+    p0 = plx::pack_bf16x2(x, y);
+    const float rx = x - __uint_as_float(p0 << 16), ry = y - __uint_as_float(p0 & 0xffff0000u);
+    p1 = plx::pack_bf16x2(rx, ry);
+    const float sx = rx - __uint_as_float(p1 << 16), sy = ry - __uint_as_float(p1 & 0xffff0000u);
+    p2 = plx::pack_bf16x2(sx, sy);
+    return __builtin_isunordered(sx, sy);
+}
+
 // The same split in two halves, for kernels that place them between other instructions: the first half gives the first
-// piece and what it leaves, the second the other two pieces.  `second` returns true if x or y was a value the split cannot
-// carry (see needs_care): the first piece of such a value is Inf or NaN, which leaves NaN as the last residual, and no
-// other value does -- one compare for the two values.
+// piece and what it leaves, the second the other two pieces and the same answer as split2_checked.
 __device__ __forceinline__ void split2_first(float x, float y, uint32_t &p0, float &rx, float &ry)
 {
     p0 = plx::pack_bf16x2(x, y);
