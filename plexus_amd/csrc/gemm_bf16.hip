@@ -307,12 +307,12 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     constexpr bool BITS = MASK == 2;
     static_assert(!BITS || FAST, "the bit mask is read by the unconditional kernel only");
     constexpr int kSteps = KS;             // chunk positions of a panel (positions past K are skipped)
-    constexpr int kRing = (MASKED || TN > 4) ? 4 : KS; // register slots = positions ahead that a chunk is requested
+    constexpr int kRing = (MASKED || FAST || TN > 4) ? 4 : KS;  // register slots = positions ahead that a chunk is requested
     static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;  // [kRMax][kRBS]
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: panel arithmetic stays scalar
     const int li = lane & 31;
     const int h = lane >> 5;
     uint16_t *const apriv = rlds + kRMax * kRBS + wave * kRPrivate;
@@ -344,22 +344,40 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     uint4 pb_cur[KS / 4], pb_next[KS / 4];  // bit mask: word kc of the lane's row covers chunk position kc
 #pragma unroll
     for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q] = make_uint4(~0u, ~0u, ~0u, ~0u);
+    // byte offsets of a lane's row inside a panel (in the last panel: clamped to the last row of the matrix) and of the last
+    // eight columns, to which a lane's columns are clamped; the host keeps 128 leading dimensions below 2^32 bytes for the
+    // unconditional kernel
+    uint32_t a_off = 0, a_off_last = 0, m_off = 0, m_off_last = 0, w_off = 0, w_off_last = 0;
+    const uint32_t k_last = 2u * (uint32_t)(K - 8);
+    if constexpr (FAST) {
+        const uint32_t row_last = (uint32_t)min(r, (int)(g.M - (n_panels - 1) * 32) - 1);
+        a_off = (uint32_t)r * (uint32_t)g.lda * 2u;
+        a_off_last = row_last * (uint32_t)g.lda * 2u;
+        if constexpr (MASKED) m_off = (uint32_t)r * (uint32_t)g.ldmask * 2u, m_off_last = row_last * (uint32_t)g.ldmask * 2u;
+        if constexpr (BITS) w_off = (uint32_t)r * (uint32_t)g.ldw * 4u, w_off_last = row_last * (uint32_t)g.ldw * 4u;
+    }
     // `pos`, `of_panel`: the position a request is for (the unconditional form takes them from its caller, where they are
     // compile-time and loop-invariant values; the guarded form follows its cursor)
     auto fetch = [&](uint4(&dst)[2], uint4(&mdst)[2], int pos, int64_t of_panel) __attribute__((always_inline)) {
         if constexpr (FAST) {
-            const int64_t row = min(min(of_panel, n_panels - 1) * 32 + r, g.M - 1);
+            // the panel's address is the same in every lane (scalar arithmetic); a lane adds a 32-bit byte offset that does
+            // not depend on the panel, except that the rows of the last panel are clamped into the matrix
+            const int64_t panel = min(of_panel, n_panels - 1);
+            const bool last = panel == n_panels - 1;
+            const char *const pa = reinterpret_cast<const char *>(g.A) + panel * 64 * g.lda;
+            const char *const pm = MASKED ? reinterpret_cast<const char *>(g.mask) + panel * 64 * g.ldmask : nullptr;
             if constexpr (BITS) {
                 if (pos == 0) {
+                    const char *const pw = reinterpret_cast<const char *>(g.mask_bits) + panel * 128 * g.ldw + (last ? w_off_last : w_off);
 #pragma unroll
-                    for (int q = 0; q < KS / 4; ++q) pb_next[q] = *reinterpret_cast<const uint4 *>(g.mask_bits + row * g.ldw + 4 * q);
+                    for (int q = 0; q < KS / 4; ++q) pb_next[q] = *reinterpret_cast<const uint4 *>(pw + 16 * q);
                 }
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int k = min(pos * kRCK + half * 16 + 8 * j, K - 8);
-                dst[j] = *reinterpret_cast<const uint4 *>(g.A + row * g.lda + k);
-                if constexpr (MASKED) mdst[j] = *reinterpret_cast<const uint4 *>(g.mask + row * g.ldmask + k);
+                const uint32_t k_off = min((uint32_t)(pos * kRCK * 2 + half * 32 + 16 * j), k_last);
+                dst[j] = *reinterpret_cast<const uint4 *>(pa + ((last ? a_off_last : a_off) + k_off));
+                if constexpr (MASKED) mdst[j] = *reinterpret_cast<const uint4 *>(pm + ((last ? m_off_last : m_off) + k_off));
             }
             return;
         }
@@ -434,17 +452,9 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     float *const cs = reinterpret_cast<float *>(apriv);
     const int srow = lane >> 2, scq = lane & 3;  // staged half tile: this lane reads 8 columns of row srow
 
-#pragma unroll
-    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
     uint32_t wkeep[2][(TN + 3) / 4] = {};
-    for (int64_t panel = first; panel < n_panels; panel += stride) {
-        cur_panel = panel;
-        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
-#pragma unroll
-            for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q];
-        }
-#pragma unroll
-        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+    // a finished panel: scaling, ReLU, dropout, sign bits, stores; leaves the accumulators zero
+    auto finish_panel = [&](int64_t panel) __attribute__((always_inline)) {
         // register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -511,6 +521,102 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
                     if (row < g.M && (scq + 4 * q) * 32 < N) g.relu_bits[row * g.ldw_out + scq + 4 * q] = wkeep[pass][q];
             }
         }
+    };
+
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) fetch(ring[i], mring[MASKED ? i : 0], i, first);
+
+    if constexpr (FAST) {
+        // The positions run as a pipeline inside the wavefront: the pieces of B are read kPiecesAhead products before the product
+        // that takes them (B is resident, so this runs across positions and panels), the next position of A goes to the
+        // private tile in the middle of the current one -- the tile is free once the current position's operands are in
+        // registers -- and comes back as operands before the current one ends.  The order written here is pinned: an empty
+        // asm statement takes each product's result as its operand, and a scheduling barrier follows.
+        constexpr int kPiecesAhead = (MASKED && TN > 6) ? 1 : 4;  // (the widest kernel that carries mask values has registers for one)
+        constexpr int kPer = 2 * TN;   // products of a position
+        constexpr int kStoreAt = TN;   // the product before which the next position is stored
+        static_assert(kRing == 4 && (kSteps * kPer) % kPiecesAhead == 0, "buffers are chosen by compile-time counts");
+        bf16x8 aa[2][2], bq[kPiecesAhead];
+        auto load_a = [&](bf16x8(&a)[2]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) a[sub] = *reinterpret_cast<const bf16x8 *>(a_src + 16 * sub);
+        };
+        auto load_b = [&](bf16x8 &b, int kc, int idx) __attribute__((always_inline)) {
+            b = *reinterpret_cast<const bf16x8 *>(b_src + (idx % TN) * 32 * kRBS + kc * kRCK + 16 * (idx / TN));
+        };
+        auto store_chunk = [&](const uint4(&c)[2], const uint4(&mc)[2], const uint4(&pb)[KS / 4], int kc) __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 v = c[j];
+                if constexpr (MASKED) v = mask8(v, mc[j]);
+                if constexpr (BITS) {
+                    const uint4 w4 = pb[kc >> 2];
+                    const uint32_t word = (kc & 3) == 0 ? w4.x : ((kc & 3) == 1 ? w4.y : ((kc & 3) == 2 ? w4.z : w4.w));
+                    v = mask8_bits(v, word >> (16 * half + 8 * j));
+                }
+                *reinterpret_cast<uint4 *>(a_dst + 8 * j) = v;
+            }
+        };
+        if constexpr (BITS) {
+#pragma unroll
+            for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q];
+        }
+        store_chunk(ring[0], mring[0], pb_cur, 0);
+        plx::wave_lds_fence();
+        load_a(aa[0]);
+#pragma unroll
+        for (int d = 0; d < kPiecesAhead; ++d) load_b(bq[d], (d / kPer) % kSteps, d % kPer);
+        plx::wave_lds_fence();
+
+        for (int64_t panel = first; panel < n_panels; panel += stride) {
+#pragma unroll
+            for (int kc = 0; kc < kSteps; ++kc) {
+                const bool wrap = kc + 1 == kSteps;  // the next position is the first of this wavefront's next panel
+                const int nc = wrap ? 0 : kc + 1, slot = (kc + 1) % kRing;
+#pragma unroll
+                for (int idx = 0; idx < kPer; ++idx) {
+                    const int count = kc * kPer + idx;  // products since the panel began
+                    if (idx == kStoreAt) {
+                        plx::wave_lds_fence();  // after the loads of this position's operands (and a finished panel's staging)
+                        store_chunk(ring[slot], mring[MASKED ? slot : 0], wrap ? pb_next : pb_cur, nc);
+                        if constexpr (BITS) {
+                            if (wrap) {  // before a request replaces them with the bits of the panel after
+#pragma unroll
+                                for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q];
+                            }
+                        }
+                        // requests go out for two positions at a time, which share their 128-byte lines: positions kc + 4
+                        // and kc + 5 into the slots of positions kc and kc + 1, both stored by now
+                        if ((kc & 1) == 0) {
+                            fetch(ring[kc % kRing], mring[MASKED ? kc % kRing : 0], (kc + kRing) % kSteps, panel + ((kc + kRing) / kSteps) * stride);
+                            fetch(ring[slot], mring[MASKED ? slot : 0], (kc + 1 + kRing) % kSteps, panel + ((kc + 1 + kRing) / kSteps) * stride);
+                        }
+                        plx::wave_lds_fence();
+                        load_a(aa[(kc + 1) & 1]);
+                        plx::wave_lds_fence();
+                    }
+                    acc[idx % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aa[kc & 1][idx / TN], bq[count % kPiecesAhead], acc[idx % TN], 0, 0, 0);
+                    asm volatile("" : "+v"(acc[idx % TN]));
+                    const int ahead = count + kPiecesAhead;  // the product that takes the piece read now, into the buffer just used
+                    load_b(bq[count % kPiecesAhead], (ahead / kPer) % kSteps, ahead % kPer);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            plx::wave_lds_fence();  // the staging of the panel comes after the loads of the next position's operands
+            finish_panel(panel);
+        }
+        return;
+    }
+
+    for (int64_t panel = first; panel < n_panels; panel += stride) {
+        cur_panel = panel;
+        if constexpr (BITS) {  // the bits that came with this panel's first chunk; the steps below fetch the next panel's
+#pragma unroll
+            for (int q = 0; q < KS / 4; ++q) pb_cur[q] = pb_next[q];
+        }
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) step(i, ring[i % kRing], mring[MASKED ? i % kRing : 0]);
+        finish_panel(panel);
     }
 }
 
@@ -528,9 +634,16 @@ int launch_nt_resident_one(const Bf16Args &g, unsigned blocks, hipStream_t st)
 // operands that take 16-byte loads go to the kernel whose requests are unconditional, with as many chunk positions as K needs
 // whether the resident kernel can read the mask of this product as bits: the unconditional form, rows of bits that take
 // 16-byte loads and hold a word for every chunk position the kernel walks
+// the unconditional kernel's lanes address a panel with 32-bit byte offsets
+bool resident_offsets_fit(const Bf16Args &g)
+{
+    const int64_t ld_max = (int64_t)1 << 24;
+    return g.lda < ld_max && g.ldmask < ld_max && g.ldw < ld_max;
+}
+
 bool resident_takes_bits(const Bf16Args &g)
 {
-    if (g.mask_bits == nullptr || !(g.a_vec && g.K % 8 == 0 && g.K >= 8)) return false;
+    if (g.mask_bits == nullptr || !(g.a_vec && g.K % 8 == 0 && g.K >= 8) || !resident_offsets_fit(g)) return false;
     const int64_t words = g.K <= 4 * kRCK ? 4 : 8;
     return reinterpret_cast<uintptr_t>(g.mask_bits) % 16 == 0 && g.ldw % 4 == 0 && g.ldw >= words;
 }
@@ -545,7 +658,7 @@ int launch_nt_resident(const Bf16Args &g, unsigned blocks, hipStream_t st)
         }
     }
     constexpr int MASK = MASKED ? 1 : 0;
-    if (g.a_vec && g.m_vec && g.K % 8 == 0 && g.K >= 8) {
+    if (g.a_vec && g.m_vec && g.K % 8 == 0 && g.K >= 8 && resident_offsets_fit(g)) {
         if constexpr (!MASKED) {
             if (g.relu_bits != nullptr) {
                 if (g.K <= 4 * kRCK) return launch_nt_resident_one<TN, 0, true, 4, true>(g, blocks, st);
