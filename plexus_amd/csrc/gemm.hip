@@ -171,8 +171,9 @@ struct TotalsTN<true, TN> {
     }
 };
 
+// one output tile; `bx` is the workgroup's first grid coordinate (row tile of NN / NT, stretch of rows of TN)
 template <int MODE, int TN>
-__global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
+__device__ __forceinline__ void gemm_f32_tile(const GemmArgs &g, float *lds, const int64_t bx)
 {
     constexpr int BN = 32 * TN;
     constexpr bool kAX = (MODE != kTN);  // A tile x-major?
@@ -184,8 +185,6 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     using ATile = Tile<(kAX ? kBM : kBK), (kAX ? kBK : kBM), kAStride>;
     using BTile = Tile<(kBX ? BN : kBK), (kBX ? kBK : BN), kBStride>;
 
-    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
-    if (guard_says_skip(g)) return;
     auto a_buf = [&](int i) { return lds + i * kASize; };
     auto b_buf = [&](int i) { return lds + 2 * kASize + i * kBSize; };
 
@@ -199,10 +198,10 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     if constexpr (MODE == kTN) {
         row0 = (int64_t)blockIdx.y * kBM;  // rows of C = columns of A
         col0 = (int64_t)blockIdx.z * BN;
-        kbeg = (int64_t)blockIdx.x * g.rows_per_split;
+        kbeg = bx * g.rows_per_split;
         kend = min(kbeg + g.rows_per_split, g.M);
     } else {
-        row0 = (int64_t)blockIdx.x * kBM;
+        row0 = bx * kBM;
         col0 = (int64_t)blockIdx.y * BN;
         kbeg = 0;
         kend = g.K;
@@ -298,7 +297,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     int64_t ldo, nrows, ncols;
     if constexpr (MODE == kTN) {
         if (g.ws != nullptr) {
-            out = g.ws + (int64_t)blockIdx.x * g.ws_slab;
+            out = g.ws + bx * g.ws_slab;
             ldo = g.ws_ld;
         } else {
             out = g.C;
@@ -330,6 +329,27 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
     }
 }
 
+// NN / NT: a workgroup walks the row tiles bx, bx + gridDim.x, ... (one each unless the launch is a guarded one, whose grid
+// is small so that it costs little when it has nothing to do); TN: one stretch of rows per workgroup
+template <int MODE, int TN>
+__global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr int kASize = (MODE != kTN) ? kBM * kXS : kBK * kBM;
+    constexpr int kBSize = (MODE == kNT) ? BN * kXS : kBK * BN;
+    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+    if (guard_says_skip(g)) return;
+    if constexpr (MODE == kTN) {
+        gemm_f32_tile<MODE, TN>(g, lds, (int64_t)blockIdx.x);
+    } else {
+        const int64_t row_tiles = (g.M + kBM - 1) / kBM;
+        for (int64_t bx = blockIdx.x; bx < row_tiles; bx += gridDim.x) {
+            gemm_f32_tile<MODE, TN>(g, lds, bx);
+            __syncthreads();  // the next tile's first chunk overwrites the buffers
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Lean variant for aligned operands (every base 16-byte aligned, every leading dimension and the
 // contraction / column extents multiples of 4).  Same tiling and LDS layouts as gemm_f32_kernel; the
@@ -338,7 +358,7 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g)
 // ~8 vector-ALU instructions per MFMA, which is what keeps its MFMA pipe half idle.
 // ---------------------------------------------------------------------------------------------------
 template <int MODE, int TN, bool MASKED>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm_f32_vec_kernel(const GemmArgs g)
+__device__ __forceinline__ void gemm_f32_vec_tile(const GemmArgs &g, float *lds, const int64_t bx)
 {
     constexpr int BN = 32 * TN;
     constexpr bool kAX = (MODE != kTN);
@@ -352,8 +372,6 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
     constexpr int kBV = (kBX ? kBK : BN) / 4, kBRows = kBX ? BN : kBK, kBPass = kThreads / kBV;
     constexpr int kAPer = (kARows + kAPass - 1) / kAPass, kBPer = (kBRows + kBPass - 1) / kBPass;
 
-    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
-    if (guard_says_skip(g)) return;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -364,10 +382,10 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
     if constexpr (MODE == kTN) {
         row0 = (int64_t)blockIdx.y * kBM;
         col0 = (int64_t)blockIdx.z * BN;
-        kbeg = (int64_t)blockIdx.x * g.rows_per_split;
+        kbeg = bx * g.rows_per_split;
         kend = min(kbeg + g.rows_per_split, g.M);
     } else {
-        row0 = (int64_t)blockIdx.x * kBM;
+        row0 = bx * kBM;
         col0 = (int64_t)blockIdx.y * BN;
         kbeg = 0;
         kend = g.K;
@@ -522,7 +540,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
     int64_t ldo, nrows, ncols;
     if constexpr (MODE == kTN) {
         if (g.ws != nullptr) {
-            out = g.ws + (int64_t)blockIdx.x * g.ws_slab;
+            out = g.ws + bx * g.ws_slab;
             ldo = g.ws_ld;
         } else {
             out = g.C;
@@ -555,6 +573,25 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
                     if (t * 32 < cols_left) q[t * 32] = x;
                 }
             }
+        }
+    }
+}
+
+template <int MODE, int TN, bool MASKED>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) gemm_f32_vec_kernel(const GemmArgs g)
+{
+    constexpr int BN = 32 * TN;
+    constexpr int kASize = (MODE != kTN) ? kBM * kXS : kBK * kBM;
+    constexpr int kBSize = (MODE == kNT) ? BN * kXS : kBK * BN;
+    __shared__ __attribute__((aligned(16))) float lds[2 * (kASize + kBSize)];
+    if (guard_says_skip(g)) return;
+    if constexpr (MODE == kTN) {
+        gemm_f32_vec_tile<MODE, TN, MASKED>(g, lds, (int64_t)blockIdx.x);
+    } else {
+        const int64_t row_tiles = (g.M + kBM - 1) / kBM;
+        for (int64_t bx = blockIdx.x; bx < row_tiles; bx += gridDim.x) {
+            gemm_f32_vec_tile<MODE, TN, MASKED>(g, lds, bx);
+            __syncthreads();  // the next tile's first chunk overwrites the buffers
         }
     }
 }
@@ -633,6 +670,14 @@ void launch_gemm(const GemmArgs &g, int tn, dim3 grid, hipStream_t st)
     }
 }
 
+// Row tiles of an NN / NT launch.  A guarded launch (one that runs only if a split product has raised its flag, which is
+// rare) takes a grid of at most 1,024 workgroups that walk the row tiles: 19,000 workgroups that all return at once still
+// keep the GPU busy for 15 us.
+unsigned guarded_grid(int64_t row_tiles, const unsigned *run_if)
+{
+    return (unsigned)(run_if != nullptr ? std::min<int64_t>(row_tiles, 1024) : row_tiles);
+}
+
 int check_common(const char *who, int64_t M, int64_t N, int64_t K, const void *A, const void *B, const void *C)
 {
     PLX_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative dimension", who);
@@ -664,7 +709,7 @@ int gemm_nn_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb);
     g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
-    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
+    dim3 grid(guarded_grid(plx::ceil_div(M, kBM), run_if), (unsigned)plx::ceil_div(N, 32 * tn), 1);
     launch_gemm<kNN>(g, tn, grid, plx::as_stream(stream));
     PLX_LAUNCH_CHECK("gemm_f32_kernel<NN>");
     return PLX_OK;
@@ -683,7 +728,7 @@ int gemm_nt_impl(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, c
     g.a_vec = vec_ok(A, lda); g.b_vec = vec_ok(B, ldb); g.m_vec = vec_ok(mask, ldmask);
     g.run_if = run_if; g.n_run_if = n_run_if;
     const int tn = pick_tn(N);
-    dim3 grid((unsigned)plx::ceil_div(M, kBM), (unsigned)plx::ceil_div(N, 32 * tn), 1);
+    dim3 grid(guarded_grid(plx::ceil_div(M, kBM), run_if), (unsigned)plx::ceil_div(N, 32 * tn), 1);
     launch_gemm<kNT>(g, tn, grid, plx::as_stream(stream));
     PLX_LAUNCH_CHECK("gemm_f32_kernel<NT>");
     return PLX_OK;

@@ -842,7 +842,9 @@ int launch_dropout(int64_t M, int64_t N, float *X, int64_t ldx, const DropArgs &
 {
     const int64_t calls = (M * N + 7) / 8;
     if (calls == 0) return PLX_OK;
-    dropout_f32_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(calls, 256), 1 << 20), 256, 0, st>>>(M, N, X, ldx, a, run_if);
+    // (a guarded launch, which seldom has anything to do, takes a small grid: returning at once from 150,000 workgroups takes 50 us)
+    const int64_t max_blocks = run_if != nullptr ? 2048 : 1 << 20;
+    dropout_f32_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(calls, 256), max_blocks), 256, 0, st>>>(M, N, X, ldx, a, run_if);
     PLX_LAUNCH_CHECK("dropout_f32_kernel");
     return PLX_OK;
 }
@@ -866,22 +868,26 @@ __global__ void __launch_bounds__(256) sign_bits_kernel(int64_t M, int64_t N, co
                                                         uint32_t *__restrict__ bits, int64_t ldw, const unsigned *__restrict__ run_if)
 {
     if (run_if != nullptr && *run_if == 0u) return;
-    const int64_t words = (N + 31) / 32;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < M * words; i += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t row = i / words, w = i % words;
-        const float *x = X + row * ldx + w * 32;
-        const int n = (int)min((int64_t)32, N - w * 32);
-        uint32_t word = 0;
-        for (int c = 0; c < n; ++c) word |= (x[c] > 0.f ? 1u : 0u) << c;
-        bits[row * ldw + w] = word;
+    // a wavefront takes 64 consecutive columns of a row: one element per lane, one vote, two words
+    const int lane = threadIdx.x & 63;
+    const int64_t groups = (N + 63) / 64;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6, waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    for (int64_t i = wave; i < M * groups; i += waves) {
+        const int64_t row = i / groups, c0 = (i % groups) * 64;
+        const bool positive = c0 + lane < N && X[row * ldx + c0 + lane] > 0.f;
+        const uint64_t votes = __ballot(positive);
+        if (lane == 0) bits[row * ldw + c0 / 32] = (uint32_t)votes;
+        if (lane == 32 && c0 + 32 < N) bits[row * ldw + c0 / 32 + 1] = (uint32_t)(votes >> 32);
     }
 }
 
 int launch_sign_bits(int64_t M, int64_t N, const float *X, int64_t ldx, uint32_t *bits, int64_t ldw, const unsigned *run_if, hipStream_t st)
 {
-    const int64_t items = M * ((N + 31) / 32);
+    const int64_t items = M * ((N + 63) / 64);  // one wavefront each
     if (items == 0) return PLX_OK;
-    sign_bits_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(items, 256), 8192), 256, 0, st>>>(M, N, X, ldx, bits, ldw, run_if);
+    // (a guarded launch, which seldom has anything to do, takes a small grid)
+    const int64_t max_blocks = run_if != nullptr ? 2048 : 1 << 16;
+    sign_bits_kernel<<<(unsigned)std::min<int64_t>(plx::ceil_div(items, 4), max_blocks), 256, 0, st>>>(M, N, X, ldx, bits, ldw, run_if);
     PLX_LAUNCH_CHECK("sign_bits_kernel");
     return PLX_OK;
 }
