@@ -33,6 +33,11 @@ constexpr int kBK = 32;      // contraction chunk
 constexpr int kS = kBK + 8;  // LDS row stride of a plane in bf16 elements (80 bytes: 128-bit reads conflict-free)
 constexpr int kThreads = 256;
 
+// four floats at an address that is a multiple of 4 only
+struct __attribute__((packed, aligned(4))) Float4Align4 {
+    float x, y, z, w;
+};
+
 struct SplitArgs {
     const float *A;
     const float *mask;
@@ -319,7 +324,11 @@ constexpr size_t kRLdsBytes = ((size_t)3 * kRMaxN * kRBS + (size_t)kRWaves * 3 *
 // four and meet the zero padding of the planes), with no branch around it: the wait the compiler places before a
 // chunk is used can then name how many younger requests may stay in flight, where loads inside branches make it wait
 // for all of them -- which is what decides the speed of this kernel.
-template <int TN, int MASK, bool DROP = false, bool FAST = false, int KS = 8>
+// ROWS16 = false (unconditional kernel without a mask): the rows of A are only 4-byte aligned and K is any number from 4 up (the
+// 47-wide gradient of a last layer).  The same 16-byte requests -- the compiler emits them for 4-byte aligned data, which this
+// hardware reads -- except that the vector which would reach past the end of a row is requested from the row's last four
+// elements and shifted into place when it is used.
+template <int TN, int MASK, bool DROP = false, bool FAST = false, int KS = 8, bool ROWS16 = true>
 __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel(const SplitArgs g)
 {
     constexpr bool MASKED = MASK == 1;      // the fp32 mask travels in registers beside its chunk
@@ -327,6 +336,7 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     constexpr int kSteps = KS;              // chunk positions of a panel (positions past K are skipped)
     constexpr int kRing = (MASKED || FAST) ? 4 : KS;  // register slots = how many positions ahead a chunk is requested
     static_assert(KS == 8 || (FAST && KS == 4), "the guarded kernel walks all eight positions");
+    static_assert(ROWS16 || (FAST && MASK == 0 && !DROP), "rows without 16-byte alignment: the plain unconditional kernel only");
     extern __shared__ __attribute__((aligned(16))) uint16_t rlds[];
     uint16_t *const bres = rlds;                               // [3][kRMaxN][kRBS]
     constexpr int kBPlane = kRMaxN * kRBS;
@@ -404,7 +414,12 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
             const uint32_t k_off = min((uint32_t)(pos * kRCK * 4 + kq * 16), k_last);
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                dst[p] = *reinterpret_cast<const float4 *>(pa + ((last ? a_off_last[p] : a_off[p]) + k_off));
+                if constexpr (ROWS16) {
+                    dst[p] = *reinterpret_cast<const float4 *>(pa + ((last ? a_off_last[p] : a_off[p]) + k_off));
+                } else {
+                    const Float4Align4 v = *reinterpret_cast<const Float4Align4 *>(pa + ((last ? a_off_last[p] : a_off[p]) + k_off));
+                    dst[p] = make_float4(v.x, v.y, v.z, v.w);
+                }
                 if constexpr (MASKED) mdst[p] = *reinterpret_cast<const float4 *>(pm + ((last ? m_off_last[p] : m_off[p]) + k_off));
                 if constexpr (BITS) {
                     if (pos == 0) pb_next[p] = *reinterpret_cast<const u32x4 *>(pw + (last ? w_off_last[p] : w_off[p]));
@@ -642,6 +657,17 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
         };
         auto masked = [&](const float4 &a, const float4 &m, const u32x4 &bits, int kc) __attribute__((always_inline)) -> float4 {
             float4 v = a;
+            if constexpr (!ROWS16) {
+                // this lane's columns are kc 16 + 4 kq ...; the request was clamped to K - 4, so what it brought lies `over`
+                // elements to the right of its place, and the elements past K count as zero
+                const int over = kc * kRCK + kq * 4 - (K - 4);
+                if (over > 0) {
+                    v.x = over == 1 ? a.y : over == 2 ? a.z : over == 3 ? a.w : 0.f;
+                    v.y = over == 1 ? a.z : over == 2 ? a.w : 0.f;
+                    v.z = over == 1 ? a.w : 0.f;
+                    v.w = 0.f;
+                }
+            }
             if constexpr (MASKED) v = make_float4(m.x > 0.f ? v.x : 0.f, m.y > 0.f ? v.y : 0.f, m.z > 0.f ? v.z : 0.f, m.w > 0.f ? v.w : 0.f);
             if constexpr (BITS) {
                 // chunk kc holds contraction elements 16 kc ...: bits 16 (kc % 2) + 4 kq ... of word kc / 2
@@ -773,14 +799,14 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
     }
 }
 
-template <int TN, int MASK, bool DROP, bool FAST, int KS>
+template <int TN, int MASK, bool DROP, bool FAST, int KS, bool ROWS16 = true>
 int launch_resident_one(const SplitArgs &g, unsigned blocks, hipStream_t st)
 {
     static std::atomic<uint64_t> allowed{0};  // devices on which this instantiation may take its LDS
-    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS>), kRLdsBytes,
-                                          allowed);
+    const int rc = plx::allow_dynamic_lds(reinterpret_cast<const void *>(&gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS, ROWS16>),
+                                          kRLdsBytes, allowed);
     if (rc != PLX_OK) return rc;
-    gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
+    gemm_split_nt_resident_kernel<TN, MASK, DROP, FAST, KS, ROWS16><<<blocks, kRWaves * 64, kRLdsBytes, st>>>(g);
     return PLX_OK;
 }
 
@@ -793,6 +819,12 @@ int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
     if (g.a_vec && g.K >= 4 && g.lda < ld_max && g.ldmask < ld_max && g.ldw < ld_max) {
         if (g.K <= 64) return launch_resident_one<TN, MASK, DROP, true, 4>(g, blocks, st);
         return launch_resident_one<TN, MASK, DROP, true, 8>(g, blocks, st);
+    }
+    if constexpr (MASK == 0 && !DROP) {  // rows of A without 16-byte alignment, or a K that is not a multiple of 4
+        if (g.K >= 4 && g.lda < ld_max) {
+            if (g.K <= 64) return launch_resident_one<TN, 0, false, true, 4, false>(g, blocks, st);
+            return launch_resident_one<TN, 0, false, true, 8, false>(g, blocks, st);
+        }
     }
     return launch_resident_one<TN, MASK, DROP, false, 8>(g, blocks, st);
 }
