@@ -315,20 +315,51 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
     // a lane reads row li of its 32-row block of a plane: words 8 s + 4 h ... + 3 are contraction rows 16 s + 8 h ... + 7
     const uint16_t *const a_src = reinterpret_cast<const uint16_t *>(lds) + ((kb * 32 + li) * kSW + 4 * h) * 2;
     const uint16_t *const b_src = reinterpret_cast<const uint16_t *>(lds + kAWords) + ((nh * TNH * 32 + li) * kSW + 4 * h) * 2;
+    // With two column tiles per wavefront the pieces of B are read one tile ahead of their products into a second register set
+    // (the order is pinned: an empty asm statement takes each tile's accumulator, a scheduling barrier follows).  With four tiles
+    // the 128 accumulators and totals leave no registers for that set (12 wavefronts: 168 registers each), and the pieces are
+    // read where they are used.
+    constexpr bool kAheadB = TNH <= 2;
     auto compute = [&](int buf) {
         const uint16_t *as = a_src + buf * kBuf * 2, *bs = b_src + buf * kBuf * 2;
+        if constexpr (!kAheadB) {
 #pragma unroll
-        for (int s = 0; s < kRows / 16; ++s) {
-            const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(as + 16 * s);
-            const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(as + 16 * s + kTileK * kSW * 2);
-            const bf16x8 a2 = *reinterpret_cast<const bf16x8 *>(as + 16 * s + 2 * kTileK * kSW * 2);
+            for (int s = 0; s < kRows / 16; ++s) {
+                const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(as + 16 * s);
+                const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(as + 16 * s + kTileK * kSW * 2);
+                const bf16x8 a2 = *reinterpret_cast<const bf16x8 *>(as + 16 * s + 2 * kTileK * kSW * 2);
+#pragma unroll
+                for (int t = 0; t < TNH; ++t) {
+                    const uint16_t *bt = bs + t * 32 * kSW * 2 + 16 * s;
+                    const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(bt);
+                    const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(bt + BN * kSW * 2);
+                    const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bt + 2 * BN * kSW * 2);
+                    acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
+                }
+            }
+            return;
+        }
+        auto load_b = [&](bf16x8(&b)[3], int sub, int t) __attribute__((always_inline)) {
+            const uint16_t *bt = bs + t * 32 * kSW * 2 + 16 * sub;
+            b[0] = *reinterpret_cast<const bf16x8 *>(bt);
+            b[1] = *reinterpret_cast<const bf16x8 *>(bt + BN * kSW * 2);
+            b[2] = *reinterpret_cast<const bf16x8 *>(bt + 2 * BN * kSW * 2);
+        };
+        bf16x8 bb[2][3];
+        load_b(bb[0], 0, 0);
+#pragma unroll
+        for (int sub = 0; sub < kRows / 16; ++sub) {
+            const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(as + 16 * sub);
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(as + 16 * sub + kTileK * kSW * 2);
+            const bf16x8 a2 = *reinterpret_cast<const bf16x8 *>(as + 16 * sub + 2 * kTileK * kSW * 2);
 #pragma unroll
             for (int t = 0; t < TNH; ++t) {
-                const uint16_t *bt = bs + t * 32 * kSW * 2 + 16 * s;
-                const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(bt);
-                const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(bt + BN * kSW * 2);
-                const bf16x8 b2 = *reinterpret_cast<const bf16x8 *>(bt + 2 * BN * kSW * 2);
-                acc[t] = mfma6(a0, a1, a2, b0, b1, b2, acc[t]);
+                const int group = sub * TNH + t;
+                if (t + 1 < TNH) load_b(bb[(group + 1) & 1], sub, t + 1);
+                else if (sub + 1 < kRows / 16) load_b(bb[(group + 1) & 1], sub + 1, 0);
+                acc[t] = mfma6(a0, a1, a2, bb[group & 1][0], bb[group & 1][1], bb[group & 1][2], acc[t]);
+                asm volatile("" : "+v"(acc[t]));
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
