@@ -47,6 +47,7 @@ struct Bf16Args {
     float keep_scale;    // 1 / (1 - p)
     uint32_t seed_lo, seed_hi, off_lo, off_hi;
     int a_vec, b_vec, c_vec, m_vec;
+    int c_flat;  // resident NT kernel: C 16-byte aligned and contiguous (ldc == N), N <= 64, no dropout, no sign bits: half panels leave as flat runs
     // the mask as one bit per element (bit c % 32 of word [row * ldw + c / 32]): read in place of `mask` by the resident NT
     // kernel and the whole-tile TN kernel, written for C (its positive elements) by the resident NT kernel
     const uint32_t *mask_bits;
@@ -456,6 +457,38 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_bf16_nt_resident_kernel(
     // a finished panel: scaling, ReLU, dropout, sign bits, stores; leaves the accumulators zero
     auto finish_panel = [&](int64_t panel) __attribute__((always_inline)) {
         // register v of a lane is row 8 (v / 4) + 4 h + v % 4, column lane % 32 of each 32 x 32 block
+        // A contiguous C whose rows are not multiples of 16 bytes (47 columns): 16 rows of it are still one aligned run of 32 N
+        // bytes.  The half panel is staged row-major as bf16 without padding (N <= 64 here)
+        // and leaves in 16-byte stores.
+        if constexpr (TN <= 2) if (g.c_flat) {  // (N <= 64: the wider kernels have no registers to spare for a second epilogue)
+            uint16_t *const stage = apriv;  // [16][N]
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+                for (int t = 0; t < TN; ++t) {
+#pragma unroll
+                    for (int v = 0; v < 8; ++v) {
+                        float x = acc[t][8 * pass + v] * g.alpha;
+                        if (relu) x = fmaxf(x, 0.f);
+                        if (li + t * 32 < N) stage[(8 * (v / 4) + 4 * h + (v % 4)) * N + t * 32 + li] = (uint16_t)plx::f32_to_bf16(x);
+                        acc[t][8 * pass + v] = 0.f;
+                    }
+                }
+                plx::wave_lds_fence();
+                const int64_t row_first = panel * 32 + 16 * pass;
+                const int valid = (int)min(max(g.M - row_first, (int64_t)0), (int64_t)16) * N;  // elements of this half panel that exist
+                uint16_t *const dst = C + row_first * N;
+                for (int i = 8 * lane; i < valid; i += 512) {
+                    if (i + 8 <= valid) {
+                        *reinterpret_cast<uint4 *>(dst + i) = *reinterpret_cast<const uint4 *>(stage + i);
+                    } else {
+                        for (int e = i; e < valid; ++e) dst[e] = stage[e];
+                    }
+                }
+                plx::wave_lds_fence();  // the next half, or the next panel's first chunk, overwrites the staging
+            }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
 #pragma unroll
@@ -1126,7 +1159,9 @@ int plx_gemm_nt_bf16_bits(int64_t M, int64_t N, int64_t K, const uint16_t *A, in
     dim3 grid((unsigned)blocks, 1, 1);
     const bool vec = g.a_vec && g.b_vec && g.m_vec && K % 8 == 0;
     hipStream_t st = plx::as_stream(stream);
-    const bool resident = g.c_vec && N % 8 == 0 && N <= kRMax && K <= kRMax && K > 0;
+    g.c_flat = (!(g.c_vec && N % 8 == 0) && reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc == N && N <= 64 && (flags & PLX_GEMM_DROPOUT) == 0 &&
+                relu_bits == nullptr) ? 1 : 0;
+    const bool resident = ((g.c_vec && N % 8 == 0) || g.c_flat) && N <= kRMax && K <= kRMax && K > 0;
     if (relu_bits != nullptr && !(resident && mask == nullptr && g.a_vec && K % 8 == 0 && K >= 8))  // only one form of the kernel writes them
         return plx::fail(PLX_ERR_UNSUPPORTED, "gemm_nt_bf16: sign bits are written for N, K <= %d with N and K multiples of 8, 16-byte rows of A "
                                               "and C, and no mask", kRMax);

@@ -50,6 +50,7 @@ struct SplitArgs {
     unsigned *nonfinite;  // device word raised when an operand holds a value the split cannot carry
     int a_vec;  // A (and mask) 16-byte aligned, leading dimensions and K multiples of 4: 128-bit loads
     int c_vec;  // C 16-byte aligned, ldc and N multiples of 4: 128-bit stores
+    int c_flat;  // C 16-byte aligned and contiguous (ldc == N), N <= 64, no sign bits asked for: half panels leave as flat runs of 16-byte stores
     // dropout after the ReLU (resident NT kernel): element e = row * N + col is kept iff 16-bit lane e % 8 of
     // Philox-4x32-10(counter = (e / 8, offset), key = seed) is >= thresh16, and then scaled by keep_scale
     uint32_t thresh16, seed_lo, seed_hi, off_lo, off_hi;
@@ -599,6 +600,39 @@ __global__ void __launch_bounds__(kRWaves * 64, 1) gemm_split_nt_resident_kernel
                 }
                 return;
             }
+            // A contiguous C whose rows are not multiples of 16 bytes (47 columns): 16 rows of it are still one aligned run of
+            // 64 N bytes.  The half panel is staged row-major without padding (16 N floats fit the private tile; N <= 64 here)
+            // and leaves in ceil(4 N / 64) stores of 16 bytes per lane instead of 16 TN stores of 4.
+            if constexpr (TN <= 2) if (g.c_flat) {  // (N <= 64: the widest kernel has no registers to spare for a third epilogue)
+                float *const stage = reinterpret_cast<float *>(apriv);  // [16][N]
+#pragma unroll
+                for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+                    for (int t = 0; t < TN; ++t) {
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) {
+                            const int d = 8 * (v / 4) + (v % 4) + 4 * h;  // row within the half panel
+                            float x = acc[t][8 * pass + v];
+                            if (relu) x = fmaxf(x, 0.f);
+                            if (li + t * 32 < N) stage[d * N + t * 32 + li] = x;
+                            acc[t][8 * pass + v] = 0.f;
+                        }
+                    }
+                    plx::wave_lds_fence();
+                    const int64_t row_first = panel * 32 + 16 * pass;
+                    const int valid = (int)min(max(g.M - row_first, (int64_t)0), (int64_t)16) * N;  // floats of this half panel that exist
+                    float *const dst = g.C + row_first * N;
+                    for (int i = 4 * lane; i < valid; i += 256) {
+                        if (i + 4 <= valid) {
+                            *reinterpret_cast<float4 *>(dst + i) = *reinterpret_cast<const float4 *>(stage + i);
+                        } else {
+                            for (int e = i; e < valid; ++e) dst[e] = stage[e];
+                        }
+                    }
+                    plx::wave_lds_fence();  // the next half, or the next panel's first chunk, overwrites the staging
+                }
+                return;
+            }
         }
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -821,9 +855,10 @@ int launch_resident(const SplitArgs &g, unsigned blocks, hipStream_t st)
         return launch_resident_one<TN, MASK, DROP, true, 8>(g, blocks, st);
     }
     if constexpr (MASK == 0 && !DROP) {  // rows of A without 16-byte alignment, or a K that is not a multiple of 4
+        // (four column tiles over eight positions: the shifting does not fit the registers, the guarded form below takes those)
         if (g.K >= 4 && g.lda < ld_max) {
             if (g.K <= 64) return launch_resident_one<TN, 0, false, true, 4, false>(g, blocks, st);
-            return launch_resident_one<TN, 0, false, true, 8, false>(g, blocks, st);
+            if constexpr (TN <= 2) return launch_resident_one<TN, 0, false, true, 8, false>(g, blocks, st);
         }
     }
     return launch_resident_one<TN, MASK, DROP, false, 8>(g, blocks, st);
@@ -1000,6 +1035,7 @@ int nt_form(const char *who, int64_t M, int64_t N, int64_t K, const float *A, in
     g.A = A; g.mask = mask; g.Bp = planes; g.C = C; g.lda = lda; g.ldmask = ldmask; g.ldc = ldc;
     g.M = M; g.N = N; g.K = K; g.Np = Np; g.Kp = Kp; g.flags = mm_flags; g.a_vec = vec;
     g.c_vec = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc % 4 == 0 && N % 4 == 0) ? 1 : 0;
+    g.c_flat = (!g.c_vec && reinterpret_cast<uintptr_t>(C) % 16 == 0 && ldc == N && N <= 64 && relu_bits == nullptr) ? 1 : 0;
     g.nonfinite = flag_words;
     g.ldw = ldw;
     if (drop != nullptr) {
