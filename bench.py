@@ -377,13 +377,13 @@ def bench_dense_kernels(args, dev):
     def rec(name, fn, bytes_, flops):
         # ten warm-up launches, then blocks of launches until two successive blocks agree within 2 % (four at most): the first
         # kernels after a change of load meet a clock that is still settling and run up to 15 % longer than later on
-        ms = time_gpu(fn, 10, args.spmm_iters)
+        blocks = [time_gpu(fn, 10, args.spmm_iters)]
         for _ in range(3):
-            again = time_gpu(fn, 0, args.spmm_iters)
-            settled = abs(again - ms) <= 0.02 * ms
-            ms = again
-            if settled:
+            blocks.append(time_gpu(fn, 0, args.spmm_iters))
+            if abs(blocks[-1] - blocks[-2]) <= 0.02 * blocks[-2]:
                 break
+        # the mean of the two blocks that agree; if none did, the median of the blocks after the first
+        ms = 0.5 * (blocks[-1] + blocks[-2]) if abs(blocks[-1] - blocks[-2]) <= 0.02 * blocks[-2] else sorted(blocks[1:])[len(blocks[1:]) // 2]
         rows.append({"kernel": name, "ms": ms, "GBps": bytes_ / ms / 1e6, "TFLOPs": flops / ms / 1e9,
                      "frac_hbm_peak": bytes_ / ms / 1e6 / HBM_PEAK_GBPS})
         note("%-44s %7.3f ms  %7.0f GB/s (%4.1f %% of HBM peak)  %6.1f TFLOP/s" % (name, ms, rows[-1]["GBps"], 100 * rows[-1]["frac_hbm_peak"],
