@@ -1718,3 +1718,48 @@ def test_device_block_csr_from_edge_list_matches_loader_sequence():
     a_ref, at_ref = po.build_csr_pair(ei, w, (n, n))
     assert rel_err(ops.spmm(a, h.to(DEV)), po.spmm(a_ref, h)) <= FP32_TOL
     assert rel_err(ops.spmm(at, h.to(DEV)), po.spmm(at_ref, h)) <= FP32_TOL
+
+
+@pytest.mark.parametrize("k", [4, 5, 6, 7, 9, 33, 47, 63, 65, 100, 127])
+@pytest.mark.parametrize("n", [16, 64, 128])
+def test_rows_without_16_byte_alignment_give_exact_integer_products(k, n):
+    """Small integers make every product exact in fp32, so a column that the shifted last vector of a row puts in the wrong
+    place changes the result.  A has K columns (rows of 4 K bytes) and a base that is only 4-byte aligned."""
+    say("exact integer products, K=%d N=%d, 4-byte aligned rows" % (k, n))
+    gen = torch.Generator().manual_seed(100 * k + n)
+    m = 1000 + k
+    flat = torch.zeros(m * k + 1)
+    flat[1:] = torch.randint(-3, 4, (m * k,), generator=gen).float()
+    a = flat.to(DEV)[1:].view(m, k)
+    assert a.data_ptr() % 16 != 0
+    w = torch.randint(-3, 4, (k, n), generator=gen).float()
+    ref = flat[1:].view(m, k).double() @ w.double()
+    assert torch.equal(ops.gemm_nn(a, w.to(DEV)).cpu().double(), ref)
+    assert torch.equal(ops.gemm_nt(a, w.t().contiguous().to(DEV)).cpu().double(), ref)
+
+
+@pytest.mark.parametrize("n", [1, 3, 47, 63, 64])
+@pytest.mark.parametrize("m", [16, 777, 4101])
+def test_narrow_contiguous_results_leave_in_flat_runs_exactly(m, n):
+    """A contiguous result of at most 64 columns whose rows are not multiples of 16 bytes is written as flat runs of 16-byte
+    stores, 16 rows at a time; the last run of a short last panel ends element by element.  Integer operands: exact results,
+    fp32 and bf16, and nothing written past the end of C."""
+    say("flat epilogue %d x %d" % (m, n))
+    gen = torch.Generator().manual_seed(m + n)
+    k = 128
+    a = torch.randint(-1, 2, (m, k), generator=gen).float()
+    w = torch.randint(-1, 2, (k, n), generator=gen).float()
+    ref = a.double() @ w.double()
+    guard = torch.full((m * n + 64,), 7.0, device=DEV)  # C is the front of this buffer: what lies behind it must stay
+    c = guard[: m * n].view(m, n)
+    from plexus_amd import _lib
+    lib = _lib.load()
+    ws, need = ops._split_ws(n, k, torch.device(DEV))
+    ad, wd = a.to(DEV), w.to(DEV)
+    _lib.check(lib.plx_gemm_nn_f32_split(m, n, k, ad.data_ptr(), k, wd.data_ptr(), n, c.data_ptr(), n, 0, ws.data_ptr(), need,
+                                         torch.cuda.current_stream().cuda_stream), "plx_gemm_nn_f32_split")
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu().double(), ref) and bool((guard[m * n:] == 7.0).all())
+    cb = ops.gemm_nt_bf16(bf(a).to(DEV), bf(w.t().contiguous()).to(DEV)).float().cpu()
+    assert torch.equal(cb.double(), ref)  # |sum| <= 128: exact in bf16
+    assert torch.equal(torch.relu(cb), ops.gemm_nt_bf16(bf(a).to(DEV), bf(w.t().contiguous()).to(DEV), relu=True).float().cpu())
