@@ -200,13 +200,15 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_split_tn_kernel(const TnArgs
         auto stash_quad = [&](uint32_t *dst, int plane_words, const float4 &r0, const float4 &r1) -> bool {
             const float x0[4] = {r0.x, r0.y, r0.z, r0.w}, x1[4] = {r1.x, r1.y, r1.z, r1.w};
             bool care = false;
+            uint32_t piece[3][4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                uint32_t p0, p1, p2;
-                care |= split2_checked(x0[e], x1[e], p0, p1, p2);
-                dst[e * kSW] = p0;
-                dst[e * kSW + plane_words] = p1;
-                dst[e * kSW + 2 * plane_words] = p2;
+            for (int e = 0; e < 4; ++e) care |= split2_checked(x0[e], x1[e], piece[0][e], piece[1][e], piece[2][e]);
+            // plane by plane: four stores at fixed distances from one address pair up into two-word store instructions
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                uint32_t *const d = dst + q * plane_words;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) d[e * kSW] = piece[q][e];
             }
             return care;
         };
